@@ -1,0 +1,255 @@
+"""Tensor-level entry points of the hybrid-cache operators.
+
+Each function validates its tensors on the host (device, dtype, innermost
+contiguity, index dtype), then hands raw device pointers, sizes, strides and
+the caller's current stream to the C ABI.  Nothing here computes: without the
+HIP library these functions raise.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+APS_F16, APS_BF16, APS_F32, APS_F64, APS_FP8_E4M3 = 0, 1, 2, 3, 4
+MIXED_LITERAL_MODULO = 1
+MIXED_SKIP_MIRROR = 2
+
+_DTYPE_CODE = {
+    torch.float16: APS_F16,
+    torch.bfloat16: APS_BF16,
+    torch.float32: APS_F32,
+    torch.float64: APS_F64,
+    torch.uint8: APS_FP8_E4M3,
+}
+if hasattr(torch, "float8_e4m3fn"):
+    _DTYPE_CODE[torch.float8_e4m3fn] = APS_FP8_E4M3
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _check_data(name: str, t: torch.Tensor, dev) -> None:
+    _need(isinstance(t, torch.Tensor), f"{name} must be a tensor")
+    _need(t.is_cuda, f"{name} must live on the GPU")
+    _need(t.device == dev, f"{name} is on {t.device}, expected {dev}")
+    _need(t.dim() == 0 or t.stride(-1) == 1 or t.size(-1) <= 1, f"{name}: innermost dimension must be contiguous")
+
+
+def _check_index(name: str, t: torch.Tensor, dev, dtype=torch.int64) -> None:
+    _need(isinstance(t, torch.Tensor), f"{name} must be a tensor")
+    _need(t.dtype == dtype, f"{name} must be {dtype}, got {t.dtype}")
+    _need(t.is_cuda and t.device == dev, f"{name} must live on {dev}")
+    _need(t.dim() == 1 and (t.numel() <= 1 or t.stride(0) == 1), f"{name} must be a contiguous vector")
+
+
+def _check_paged(paged_cache: torch.Tensor, width: int) -> None:
+    _need(paged_cache.dim() == 5, "paged_cache must be (2, num_blocks, block_size, heads, head_dim)")
+    _need(paged_cache.is_contiguous(), "paged_cache must be contiguous")
+    _need(paged_cache.stride(2) >= width, "row is wider than a cache slot")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None or t.numel() == 0 else t.data_ptr()
+
+
+# --------------------------------------------------------------------- a1 / a2
+
+def hidden_to_cache(hidden, paged_cache, slot_mapping, src_idx, target_slot_idx) -> None:
+    """Drop-in for ``mixed_cache_ops.hidden_to_cache``
+    (additional_designs/mixed_cache_kernels/mixed_cache.cu:119-147)."""
+    dev = hidden.device
+    _check_data("hidden", hidden, dev)
+    _check_data("paged_cache", paged_cache, dev)
+    _need(hidden.dim() == 2, "hidden must be [rows, hidden_size]")
+    _need(hidden.dtype == paged_cache.dtype, "hidden and paged_cache dtypes differ")
+    _check_paged(paged_cache, hidden.size(1))
+    for n, t in (("slot_mapping", slot_mapping), ("src_idx", src_idx), ("target_slot_idx", target_slot_idx)):
+        _check_index(n, t, dev)
+    _need(src_idx.numel() == target_slot_idx.numel(), "src_idx and target_slot_idx lengths differ")
+    slot_stride = paged_cache.stride(2)
+    with torch.cuda.device(dev):
+        st = _lib.load().aps_hidden_to_cache(
+            hidden.data_ptr(), paged_cache.data_ptr(), _ptr(slot_mapping), _ptr(src_idx), _ptr(target_slot_idx),
+            src_idx.numel(), hidden.size(1), hidden.stride(0), slot_stride, paged_cache.numel() // slot_stride,
+            hidden.size(0), slot_mapping.numel(), hidden.element_size(), _stream(hidden))
+    _lib.check(st, "hidden_to_cache")
+
+
+def cache_to_hidden(hidden, paged_cache, slot_mapping, dst_idx) -> None:
+    """Drop-in for ``mixed_cache_ops.cache_to_hidden`` (mixed_cache.cu:150-176)."""
+    dev = hidden.device
+    _check_data("hidden", hidden, dev)
+    _check_data("paged_cache", paged_cache, dev)
+    _need(hidden.dim() == 2, "hidden must be [rows, hidden_size]")
+    _need(hidden.dtype == paged_cache.dtype, "hidden and paged_cache dtypes differ")
+    _check_paged(paged_cache, hidden.size(1))
+    _check_index("slot_mapping", slot_mapping, dev)
+    _check_index("dst_idx", dst_idx, dev)
+    slot_stride = paged_cache.stride(2)
+    with torch.cuda.device(dev):
+        st = _lib.load().aps_cache_to_hidden(
+            hidden.data_ptr(), paged_cache.data_ptr(), _ptr(slot_mapping), _ptr(dst_idx), dst_idx.numel(),
+            hidden.size(1), hidden.stride(0), slot_stride, paged_cache.numel() // slot_stride, hidden.size(0),
+            slot_mapping.numel(), hidden.element_size(), _stream(hidden))
+    _lib.check(st, "cache_to_hidden")
+
+
+def hybrid_decode_gather(holder, hidden_states, paged_cache, slot_mapping, hidden_holder_upd,
+                         hidden_holder_pull, hidden_cache_use_input, hidden_cache_store_tot) -> None:
+    """One launch for the decode-side store + holder assembly of
+    additional_designs/model_executor/models/aptserve_opt.py:108-121.  ``holder``
+    may be uninitialised memory (``torch.empty``): every row is written."""
+    dev = holder.device
+    for n, t in (("holder", holder), ("hidden_states", hidden_states), ("paged_cache", paged_cache)):
+        _check_data(n, t, dev)
+    _need(holder.dim() == 2 and hidden_states.dim() == 2, "holder and hidden_states must be 2-D")
+    _need(holder.size(1) == hidden_states.size(1), "holder and hidden_states widths differ")
+    _need(holder.dtype == hidden_states.dtype == paged_cache.dtype, "dtypes differ")
+    _check_paged(paged_cache, holder.size(1))
+    for n, t in (("slot_mapping", slot_mapping), ("hidden_holder_upd", hidden_holder_upd),
+                 ("hidden_holder_pull", hidden_holder_pull), ("hidden_cache_use_input", hidden_cache_use_input),
+                 ("hidden_cache_store_tot", hidden_cache_store_tot)):
+        _check_index(n, t, dev)
+    _need(hidden_holder_upd.numel() == hidden_states.size(0), "one upd row per sequence expected")
+    _need(hidden_holder_upd.numel() + hidden_holder_pull.numel() == holder.size(0),
+          "upd and pull must partition the holder rows")
+    _need(slot_mapping.numel() == holder.size(0), "slot_mapping must have one entry per holder row")
+    _need(hidden_cache_use_input.numel() == hidden_cache_store_tot.numel(), "store index lengths differ")
+    slot_stride = paged_cache.stride(2)
+    with torch.cuda.device(dev):
+        st = _lib.load().aps_hybrid_decode_gather(
+            holder.data_ptr(), hidden_states.data_ptr(), paged_cache.data_ptr(), _ptr(slot_mapping),
+            _ptr(hidden_holder_upd), hidden_holder_upd.numel(), _ptr(hidden_holder_pull),
+            hidden_holder_pull.numel(), _ptr(hidden_cache_use_input), _ptr(hidden_cache_store_tot),
+            hidden_cache_store_tot.numel(), holder.size(1), holder.stride(0), hidden_states.stride(0), slot_stride,
+            paged_cache.numel() // slot_stride, holder.size(0), holder.element_size(), _stream(holder))
+    _lib.check(st, "hybrid_decode_gather")
+
+
+# --------------------------------------------------------------------- a3 / a4
+
+def _check_kv_cache(name: str, c: torch.Tensor, heads: int, head_size: int) -> None:
+    _need(c.dim() == 4, f"{name} must be [num_blocks, block_size, heads, head_dim]")
+    _need(c.size(2) == heads and c.size(3) == head_size, f"{name}: head layout differs from key/value")
+    _need(c.stride(3) == 1 and c.stride(2) == head_size and c.stride(1) == heads * head_size,
+          f"{name}: a block must be contiguous")
+
+
+def _as_thd(name: str, t: torch.Tensor, heads: int, head_size: int) -> torch.Tensor:
+    if t.dim() == 2:
+        _need(t.size(1) == heads * head_size, f"{name} has the wrong width")
+        return t
+    _need(t.dim() == 3 and t.size(1) == heads and t.size(2) == head_size, f"{name} must be [tokens, heads, head_dim]")
+    _need(t.stride(2) == 1 and t.stride(1) == head_size, f"{name}: a token row must be contiguous")
+    return t
+
+
+def reshape_and_cache_flash(key, value, key_cache, value_cache, slot_mapping, kv_cache_dtype: str = "auto",
+                            k_scale: float = 1.0, v_scale: float = 1.0,
+                            token_idx: Optional[torch.Tensor] = None) -> None:
+    """Same call shape as ``vllm._custom_ops.reshape_and_cache_flash`` as used at
+    additional_designs/attention/backends/aptserve_flash_attn.py:338-345.
+    ``kv_cache_dtype``: ``"auto"`` (cache dtype == key dtype) or ``"fp8"``
+    (uint8 / float8_e4m3fn cache holding e4m3 codes of ``x / scale``).
+    ``token_idx`` selects a subset of tokens without gather copies (``:348-355``)."""
+    dev = key.device
+    heads, head_size = key_cache.size(2), key_cache.size(3)
+    for n, t in (("key", key), ("value", value), ("key_cache", key_cache), ("value_cache", value_cache)):
+        _check_data(n, t, dev)
+    key = _as_thd("key", key, heads, head_size)
+    value = _as_thd("value", value, heads, head_size)
+    _check_kv_cache("key_cache", key_cache, heads, head_size)
+    _check_kv_cache("value_cache", value_cache, heads, head_size)
+    _need(key.dtype == value.dtype and key_cache.dtype == value_cache.dtype, "K and V dtypes differ")
+    _need(key_cache.shape == value_cache.shape and key_cache.stride(0) == value_cache.stride(0),
+          "key_cache and value_cache layouts differ")
+    _check_index("slot_mapping", slot_mapping, dev)
+    if kv_cache_dtype == "auto":
+        _need(key_cache.dtype == key.dtype, "kv_cache_dtype='auto' needs cache dtype == key dtype")
+    elif kv_cache_dtype in ("fp8", "fp8_e4m3"):
+        _need(key_cache.element_size() == 1, "fp8 cache must be uint8 / float8_e4m3fn")
+    else:
+        raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
+    _need(key.dtype in (torch.float16, torch.bfloat16, torch.float32), f"unsupported key dtype {key.dtype}")
+    if token_idx is not None:
+        _check_index("token_idx", token_idx, dev)
+        n = token_idx.numel()
+        _need(slot_mapping.numel() >= key.size(0) or n == 0, "slot_mapping shorter than key")
+        num_tokens = min(key.size(0), slot_mapping.numel())
+    else:
+        n = slot_mapping.numel()
+        _need(n <= key.size(0) and n <= value.size(0), "slot_mapping longer than key/value")
+        num_tokens = n
+    with torch.cuda.device(dev):
+        st = _lib.load().aps_reshape_and_cache_flash(
+            key.data_ptr(), value.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), _ptr(slot_mapping),
+            _ptr(token_idx), n, num_tokens, heads, head_size, key_cache.size(1), key.stride(0), value.stride(0),
+            key_cache.stride(0), key_cache.size(0), _DTYPE_CODE[key.dtype], _DTYPE_CODE[key_cache.dtype],
+            float(k_scale), float(v_scale), _stream(key))
+    _lib.check(st, "reshape_and_cache_flash")
+
+
+def mixed_kv_to_cache(key, value, k_cache, v_cache, shared_k_cache, shared_v_cache, slot_mapping,
+                      slot_mapping_shared, kv_cache_use_tot, hidden_cache_use_tot, *,
+                      literal_modulo: bool = False, skip_mirror: bool = False) -> None:
+    """Drop-in for ``mixed_cache_ops.mixed_kv_to_cache`` (mixed_cache.cu:179-230).
+
+    Range C uses ``off = blk - 2*nkv``.  The reference's ``blk % (2*nkv)`` (``:88``)
+    is the same value while ``len(slot_mapping_shared) <= 2*len(kv_cache_use_tot)``;
+    ``literal_modulo=True`` reproduces the reference beyond that point too."""
+    dev = key.device
+    heads, head_size = k_cache.size(2), k_cache.size(3)
+    for n, t in (("key", key), ("value", value), ("k_cache", k_cache), ("v_cache", v_cache),
+                 ("shared_k_cache", shared_k_cache), ("shared_v_cache", shared_v_cache)):
+        _check_data(n, t, dev)
+    key = _as_thd("key", key, heads, head_size)
+    value = _as_thd("value", value, heads, head_size)
+    for n, c in (("k_cache", k_cache), ("v_cache", v_cache), ("shared_k_cache", shared_k_cache),
+                 ("shared_v_cache", shared_v_cache)):
+        _check_kv_cache(n, c, heads, head_size)
+        _need(c.dtype == key.dtype, f"{n} dtype differs from key")
+    _need(value.dtype == key.dtype, "key and value dtypes differ")
+    # the reference's single check (mixed_cache.cu:202), as a RuntimeError like TORCH_CHECK
+    if k_cache.stride(0) != v_cache.stride(0):
+        raise RuntimeError("k_cache.stride(0) == v_cache.stride(0) must hold")
+    _need(shared_k_cache.stride(0) == shared_v_cache.stride(0), "shared cache block strides differ")
+    _need(k_cache.size(1) == shared_k_cache.size(1), "block sizes differ")
+    for n, t in (("slot_mapping", slot_mapping), ("slot_mapping_shared", slot_mapping_shared),
+                 ("kv_cache_use_tot", kv_cache_use_tot), ("hidden_cache_use_tot", hidden_cache_use_tot)):
+        _check_index(n, t, dev)
+    _need(hidden_cache_use_tot.numel() >= slot_mapping_shared.numel(),
+          "hidden_cache_use_tot shorter than slot_mapping_shared")
+    num_tot = min(key.size(0), value.size(0))
+    if kv_cache_use_tot.numel():
+        num_tot = min(num_tot, slot_mapping.numel())
+    n_hidden = slot_mapping_shared.numel()
+    flags = (MIXED_LITERAL_MODULO if literal_modulo else 0) | (MIXED_SKIP_MIRROR if skip_mirror else 0)
+    with torch.cuda.device(dev):
+        st = _lib.load().aps_mixed_kv_to_cache(
+            key.data_ptr(), value.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), shared_k_cache.data_ptr(),
+            shared_v_cache.data_ptr(), _ptr(slot_mapping), _ptr(slot_mapping_shared), _ptr(kv_cache_use_tot),
+            _ptr(hidden_cache_use_tot), kv_cache_use_tot.numel(), n_hidden, num_tot, heads, head_size,
+            k_cache.size(1), key.stride(0), value.stride(0), k_cache.stride(0), k_cache.size(0),
+            shared_k_cache.stride(0), shared_k_cache.size(0), key.element_size(), flags, _stream(key))
+    _lib.check(st, "mixed_kv_to_cache")
+
+
+def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
+    """Plain device copy (calibration kernel for hardware counters)."""
+    _need(dst.is_cuda and src.is_cuda and dst.device == src.device, "both tensors must be on one GPU")
+    _need(dst.is_contiguous() and src.is_contiguous(), "tensors must be contiguous")
+    nbytes = src.numel() * src.element_size()
+    _need(nbytes == dst.numel() * dst.element_size(), "sizes differ")
+    with torch.cuda.device(src.device):
+        st = _lib.load().aps_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, _stream(src))
+    _lib.check(st, "copy_bytes")

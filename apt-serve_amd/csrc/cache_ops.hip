@@ -1,0 +1,492 @@
+// Row scatter / gather kernels of the hybrid cache for gfx950.
+//
+// Every operator here moves whole rows (a hidden vector, or the K or V vector
+// of one token) between a dense tensor and slots of a paged cache.  They share
+// one kernel shape, row_mover: a workgroup resolves ROWS row descriptors
+// (source pointer, destination pointer) with wave-uniform index loads, then
+// all lanes stream the rows with 128-bit loads kept in flight together before
+// the matching 128-bit stores.  A row of OPT-13B is 10 KiB = ten 1 KiB
+// wavefront-wide transactions, so loads and stores are fully coalesced.
+#include <hip/hip_fp16.h>
+#include <hip/hip_bf16.h>
+
+#include "aps_common.h"
+
+namespace aps {
+namespace {
+
+constexpr int kMaxThreads = 256;
+
+struct RowDesc {
+  const char* src;  // nullptr with dst != nullptr: fill the row with zeros
+  char* dst;        // nullptr: skip the row
+};
+
+template <int VB, int ROWS, class Op>
+__global__ __launch_bounds__(kMaxThreads) void row_mover(Op op, int64_t n_items, uint32_t row_bytes) {
+  typedef typename VecOf<VB>::type vec_t;
+  RowDesc rd[ROWS];
+  const int64_t item0 = (int64_t)blockIdx.x * ROWS;
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    rd[r].src = nullptr;
+    rd[r].dst = nullptr;
+    if (item0 + r < n_items) rd[r] = op(item0 + r);
+  }
+  const uint32_t step = blockDim.x * VB;
+  for (uint32_t c = threadIdx.x * VB; c < row_bytes; c += step) {
+    vec_t v[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      v[r] = vec_t{};
+      if (rd[r].dst != nullptr && rd[r].src != nullptr) v[r] = load_vec_stream<VB>(rd[r].src + c);
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      if (rd[r].dst != nullptr) store_vec_stream<VB>(rd[r].dst + c, v[r]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------- descriptors
+
+struct HiddenToCacheOp {
+  const char* hidden; char* cache;
+  const int64_t* slot_mapping; const int64_t* src_idx; const int64_t* tgt_idx;
+  int64_t hidden_stride_b, slot_stride_b, num_slots, num_hidden_rows, slot_mapping_len;
+  __device__ RowDesc operator()(int64_t b) const {
+    RowDesc r{nullptr, nullptr};
+    const int64_t tok = src_idx[b];
+    const int64_t ti = tgt_idx[b];
+    if (tok < 0 || tok >= num_hidden_rows || ti < 0 || ti >= slot_mapping_len) return r;
+    const int64_t slot = slot_mapping[ti];
+    if (slot < 0 || slot >= num_slots) return r;
+    r.src = hidden + tok * hidden_stride_b;
+    r.dst = cache + slot * slot_stride_b;
+    return r;
+  }
+};
+
+struct CacheToHiddenOp {
+  char* hidden; const char* cache;
+  const int64_t* slot_mapping; const int64_t* dst_idx;
+  int64_t hidden_stride_b, slot_stride_b, num_slots, num_hidden_rows, slot_mapping_len;
+  __device__ RowDesc operator()(int64_t b) const {
+    RowDesc r{nullptr, nullptr};
+    const int64_t tok = dst_idx[b];
+    if (tok < 0 || tok >= num_hidden_rows || tok >= slot_mapping_len) return r;
+    const int64_t slot = slot_mapping[tok];
+    if (slot < 0 || slot >= num_slots) return r;
+    r.src = cache + slot * slot_stride_b;
+    r.dst = hidden + tok * hidden_stride_b;
+    return r;
+  }
+};
+
+struct HybridDecodeGatherOp {
+  char* holder; const char* hidden_states; char* cache;
+  const int64_t* slot_mapping; const int64_t* upd; const int64_t* pull;
+  const int64_t* use_input; const int64_t* store_tot;
+  int64_t n_upd, n_pull, n_store;
+  int64_t holder_stride_b, hidden_stride_b, slot_stride_b, num_slots, num_tot;
+  __device__ RowDesc operator()(int64_t i) const {
+    RowDesc r{nullptr, nullptr};
+    if (i < n_upd) {  // newest row of every sequence comes from the layer input
+      const int64_t t = upd[i];
+      if (t < 0 || t >= num_tot) return r;
+      r.src = hidden_states + i * hidden_stride_b;
+      r.dst = holder + t * holder_stride_b;
+    } else if (i < n_upd + n_pull) {  // context rows of hidden sequences come from the cache
+      const int64_t t = pull[i - n_upd];
+      if (t < 0 || t >= num_tot) return r;
+      r.dst = holder + t * holder_stride_b;
+      const int64_t slot = slot_mapping[t];
+      if (slot >= 0 && slot < num_slots) r.src = cache + slot * slot_stride_b;  // else zero row
+    } else {  // newest hidden row is also persisted
+      const int64_t j = i - n_upd - n_pull;
+      const int64_t b = use_input[j];
+      const int64_t t = store_tot[j];
+      if (b < 0 || b >= n_upd || t < 0 || t >= num_tot) return r;
+      const int64_t slot = slot_mapping[t];
+      if (slot < 0 || slot >= num_slots) return r;
+      r.src = hidden_states + b * hidden_stride_b;
+      r.dst = cache + slot * slot_stride_b;
+    }
+    return r;
+  }
+};
+
+// item = 2*t + plane (0 = K, 1 = V)
+struct KvScatterOp {
+  const char* key; const char* value; char* k_cache; char* v_cache;
+  const int64_t* slot_mapping; const int64_t* token_idx;
+  int64_t num_tokens, key_stride_b, value_stride_b, block_stride_b, row_b, num_blocks;
+  int block_size;
+  __device__ RowDesc operator()(int64_t item) const {
+    RowDesc r{nullptr, nullptr};
+    const int64_t t = item >> 1;
+    const int64_t tok = token_idx ? token_idx[t] : t;
+    if (tok < 0 || tok >= num_tokens) return r;
+    const int64_t slot = slot_mapping[tok];
+    if (slot < 0) return r;
+    const int64_t blk = slot / block_size;
+    if (blk >= num_blocks) return r;
+    const int64_t off = blk * block_stride_b + (slot - blk * block_size) * row_b;
+    if (item & 1) { r.src = value + tok * value_stride_b; r.dst = v_cache + off; }
+    else          { r.src = key + tok * key_stride_b;     r.dst = k_cache + off; }
+    return r;
+  }
+};
+
+// item = 2*blk + plane over the reference's grid of 2*nkv + nh blocks
+struct MixedKvOp {
+  const char* key; const char* value;
+  char* k_cache; char* v_cache; char* sk_cache; char* sv_cache;
+  const int64_t* slot_mapping; const int64_t* slot_mapping_shared;
+  const int64_t* kv_use_tot; const int64_t* hidden_use_tot;
+  int64_t n_kv, n_hidden, num_tot;
+  int64_t key_stride_b, value_stride_b, block_stride_b, shared_block_stride_b, row_b;
+  int64_t num_blocks, num_shared_blocks;
+  int block_size; unsigned flags;
+  __device__ RowDesc operator()(int64_t item) const {
+    RowDesc r{nullptr, nullptr};
+    const int64_t blk = item >> 1;
+    int64_t tok, slot;
+    bool to_shared;
+    if (blk < n_kv) {
+      tok = kv_use_tot[blk];
+      if (tok < 0 || tok >= num_tot) return r;
+      slot = slot_mapping[tok];
+      to_shared = false;
+    } else if (blk < 2 * n_kv) {
+      if (flags & APS_MIXED_SKIP_MIRROR) return r;
+      tok = kv_use_tot[blk - n_kv];
+      if (tok < 0 || tok >= num_tot) return r;
+      slot = slot_mapping[tok];
+      to_shared = true;
+    } else {
+      int64_t off = blk - 2 * n_kv;
+      if ((flags & APS_MIXED_LITERAL_MODULO) && n_kv > 0) off = blk % (2 * n_kv);
+      if (off >= n_hidden) return r;
+      tok = hidden_use_tot[off];
+      if (tok < 0 || tok >= num_tot) return r;
+      slot = slot_mapping_shared[off];
+      to_shared = true;
+    }
+    if (slot < 0) return r;
+    const int64_t b = slot / block_size;
+    if (b >= (to_shared ? num_shared_blocks : num_blocks)) return r;
+    const int64_t off_b = b * (to_shared ? shared_block_stride_b : block_stride_b) +
+                          (slot - b * block_size) * row_b;
+    if (item & 1) { r.src = value + tok * value_stride_b; r.dst = (to_shared ? sv_cache : v_cache) + off_b; }
+    else          { r.src = key + tok * key_stride_b;     r.dst = (to_shared ? sk_cache : k_cache) + off_b; }
+    return r;
+  }
+};
+
+template <int VB, class Op>
+void launch_rows_vb(const Op& op, int64_t n_items, int64_t row_bytes, hipStream_t s) {
+  const int64_t cpr = (row_bytes + VB - 1) / VB;
+  int threads = (int)((cpr + 63) / 64 * 64);
+  if (threads > kMaxThreads) threads = kMaxThreads;
+  // Small launches (a decode step writes a few hundred rows) use one row per
+  // workgroup so that the grid still covers the 256 compute units.
+  if (n_items >= 4096) {
+    const int64_t grid = (n_items + 3) / 4;
+    hipLaunchKernelGGL((row_mover<VB, 4, Op>), dim3((unsigned)grid), dim3(threads), 0, s, op, n_items,
+                       (uint32_t)row_bytes);
+  } else {
+    hipLaunchKernelGGL((row_mover<VB, 1, Op>), dim3((unsigned)n_items), dim3(threads), 0, s, op, n_items,
+                       (uint32_t)row_bytes);
+  }
+}
+
+template <class Op>
+int launch_rows(const Op& op, int64_t n_items, int64_t row_bytes, int vb, hipStream_t s) {
+  if (n_items <= 0 || row_bytes <= 0) return APS_OK;
+  if (row_bytes >= (int64_t)1 << 31 || (n_items + 3) / 4 >= (int64_t)1 << 31) return APS_ERR_UNSUPPORTED;
+  switch (vb) {
+    case 16: launch_rows_vb<16>(op, n_items, row_bytes, s); break;
+    case 8: launch_rows_vb<8>(op, n_items, row_bytes, s); break;
+    case 4: launch_rows_vb<4>(op, n_items, row_bytes, s); break;
+    case 2: launch_rows_vb<2>(op, n_items, row_bytes, s); break;
+    default: launch_rows_vb<1>(op, n_items, row_bytes, s); break;
+  }
+  return launch_status();
+}
+
+inline bool valid_elem(int e) { return e == 1 || e == 2 || e == 4 || e == 8; }
+
+// ------------------------------------------------------- fp8 quantising write
+
+template <class T> __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<_Float16>(_Float16 v) { return (float)v; }
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+struct bf16_bits { uint16_t u; };
+template <> __device__ __forceinline__ float to_f32<bf16_bits>(bf16_bits v) {
+  return __uint_as_float((uint32_t)v.u << 16);
+}
+
+// code = e4m3fn(clamp(x / scale, +-448)), round to nearest even.  The clamp
+// makes the result independent of the conversion instruction's overflow mode;
+// NaN is kept NaN (fminf/fmaxf would drop it).
+__device__ __forceinline__ float fp8_prepare(float x, float scale) {
+  const float y = x / scale;
+  const float c = fminf(fmaxf(y, -448.0f), 448.0f);
+  return (y != y) ? y : c;
+}
+
+__device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d) {
+  int w = 0;
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+  return (uint32_t)w;
+}
+
+// One workgroup per (token, plane).  EPT elements per thread per step:
+// 8 (128-bit load of f16/bf16, 64-bit store) when everything is aligned, else 1.
+template <class InT, int EPT>
+__global__ __launch_bounds__(kMaxThreads) void kv_scatter_fp8(
+    const InT* __restrict__ key, const InT* __restrict__ value, uint8_t* __restrict__ k_cache,
+    uint8_t* __restrict__ v_cache, const int64_t* __restrict__ slot_mapping,
+    const int64_t* __restrict__ token_idx, int64_t num_tokens, int64_t key_stride, int64_t value_stride,
+    int64_t block_stride, int64_t num_blocks, int block_size, int row_elems, float k_scale, float v_scale) {
+  const int64_t item = blockIdx.x;
+  const int64_t t = item >> 1;
+  const bool is_v = item & 1;
+  const int64_t tok = token_idx ? token_idx[t] : t;
+  if (tok < 0 || tok >= num_tokens) return;
+  const int64_t slot = slot_mapping[tok];
+  if (slot < 0) return;
+  const int64_t blk = slot / block_size;
+  if (blk >= num_blocks) return;
+  const InT* src = is_v ? value + tok * value_stride : key + tok * key_stride;
+  uint8_t* dst = (is_v ? v_cache : k_cache) + blk * block_stride + (slot - blk * block_size) * (int64_t)row_elems;
+  const float scale = is_v ? v_scale : k_scale;
+  if constexpr (EPT == 8) {
+    for (int c = threadIdx.x * 8; c < row_elems; c += blockDim.x * 8) {
+      InT in[8];
+      if constexpr (sizeof(InT) == 2) {
+        *reinterpret_cast<VecOf<16>::type*>(in) = *reinterpret_cast<const VecOf<16>::type*>(src + c);
+      } else {
+        *reinterpret_cast<VecOf<16>::type*>(in) = *reinterpret_cast<const VecOf<16>::type*>(src + c);
+        *reinterpret_cast<VecOf<16>::type*>(in + 4) = *reinterpret_cast<const VecOf<16>::type*>(src + c + 4);
+      }
+      float f[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] = fp8_prepare(to_f32<InT>(in[i]), scale);
+      VecOf<8>::type out;
+      out.x = pack4_e4m3(f[0], f[1], f[2], f[3]);
+      out.y = pack4_e4m3(f[4], f[5], f[6], f[7]);
+      *reinterpret_cast<VecOf<8>::type*>(dst + c) = out;
+    }
+  } else {
+    for (int c = threadIdx.x; c < row_elems; c += blockDim.x) {
+      const float f = fp8_prepare(to_f32<InT>(src[c]), scale);
+      dst[c] = (uint8_t)(pack4_e4m3(f, 0.f, 0.f, 0.f) & 0xFFu);
+    }
+  }
+}
+
+template <class InT>
+int launch_kv_scatter_fp8(const void* key, const void* value, void* k_cache, void* v_cache,
+                          const int64_t* slot_mapping, const int64_t* token_idx, int64_t n, int64_t num_tokens,
+                          int64_t key_stride, int64_t value_stride, int64_t block_stride, int64_t num_blocks,
+                          int block_size, int row_elems, float k_scale, float v_scale, hipStream_t s) {
+  const int in_b = (int)sizeof(InT);
+  const bool aligned = row_elems % 8 == 0 &&
+                       common_vec_bytes({addr(key), addr(value), (uint64_t)key_stride * in_b,
+                                         (uint64_t)value_stride * in_b}) == 16 &&
+                       common_vec_bytes({addr(k_cache), addr(v_cache), (uint64_t)block_stride}) >= 8;
+  const int per = aligned ? 8 : 1;
+  int threads = ((row_elems + per - 1) / per + 63) / 64 * 64;
+  if (threads > kMaxThreads) threads = kMaxThreads;
+  const dim3 grid((unsigned)(2 * n));
+  if (aligned)
+    hipLaunchKernelGGL((kv_scatter_fp8<InT, 8>), grid, dim3(threads), 0, s, (const InT*)key, (const InT*)value,
+                       (uint8_t*)k_cache, (uint8_t*)v_cache, slot_mapping, token_idx, num_tokens, key_stride,
+                       value_stride, block_stride, num_blocks, block_size, row_elems, k_scale, v_scale);
+  else
+    hipLaunchKernelGGL((kv_scatter_fp8<InT, 1>), grid, dim3(threads), 0, s, (const InT*)key, (const InT*)value,
+                       (uint8_t*)k_cache, (uint8_t*)v_cache, slot_mapping, token_idx, num_tokens, key_stride,
+                       value_stride, block_stride, num_blocks, block_size, row_elems, k_scale, v_scale);
+  return launch_status();
+}
+
+__global__ __launch_bounds__(kMaxThreads) void copy_bytes_kernel(VecOf<16>::type* __restrict__ dst,
+                                                                  const VecOf<16>::type* __restrict__ src,
+                                                                  int64_t n_vec) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec; i += stride) {
+    __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+  }
+}
+
+}  // namespace
+}  // namespace aps
+
+using namespace aps;
+
+extern "C" {
+
+int aps_abi_version(void) { return APS_ABI_VERSION; }
+
+const char* aps_status_string(int status) {
+  switch (status) {
+    case APS_OK: return "ok";
+    case APS_ERR_INVALID_ARG: return "invalid argument";
+    case APS_ERR_UNSUPPORTED: return "unsupported shape or dtype";
+    case APS_ERR_WORKSPACE: return "workspace too small";
+    default: return status > 0 ? hipGetErrorString((hipError_t)status) : "unknown status";
+  }
+}
+
+int aps_hidden_to_cache(const void* hidden, void* paged_cache, const int64_t* slot_mapping, const int64_t* src_idx,
+                        const int64_t* target_slot_idx, int64_t n, int64_t hidden_size, int64_t hidden_stride,
+                        int64_t slot_stride, int64_t num_slots, int64_t num_hidden_rows, int64_t slot_mapping_len,
+                        int elem_size, aps_stream_t stream) {
+  if (n < 0 || hidden_size < 0 || !valid_elem(elem_size)) return APS_ERR_INVALID_ARG;
+  if (n == 0 || hidden_size == 0) return APS_OK;
+  if (!hidden || !paged_cache || !slot_mapping || !src_idx || !target_slot_idx) return APS_ERR_INVALID_ARG;
+  if (hidden_stride < hidden_size || slot_stride < hidden_size) return APS_ERR_INVALID_ARG;
+  const int64_t e = elem_size;
+  HiddenToCacheOp op{(const char*)hidden, (char*)paged_cache, slot_mapping, src_idx, target_slot_idx,
+                     hidden_stride * e, slot_stride * e, num_slots, num_hidden_rows, slot_mapping_len};
+  const int vb = common_vec_bytes({addr(hidden), addr(paged_cache), (uint64_t)(hidden_stride * e),
+                                   (uint64_t)(slot_stride * e), (uint64_t)(hidden_size * e)});
+  return launch_rows(op, n, hidden_size * e, vb, (hipStream_t)stream);
+}
+
+int aps_cache_to_hidden(void* hidden, const void* paged_cache, const int64_t* slot_mapping, const int64_t* dst_idx,
+                        int64_t n, int64_t hidden_size, int64_t hidden_stride, int64_t slot_stride,
+                        int64_t num_slots, int64_t num_hidden_rows, int64_t slot_mapping_len, int elem_size,
+                        aps_stream_t stream) {
+  if (n < 0 || hidden_size < 0 || !valid_elem(elem_size)) return APS_ERR_INVALID_ARG;
+  if (n == 0 || hidden_size == 0) return APS_OK;
+  if (!hidden || !paged_cache || !slot_mapping || !dst_idx) return APS_ERR_INVALID_ARG;
+  if (hidden_stride < hidden_size || slot_stride < hidden_size) return APS_ERR_INVALID_ARG;
+  const int64_t e = elem_size;
+  CacheToHiddenOp op{(char*)hidden, (const char*)paged_cache, slot_mapping, dst_idx,
+                     hidden_stride * e, slot_stride * e, num_slots, num_hidden_rows, slot_mapping_len};
+  const int vb = common_vec_bytes({addr(hidden), addr(paged_cache), (uint64_t)(hidden_stride * e),
+                                   (uint64_t)(slot_stride * e), (uint64_t)(hidden_size * e)});
+  return launch_rows(op, n, hidden_size * e, vb, (hipStream_t)stream);
+}
+
+int aps_hybrid_decode_gather(void* holder, const void* hidden_states, void* paged_cache,
+                             const int64_t* slot_mapping, const int64_t* hidden_holder_upd, int64_t n_upd,
+                             const int64_t* hidden_holder_pull, int64_t n_pull,
+                             const int64_t* hidden_cache_use_input, const int64_t* hidden_cache_store_tot,
+                             int64_t n_store, int64_t hidden_size, int64_t holder_stride, int64_t hidden_stride,
+                             int64_t slot_stride, int64_t num_slots, int64_t num_tot_tokens, int elem_size,
+                             aps_stream_t stream) {
+  if (n_upd < 0 || n_pull < 0 || n_store < 0 || hidden_size < 0 || !valid_elem(elem_size))
+    return APS_ERR_INVALID_ARG;
+  const int64_t n = n_upd + n_pull + n_store;
+  if (n == 0 || hidden_size == 0) return APS_OK;
+  if (!holder || !hidden_states || !paged_cache || !slot_mapping) return APS_ERR_INVALID_ARG;
+  if ((n_upd && !hidden_holder_upd) || (n_pull && !hidden_holder_pull) ||
+      (n_store && (!hidden_cache_use_input || !hidden_cache_store_tot)))
+    return APS_ERR_INVALID_ARG;
+  if (holder_stride < hidden_size || hidden_stride < hidden_size || slot_stride < hidden_size)
+    return APS_ERR_INVALID_ARG;
+  const int64_t e = elem_size;
+  HybridDecodeGatherOp op{(char*)holder, (const char*)hidden_states, (char*)paged_cache, slot_mapping,
+                          hidden_holder_upd, hidden_holder_pull, hidden_cache_use_input, hidden_cache_store_tot,
+                          n_upd, n_pull, n_store, holder_stride * e, hidden_stride * e, slot_stride * e,
+                          num_slots, num_tot_tokens};
+  const int vb = common_vec_bytes({addr(holder), addr(hidden_states), addr(paged_cache),
+                                   (uint64_t)(holder_stride * e), (uint64_t)(hidden_stride * e),
+                                   (uint64_t)(slot_stride * e), (uint64_t)(hidden_size * e)});
+  return launch_rows(op, n, hidden_size * e, vb, (hipStream_t)stream);
+}
+
+int aps_reshape_and_cache_flash(const void* key, const void* value, void* key_cache, void* value_cache,
+                                const int64_t* slot_mapping, const int64_t* token_idx, int64_t n,
+                                int64_t num_tokens, int num_heads, int head_size, int block_size,
+                                int64_t key_stride, int64_t value_stride, int64_t block_stride,
+                                int64_t num_blocks, int in_dtype, int cache_dtype, float k_scale, float v_scale,
+                                aps_stream_t stream) {
+  if (n < 0 || num_heads <= 0 || head_size <= 0 || block_size <= 0) return APS_ERR_INVALID_ARG;
+  const int in_b = elem_bytes_of(in_dtype);
+  if (in_b == 0 || in_dtype == APS_FP8_E4M3) return APS_ERR_INVALID_ARG;
+  if (n == 0) return APS_OK;
+  if (!key || !value || !key_cache || !value_cache || !slot_mapping) return APS_ERR_INVALID_ARG;
+  const int64_t row = (int64_t)num_heads * head_size;
+  if (key_stride < row || value_stride < row || block_stride < row * block_size) return APS_ERR_INVALID_ARG;
+  if (2 * n >= (int64_t)1 << 31) return APS_ERR_UNSUPPORTED;
+  hipStream_t s = (hipStream_t)stream;
+  if (cache_dtype == in_dtype) {
+    const int64_t e = in_b;
+    KvScatterOp op{(const char*)key, (const char*)value, (char*)key_cache, (char*)value_cache, slot_mapping,
+                   token_idx, num_tokens, key_stride * e, value_stride * e, block_stride * e, row * e, num_blocks,
+                   block_size};
+    const int vb = common_vec_bytes({addr(key), addr(value), addr(key_cache), addr(value_cache),
+                                     (uint64_t)(key_stride * e), (uint64_t)(value_stride * e),
+                                     (uint64_t)(block_stride * e), (uint64_t)(row * e)});
+    return launch_rows(op, 2 * n, row * e, vb, s);
+  }
+  if (cache_dtype != APS_FP8_E4M3) return APS_ERR_UNSUPPORTED;
+  if (!(k_scale > 0.f) || !(v_scale > 0.f) || row >= (int64_t)1 << 30) return APS_ERR_INVALID_ARG;
+  switch (in_dtype) {
+    case APS_F16:
+      return launch_kv_scatter_fp8<_Float16>(key, value, key_cache, value_cache, slot_mapping, token_idx, n,
+                                             num_tokens, key_stride, value_stride, block_stride, num_blocks,
+                                             block_size, (int)row, k_scale, v_scale, s);
+    case APS_BF16:
+      return launch_kv_scatter_fp8<bf16_bits>(key, value, key_cache, value_cache, slot_mapping, token_idx, n,
+                                              num_tokens, key_stride, value_stride, block_stride, num_blocks,
+                                              block_size, (int)row, k_scale, v_scale, s);
+    case APS_F32:
+      return launch_kv_scatter_fp8<float>(key, value, key_cache, value_cache, slot_mapping, token_idx, n,
+                                          num_tokens, key_stride, value_stride, block_stride, num_blocks,
+                                          block_size, (int)row, k_scale, v_scale, s);
+    default:
+      return APS_ERR_UNSUPPORTED;
+  }
+}
+
+int aps_mixed_kv_to_cache(const void* key, const void* value, void* k_cache, void* v_cache, void* shared_k_cache,
+                          void* shared_v_cache, const int64_t* slot_mapping, const int64_t* slot_mapping_shared,
+                          const int64_t* kv_cache_use_tot, const int64_t* hidden_cache_use_tot, int64_t n_kv,
+                          int64_t n_hidden, int64_t num_tot_tokens, int num_heads, int head_size, int block_size,
+                          int64_t key_stride, int64_t value_stride, int64_t block_stride, int64_t num_blocks,
+                          int64_t shared_block_stride, int64_t num_shared_blocks, int elem_size, unsigned flags,
+                          aps_stream_t stream) {
+  if (n_kv < 0 || n_hidden < 0 || num_heads <= 0 || head_size <= 0 || block_size <= 0 || !valid_elem(elem_size))
+    return APS_ERR_INVALID_ARG;
+  const int64_t blocks = 2 * n_kv + n_hidden;
+  if (blocks == 0) return APS_OK;
+  if (!key || !value || !shared_k_cache || !shared_v_cache) return APS_ERR_INVALID_ARG;
+  if (n_kv && (!k_cache || !v_cache || !slot_mapping || !kv_cache_use_tot)) return APS_ERR_INVALID_ARG;
+  if (n_hidden && (!slot_mapping_shared || !hidden_cache_use_tot)) return APS_ERR_INVALID_ARG;
+  const int64_t row = (int64_t)num_heads * head_size;
+  if (key_stride < row || value_stride < row || block_stride < row * block_size ||
+      shared_block_stride < row * block_size)
+    return APS_ERR_INVALID_ARG;
+  const int64_t e = elem_size;
+  MixedKvOp op{(const char*)key, (const char*)value, (char*)k_cache, (char*)v_cache, (char*)shared_k_cache,
+               (char*)shared_v_cache, slot_mapping, slot_mapping_shared, kv_cache_use_tot, hidden_cache_use_tot,
+               n_kv, n_hidden, num_tot_tokens, key_stride * e, value_stride * e, block_stride * e,
+               shared_block_stride * e, row * e, num_blocks, num_shared_blocks, block_size, flags};
+  const int vb = common_vec_bytes({addr(key), addr(value), addr(k_cache), addr(v_cache), addr(shared_k_cache),
+                                   addr(shared_v_cache), (uint64_t)(key_stride * e), (uint64_t)(value_stride * e),
+                                   (uint64_t)(block_stride * e), (uint64_t)(shared_block_stride * e),
+                                   (uint64_t)(row * e)});
+  return launch_rows(op, 2 * blocks, row * e, vb, (hipStream_t)stream);
+}
+
+int aps_copy_bytes(void* dst, const void* src, int64_t nbytes, aps_stream_t stream) {
+  if (nbytes < 0) return APS_ERR_INVALID_ARG;
+  if (nbytes == 0) return APS_OK;
+  if (!dst || !src) return APS_ERR_INVALID_ARG;
+  if (common_vec_bytes({addr(dst), addr(src), (uint64_t)nbytes}) != 16) return APS_ERR_UNSUPPORTED;
+  const int64_t n_vec = nbytes / 16;
+  int64_t grid = (n_vec + kMaxThreads * 4 - 1) / (kMaxThreads * 4);
+  if (grid > 256 * 64) grid = 256 * 64;
+  hipLaunchKernelGGL(copy_bytes_kernel, dim3((unsigned)grid), dim3(kMaxThreads), 0, (hipStream_t)stream,
+                     (VecOf<16>::type*)dst, (const VecOf<16>::type*)src, n_vec);
+  return launch_status();
+}
+
+}  // extern "C"

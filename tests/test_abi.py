@@ -1,0 +1,44 @@
+"""The C-ABI library loads and exports every symbol the public header declares."""
+import ctypes
+import re
+import subprocess
+
+from aptserve_hip import _lib
+
+
+def test_header_parses_and_every_symbol_is_exported():
+    protos = _lib.parse_header()
+    assert "aps_hidden_to_cache" in protos and "aps_cache_to_hidden" in protos
+    assert "aps_mixed_kv_to_cache" in protos
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    for name in protos:
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+
+
+def test_no_undeclared_exports():
+    out = subprocess.run(["nm", "-D", "--defined-only", str(_lib.LIB_PATH)], capture_output=True, text=True).stdout
+    exported = set(re.findall(r" T (aps_\w+)", out))
+    assert exported == set(_lib.parse_header()), "header and library disagree about the ABI"
+
+
+def test_loader_sets_prototypes_and_version():
+    lib = _lib.load()
+    assert lib.aps_abi_version() == _lib._abi_version_of_header()
+    assert lib.aps_status_string(0) == b"ok"
+    assert lib.aps_status_string(-1) == b"invalid argument"
+
+
+def test_signatures_carry_no_torch_types():
+    text = _lib.HEADER.read_text()
+    assert "torch" not in text.lower().replace("pytorch", "")
+    assert "at::" not in text and "Tensor" not in text
+
+
+def test_argument_errors_return_without_launching():
+    lib = _lib.load()
+    # negative sizes / null pointers are rejected on the host, before any GPU call
+    assert lib.aps_copy_bytes(None, None, -1, None) == -1
+    assert lib.aps_copy_bytes(None, None, 0, None) == 0
+    assert lib.aps_hidden_to_cache(None, None, None, None, None, 0, 768, 768, 768, 0, 0, 0, 2, None) == 0
+    assert lib.aps_hidden_to_cache(None, None, None, None, None, 4, 768, 768, 768, 0, 0, 0, 2, None) == -1
+    assert lib.aps_hidden_to_cache(None, None, None, None, None, 4, 768, 768, 768, 0, 0, 0, 3, None) == -1
