@@ -1,0 +1,295 @@
+"""Host side of the ragged-batch metadata: the dataclass the attention backend
+reads and the builder that fills it on the GPU.
+
+``HybridAttentionMetadata`` carries the fields of the reference's
+``AttentionMetadata`` (additional_designs/attention/backends/aptserve_abstract.py:56-80)
+and ``FlashAttentionMetadata`` (additional_designs/attention/backends/aptserve_flash_attn.py:68-222)
+under the same names, including the ``prefill_metadata`` / ``decode_metadata`` views.
+
+``build_metadata`` replaces the list-building loop and the ~15 small
+host-to-device copies of ``ModelRunner._prepare_model_input``
+(additional_designs/worker/aptserve_model_runner.py:240-842): the host sums
+O(batch) integers to size the outputs, uploads ONE packed int32 buffer
+(lengths, cache-type flags, block tables) and one kernel expands everything
+that scales with the number of cached tokens.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from . import _lib
+
+
+@dataclass
+class HybridAttentionMetadata:
+    # aptserve_abstract.py:56-80
+    num_prefills: int
+    num_prefill_tokens: int
+    num_decode_tokens: int
+    num_hidden_cache_tokens: int
+    num_tot_tokens: int
+    slot_mapping: torch.Tensor
+    slot_mapping_shared: torch.Tensor
+    hidden_cache_use_tot: torch.Tensor
+    kv_cache_use_tot: torch.Tensor
+    hidden_cache_use_input: torch.Tensor
+    hidden_cache_store_tot: torch.Tensor
+    hidden_holder_upd: torch.Tensor
+    hidden_holder_pull: torch.Tensor
+    # aptserve_flash_attn.py:76-121
+    seq_lens: Optional[List[int]]
+    seq_lens_tensor: Optional[torch.Tensor]
+    max_query_len: Optional[int]
+    max_prefill_seq_len: int
+    max_decode_seq_len: int
+    query_start_loc: Optional[torch.Tensor]
+    seq_start_loc: Optional[torch.Tensor]
+    context_lens_tensor: Optional[torch.Tensor]
+    block_tables: Optional[torch.Tensor]
+    use_cuda_graph: bool = False
+    # additions of this implementation
+    input_positions: Optional[torch.Tensor] = None
+    block_types: Optional[torch.Tensor] = None      # uint8 [batch, width]: 1 = block read from the K/V workspace
+    _cached_prefill_metadata: Optional["HybridAttentionMetadata"] = None
+    _cached_decode_metadata: Optional["HybridAttentionMetadata"] = None
+
+    @property
+    def prefill_metadata(self) -> Optional["HybridAttentionMetadata"]:
+        """aptserve_flash_attn.py:126-175: slices by ``num_prefills`` / ``num_prefill_tokens``;
+        the hybrid fields pass through unsliced."""
+        if self.num_prefills == 0:
+            return None
+        if self._cached_prefill_metadata is None:
+            self._cached_prefill_metadata = HybridAttentionMetadata(
+                num_prefills=self.num_prefills, num_prefill_tokens=self.num_prefill_tokens, num_decode_tokens=0,
+                num_hidden_cache_tokens=self.num_hidden_cache_tokens, num_tot_tokens=self.num_tot_tokens,
+                slot_mapping=self.slot_mapping[:self.num_prefill_tokens],
+                slot_mapping_shared=self.slot_mapping_shared, hidden_cache_use_tot=self.hidden_cache_use_tot,
+                kv_cache_use_tot=self.kv_cache_use_tot, hidden_cache_use_input=self.hidden_cache_use_input,
+                hidden_cache_store_tot=self.hidden_cache_store_tot, hidden_holder_upd=self.hidden_holder_upd,
+                hidden_holder_pull=self.hidden_holder_pull, seq_lens=self.seq_lens[:self.num_prefills],
+                seq_lens_tensor=self.seq_lens_tensor[:self.num_prefills], max_query_len=self.max_query_len,
+                max_prefill_seq_len=self.max_prefill_seq_len, max_decode_seq_len=0,
+                query_start_loc=self.query_start_loc[:self.num_prefills + 1],
+                seq_start_loc=self.seq_start_loc[:self.num_prefills + 1],
+                context_lens_tensor=self.context_lens_tensor[:self.num_prefills],
+                block_tables=self.block_tables[:self.num_prefills], use_cuda_graph=False,
+                input_positions=self.input_positions, block_types=None)
+        return self._cached_prefill_metadata
+
+    @property
+    def decode_metadata(self) -> Optional["HybridAttentionMetadata"]:
+        """aptserve_flash_attn.py:177-221."""
+        if self.num_decode_tokens == 0:
+            return None
+        if self._cached_decode_metadata is None:
+            self._cached_decode_metadata = HybridAttentionMetadata(
+                num_prefills=0, num_prefill_tokens=0, num_decode_tokens=self.num_decode_tokens,
+                num_hidden_cache_tokens=self.num_hidden_cache_tokens, num_tot_tokens=self.num_tot_tokens,
+                slot_mapping=self.slot_mapping[self.num_prefill_tokens:],
+                slot_mapping_shared=self.slot_mapping_shared, hidden_cache_use_tot=self.hidden_cache_use_tot,
+                kv_cache_use_tot=self.kv_cache_use_tot, hidden_cache_use_input=self.hidden_cache_use_input,
+                hidden_cache_store_tot=self.hidden_cache_store_tot, hidden_holder_upd=self.hidden_holder_upd,
+                hidden_holder_pull=self.hidden_holder_pull, seq_lens=None,
+                seq_lens_tensor=self.seq_lens_tensor[self.num_prefills:], max_query_len=None,
+                max_prefill_seq_len=0, max_decode_seq_len=self.max_decode_seq_len, query_start_loc=None,
+                seq_start_loc=None, context_lens_tensor=None, block_tables=self.block_tables[self.num_prefills:],
+                use_cuda_graph=self.use_cuda_graph, input_positions=self.input_positions,
+                block_types=None if self.block_types is None else self.block_types[self.num_prefills:])
+        return self._cached_decode_metadata
+
+
+class _Staging:
+    """Ring of pinned int32 staging buffers for the packed upload.  A buffer is
+    reused only after the copy that last read it has completed (its event)."""
+
+    def __init__(self, depth: int = 4):
+        self.bufs = [None] * depth
+        self.events = [None] * depth
+        self.next = 0
+
+    def take(self, n: int):
+        i = self.next
+        self.next = (i + 1) % len(self.bufs)
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        if self.bufs[i] is None or self.bufs[i].numel() < n:
+            self.bufs[i] = torch.empty(max(n, 4096), dtype=torch.int32, pin_memory=True)
+        return i, self.bufs[i][:n]
+
+    def upload(self, i: int, host: torch.Tensor, device) -> torch.Tensor:
+        dev = host.to(device, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(device))
+        self.events[i] = ev
+        return dev
+
+
+_staging = {}
+
+
+def _stage(device, n: int):
+    st = _staging.setdefault(device, _Staging())
+    i, host = st.take(n)
+    host.zero_()
+    return st, i, host
+
+
+def _pack_tables(tables: Sequence[Sequence[int]], width: int, out: np.ndarray) -> None:
+    for i, t in enumerate(tables):
+        n = min(len(t), width)
+        if n:
+            out[i, :n] = t[:n]
+
+
+def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequence[bool],
+                   block_tables: Sequence[Sequence[int]], block_tables_4_shared: Sequence[Sequence[int]],
+                   block_size: int, device, context_lens: Optional[Sequence[int]] = None,
+                   check_totals: bool = False) -> HybridAttentionMetadata:
+    """Build the metadata of one homogeneous batch (all prompts or all decodes, as the
+    reference's scheduler emits them, additional_designs/core/aptserve_scheduler.py:1613-1625).
+
+    ``block_tables[b]`` is sequence b's private table, ``block_tables_4_shared[b]`` its
+    shared (workspace) table (empty for K/V-cached sequences).  An empty private table
+    (the memory-profiling run) yields padding slots.
+    """
+    device = torch.device(device)
+    B = len(seq_lens)
+    if B == 0:
+        raise ValueError("empty batch")
+    lens = np.asarray(seq_lens, dtype=np.int64)
+    hid = np.asarray(use_hidden, dtype=bool)
+    if len(hid) != B or len(block_tables) != B:
+        raise ValueError("seq_lens, use_hidden and block_tables must have one entry per sequence")
+    if np.any(lens <= 0):
+        raise ValueError("sequence lengths must be positive")
+    need_blocks = -(-lens // block_size)
+    have_tables = any(len(t) for t in block_tables)
+    W = max(len(t) for t in block_tables) if have_tables else 0
+    if have_tables:
+        for b in range(B):
+            if len(block_tables[b]) < need_blocks[b]:
+                raise ValueError(f"sequence {b}: private block table shorter than ceil(seq_len/block_size)")
+    lib = _lib.load()
+    i64 = dict(dtype=torch.int64, device=device)
+    i32 = dict(dtype=torch.int32, device=device)
+
+    if not is_prompt:
+        if len(block_tables_4_shared) != B:
+            raise ValueError("block_tables_4_shared must have one entry per sequence")
+        for b in np.nonzero(hid)[0]:
+            if have_tables and len(block_tables_4_shared[b]) < need_blocks[b]:
+                raise ValueError(f"sequence {b}: shared block table shorter than ceil(seq_len/block_size)")
+        n_hs = int(hid.sum())
+        n_kv = B - n_hs
+        n_hr = int(lens[hid].sum())
+        num_tot = n_hr + n_kv
+        Ws = max((len(block_tables_4_shared[b]) for b in np.nonzero(hid)[0]), default=0) if have_tables else 0
+        # width of the table handed to attention: the longest *selected* table (:601-609)
+        Wo = max((len(block_tables_4_shared[b]) if hid[b] else len(block_tables[b]) for b in range(B)),
+                 default=0) if have_tables else 0
+        # one packed upload: lens | flags | private tables | shared tables
+        stg, slot, host = _stage(device, 2 * B + B * W + B * Ws)
+        hv = host.numpy()
+        hv[:B] = lens
+        hv[B:2 * B] = hid
+        if W:
+            _pack_tables(block_tables, W, hv[2 * B:2 * B + B * W].reshape(B, W))
+        if Ws:
+            _pack_tables(block_tables_4_shared, Ws, hv[2 * B + B * W:].reshape(B, Ws))
+        packed = stg.upload(slot, host, device)
+        d_lens, d_hid = packed[:B], packed[B:2 * B]
+        d_bt = packed[2 * B:2 * B + B * W].view(B, W)
+        d_bts = packed[2 * B + B * W:].view(B, Ws)
+        # one allocation per output dtype
+        sizes64 = [num_tot, n_hr, n_hr, n_kv, n_hs, n_hs, B, num_tot - B, B, 4]
+        buf64 = torch.empty(sum(sizes64), **i64)
+        (slot_mapping, slot_mapping_shared, use_tot, kv_use, use_input, store_tot, upd, pull, positions,
+         totals) = torch.split(buf64, sizes64)
+        sizes32 = [B * Wo, B + 1, B + 1, B]
+        buf32 = torch.empty(sum(sizes32), **i32)
+        bt_out, seq_start, query_start, ctx = torch.split(buf32, sizes32)
+        bt_out = bt_out.view(B, Wo)
+        with torch.cuda.device(device):
+            st = lib.aps_build_decode_metadata(
+                d_lens.data_ptr(), d_hid.data_ptr(), d_bt.data_ptr() if W else None, W, W,
+                d_bts.data_ptr() if Ws else None, Ws, Ws, B, block_size, slot_mapping.data_ptr(),
+                slot_mapping_shared.data_ptr() if n_hr else None, use_tot.data_ptr() if n_hr else None,
+                kv_use.data_ptr() if n_kv else None, use_input.data_ptr() if n_hs else None,
+                store_tot.data_ptr() if n_hs else None, upd.data_ptr(), pull.data_ptr() if num_tot > B else None,
+                num_tot, n_hr, n_hs, n_kv, bt_out.data_ptr() if Wo else None, Wo, Wo, seq_start.data_ptr(),
+                query_start.data_ptr(), ctx.data_ptr(), positions.data_ptr(), totals.data_ptr(),
+                torch.cuda.current_stream(device).cuda_stream)
+        _lib.check(st, "build_decode_metadata")
+        if check_totals:
+            got = totals.tolist()
+            if got != [num_tot, n_hr, n_hs, n_kv]:
+                raise RuntimeError(f"device totals {got} disagree with the host's {[num_tot, n_hr, n_hs, n_kv]}")
+        # per-block source for the hybrid attention: every block of a hidden sequence is a workspace block
+        block_types = d_hid.to(torch.uint8).unsqueeze(1).expand(B, Wo).contiguous() if (n_hs and Wo) else None
+        return HybridAttentionMetadata(
+            num_prefills=0, num_prefill_tokens=0, num_decode_tokens=B, num_hidden_cache_tokens=n_hs,
+            num_tot_tokens=num_tot, slot_mapping=slot_mapping, slot_mapping_shared=slot_mapping_shared,
+            hidden_cache_use_tot=use_tot, kv_cache_use_tot=kv_use, hidden_cache_use_input=use_input,
+            hidden_cache_store_tot=store_tot, hidden_holder_upd=upd, hidden_holder_pull=pull,
+            seq_lens=[int(x) for x in lens], seq_lens_tensor=d_lens, max_query_len=1, max_prefill_seq_len=0,
+            max_decode_seq_len=int(lens.max()), query_start_loc=query_start, seq_start_loc=seq_start,
+            context_lens_tensor=ctx, block_tables=bt_out, use_cuda_graph=False, input_positions=positions,
+            block_types=block_types)
+
+    # ------------------------------------------------------------------ prompts
+    ctxs = np.zeros(B, dtype=np.int64) if context_lens is None else np.asarray(context_lens, dtype=np.int64)
+    qlens = lens - ctxs
+    if np.any(qlens <= 0):
+        raise ValueError("every prompt needs at least one new token")
+    n_tok = int(qlens.sum())
+    n_ht = int(qlens[hid].sum())
+    n_kt = n_tok - n_ht
+    stg, slot, host = _stage(device, 3 * B + B * W)
+    hv = host.numpy()
+    hv[:B] = lens
+    hv[B:2 * B] = hid
+    hv[2 * B:3 * B] = ctxs
+    if W:
+        _pack_tables(block_tables, W, hv[3 * B:].reshape(B, W))
+    packed = stg.upload(slot, host, device)
+    d_lens, d_hid, d_ctx_in = packed[:B], packed[B:2 * B], packed[2 * B:3 * B]
+    d_bt = packed[3 * B:].view(B, W)
+    sizes64 = [n_tok, n_tok, n_ht, n_kt, 4]
+    buf64 = torch.empty(sum(sizes64), **i64)
+    slot_mapping, positions, use_input, kv_use, totals = torch.split(buf64, sizes64)
+    sizes32 = [B + 1, B + 1, B]
+    buf32 = torch.empty(sum(sizes32), **i32)
+    seq_start, query_start, ctx = torch.split(buf32, sizes32)
+    with torch.cuda.device(device):
+        st = lib.aps_build_prefill_metadata(
+            d_lens.data_ptr(), d_ctx_in.data_ptr(), d_hid.data_ptr(), d_bt.data_ptr() if W else None, W, W, B,
+            block_size, slot_mapping.data_ptr(), positions.data_ptr(), use_input.data_ptr() if n_ht else None,
+            kv_use.data_ptr() if n_kt else None, n_tok, n_ht, n_kt, seq_start.data_ptr(), query_start.data_ptr(),
+            ctx.data_ptr(), totals.data_ptr(), torch.cuda.current_stream(device).cuda_stream)
+    _lib.check(st, "build_prefill_metadata")
+    if check_totals:
+        got = totals.tolist()
+        if got[:2] != [n_tok, n_ht] or got[3] != n_kt:
+            raise RuntimeError(f"device totals {got} disagree with the host's {[n_tok, n_ht, n_kt]}")
+    empty64 = torch.empty(0, **i64)
+    return HybridAttentionMetadata(
+        num_prefills=B, num_prefill_tokens=n_tok, num_decode_tokens=0, num_hidden_cache_tokens=n_ht,
+        num_tot_tokens=n_tok, slot_mapping=slot_mapping, slot_mapping_shared=empty64,
+        hidden_cache_use_tot=use_input, kv_cache_use_tot=kv_use, hidden_cache_use_input=use_input,
+        hidden_cache_store_tot=use_input, hidden_holder_upd=empty64, hidden_holder_pull=empty64,
+        seq_lens=[int(x) for x in lens], seq_lens_tensor=d_lens, max_query_len=int(qlens.max()),
+        max_prefill_seq_len=int(lens.max()), max_decode_seq_len=0, query_start_loc=query_start,
+        seq_start_loc=seq_start, context_lens_tensor=ctx,
+        block_tables=torch.empty(B, 0, **i32), use_cuda_graph=False, input_positions=positions, block_types=None)
+
+
+def build_from_batch(batch, device, **kw) -> HybridAttentionMetadata:
+    """Convenience for :class:`aptserve_hip.workloads.Batch`."""
+    return build_metadata(batch.is_prompt, batch.seq_lens, batch.use_hidden, batch.block_tables,
+                          batch.block_tables_4_shared, batch.block_size, device, **kw)

@@ -253,3 +253,98 @@ def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
     with torch.cuda.device(src.device):
         st = _lib.load().aps_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, _stream(src))
     _lib.check(st, "copy_bytes")
+
+
+# --------------------------------------------------------------------- a8
+
+def paged_decode_attention(q, k_cache, v_cache, block_tables, seq_lens, softmax_scale=None, *,
+                           block_types=None, ws_k_cache=None, ws_v_cache=None, k_scale: float = 1.0,
+                           v_scale: float = 1.0, max_seq_len: Optional[int] = None, partition_size: int = 0,
+                           out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):
+    """Decode attention of one query token per sequence over paged K/V.
+
+    ``q`` ``[B, H, D]`` f16/bf16; caches ``[blocks, BS, H, D]`` in ``q``'s dtype or
+    uint8/float8_e4m3fn (fp8 codes, dequantised with ``k_scale``/``v_scale``);
+    ``block_tables`` int32 ``[B, W]``; ``seq_lens`` int32 ``[B]``.  ``block_types``
+    (uint8 ``[B, W]``, optional) sends a logical block to ``ws_k_cache``/``ws_v_cache``
+    when non-zero.  ``max_seq_len`` is a host-side bound on ``seq_lens`` (default
+    ``W * BS``, which needs no device read-back).  Returns ``[B, H, D]``.
+    """
+    dev = q.device
+    _check_data("q", q, dev)
+    _need(q.dim() == 3, "q must be [batch, heads, head_dim]")
+    B, H, D = q.shape
+    _need(q.dtype in (torch.float16, torch.bfloat16), "q must be float16 or bfloat16")
+    _need(q.stride(2) == 1 and q.stride(1) == D, "q: heads of one token must be contiguous")
+    _check_data("k_cache", k_cache, dev)
+    _check_data("v_cache", v_cache, dev)
+    _check_kv_cache("k_cache", k_cache, H, D)
+    _check_kv_cache("v_cache", v_cache, H, D)
+    _need(k_cache.dtype == v_cache.dtype and k_cache.stride(0) == v_cache.stride(0) and
+          k_cache.size(0) == v_cache.size(0), "k_cache and v_cache layouts differ")
+    fp8 = k_cache.element_size() == 1
+    _need(fp8 or k_cache.dtype == q.dtype, "cache dtype must equal q dtype or be an fp8 byte cache")
+    BS = k_cache.size(1)
+    _check_index("seq_lens", seq_lens, dev, torch.int32)
+    _need(seq_lens.numel() == B, "one seq_len per query expected")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.size(0) == B,
+          "block_tables must be int32 [batch, width]")
+    _need(block_tables.device == dev and (block_tables.size(1) <= 1 or block_tables.stride(1) == 1),
+          "block_tables rows must be contiguous on the same GPU")
+    W = block_tables.size(1)
+    ws_stride = ws_blocks = types_stride = 0
+    if block_types is not None:
+        _need(block_types.dtype == torch.uint8 and block_types.dim() == 2 and block_types.size(0) == B and
+              block_types.size(1) >= W and block_types.device == dev, "block_types must be uint8 [batch, >=width]")
+        _need(block_types.size(1) <= 1 or block_types.stride(1) == 1, "block_types rows must be contiguous")
+        _need(ws_k_cache is not None and ws_v_cache is not None, "block_types needs the workspace caches")
+        for n, c in (("ws_k_cache", ws_k_cache), ("ws_v_cache", ws_v_cache)):
+            _check_data(n, c, dev)
+            _check_kv_cache(n, c, H, D)
+            _need(c.dtype == k_cache.dtype and c.size(1) == BS, f"{n} must match the cache dtype and block size")
+        _need(ws_k_cache.stride(0) == ws_v_cache.stride(0) and ws_k_cache.size(0) == ws_v_cache.size(0),
+              "workspace K and V layouts differ")
+        ws_stride, ws_blocks, types_stride = ws_k_cache.stride(0), ws_k_cache.size(0), block_types.stride(0)
+    if softmax_scale is None:
+        softmax_scale = D ** -0.5
+    if max_seq_len is None:
+        max_seq_len = W * BS
+    max_seq_len = min(int(max_seq_len), W * BS)
+    if out is None:
+        out = torch.empty_like(q)
+    else:
+        _check_data("out", out, dev)
+        _need(out.shape == q.shape and out.dtype == q.dtype and out.stride(2) == 1 and out.stride(1) == D,
+              "out must look like q")
+    lib = _lib.load()
+    if partition_size <= 0:
+        partition_size = lib.aps_decode_attention_partition_size(B, H, max(max_seq_len, 1), BS)
+    need = lib.aps_decode_attention_workspace_bytes(B, H, D, max(max_seq_len, 1), partition_size)
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    ws_ptr = workspace.data_ptr() if (need and workspace is not None) else None
+    ws_bytes = workspace.numel() * workspace.element_size() if (need and workspace is not None) else 0
+    with torch.cuda.device(dev):
+        st = lib.aps_paged_decode_attention(
+            out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+            None if block_types is None else ws_k_cache.data_ptr(),
+            None if block_types is None else ws_v_cache.data_ptr(),
+            _ptr(block_tables), None if block_types is None else _ptr(block_types), _ptr(seq_lens), B, H, D, BS, W,
+            block_tables.stride(0) if W else 0, types_stride, q.stride(0), out.stride(0), k_cache.stride(0),
+            k_cache.size(0), ws_stride, ws_blocks, max_seq_len, partition_size, float(softmax_scale),
+            _DTYPE_CODE[q.dtype], APS_FP8_E4M3 if fp8 else _DTYPE_CODE[q.dtype], float(k_scale), float(v_scale),
+            ws_ptr, ws_bytes, _stream(q))
+    _lib.check(st, "paged_decode_attention")
+    return out
+
+
+def flash_attn_with_kvcache(q, k_cache, v_cache, block_table=None, cache_seqlens=None, softmax_scale=None,
+                            causal: bool = True, alibi_slopes=None, **kw):
+    """Decode case of the third-party function with the keyword names used at
+    additional_designs/attention/backends/aptserve_flash_attn.py:452-473:
+    ``q [B,1,H,D]`` -> ``[B,1,H,D]``."""
+    _need(q.dim() == 4 and q.size(1) == 1, "only one query token per sequence (decode) is supported")
+    _need(alibi_slopes is None, "alibi_slopes is not supported")
+    _need(block_table is not None and cache_seqlens is not None, "a paged cache needs block_table and cache_seqlens")
+    o = paged_decode_attention(q[:, 0], k_cache, v_cache, block_table, cache_seqlens, softmax_scale, **kw)
+    return o.unsqueeze(1)

@@ -1,0 +1,445 @@
+// Paged decode attention over a hybrid cache for gfx950.
+//
+// One wavefront (one 64-thread workgroup) owns (sequence, head, partition): a
+// partition is a run of `partition_size` consecutive tokens of one sequence.
+// Lane layout for a head vector of D elements: LPT = D*elem_bytes/16 lanes
+// hold one token (16 bytes each), so one wave-wide 128-bit load covers
+// TPL = 64/LPT tokens; a tile of 16 tokens (never crossing a block because the
+// block size is a multiple of 16) takes NG = 16/TPL loads for K and NG for V.
+// Each of the TPL token rows of the wave runs its own online softmax over the
+// tokens it sees (no cross-row traffic in the loop); rows are merged once at
+// the end.  The next tile's K/V are requested before the current tile is
+// consumed, so a wave keeps 2 tiles (2 x 16 tokens x 2 x D) in flight.
+//
+// Per tile the K or V source is chosen per block: block_types[b][i] != 0 reads
+// logical block i from the re-projection workspace, otherwise from the
+// persistent K/V cache.  Partitions of one (sequence, head) are combined by a
+// second small kernel through their log-sum-exp.
+#include <hip/hip_fp16.h>
+
+#include <math.h>
+
+#include "aps_common.h"
+
+namespace aps {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kTile = 16;  // tokens per tile
+constexpr float kLog2e = 1.4426950408889634f;
+
+enum KvKind { KV_F16 = 0, KV_BF16 = 1, KV_FP8 = 2 };
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+
+// Sum over groups of LPT consecutive lanes; every lane of the group gets the sum.
+template <int LPT>
+__device__ __forceinline__ float group_sum(float x) {
+  if constexpr (LPT >= 2) x += dpp_f32<0xB1>(x);   // quad_perm [1,0,3,2]
+  if constexpr (LPT >= 4) x += dpp_f32<0x4E>(x);   // quad_perm [2,3,0,1]
+  if constexpr (LPT >= 8) x += dpp_f32<0x141>(x);  // row_half_mirror
+  if constexpr (LPT >= 16) x += dpp_f32<0x140>(x); // row_mirror
+  if constexpr (LPT >= 32) x += __shfl_xor(x, 16);
+  return x;
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// 16 bytes of K or V as EPL floats.
+template <int KV>
+struct Unpack;
+template <>
+struct Unpack<KV_F16> {
+  static constexpr int EPL = 8;
+  __device__ static __forceinline__ void run(const u32x4& r, float (&f)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      // copy the lane out first: __builtin_bit_cast applied directly to a vector
+      // element reads element 0 whatever the index
+      const uint32_t w = r[i];
+      const half2_t h = __builtin_bit_cast(half2_t, w);
+      f[2 * i] = (float)h.x;
+      f[2 * i + 1] = (float)h.y;
+    }
+  }
+};
+template <>
+struct Unpack<KV_BF16> {
+  static constexpr int EPL = 8;
+  __device__ static __forceinline__ void run(const u32x4& r, float (&f)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = bf16_lo(r[i]);
+      f[2 * i + 1] = bf16_hi(r[i]);
+    }
+  }
+};
+template <>
+struct Unpack<KV_FP8> {
+  static constexpr int EPL = 16;
+  __device__ static __forceinline__ void run(const u32x4& r, float (&f)[16]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)r[i], false);
+      const float2_t hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)r[i], true);
+      f[4 * i] = lo.x; f[4 * i + 1] = lo.y; f[4 * i + 2] = hi.x; f[4 * i + 3] = hi.y;
+    }
+  }
+};
+
+template <int QT>
+__device__ __forceinline__ float q_to_f32(uint16_t bits) {
+  if constexpr (QT == APS_F16) return (float)__builtin_bit_cast(_Float16, bits);
+  else return __uint_as_float((uint32_t)bits << 16);
+}
+template <int QT>
+__device__ __forceinline__ uint16_t f32_to_q(float x) {
+  if constexpr (QT == APS_F16) {
+    return __builtin_bit_cast(uint16_t, (_Float16)x);
+  } else {  // bf16, round to nearest even
+    uint32_t u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+  }
+}
+
+struct AttnArgs {
+  void* out;                 // [B, H, D] (q dtype) — written when num_partitions == 1
+  float* part_out;           // [B, H, P, D] fp32
+  float* part_lse;           // [B, H, P]   fp32 (log2 domain)
+  const void* q;
+  const char* k_cache; const char* v_cache;
+  const char* ws_k_cache; const char* ws_v_cache;
+  const int32_t* block_tables; const uint8_t* block_types; const int32_t* seq_lens;
+  int64_t q_stride, out_stride, table_stride, types_stride;
+  int64_t cache_block_stride_b, ws_block_stride_b;  // bytes
+  int64_t num_cache_blocks, num_ws_blocks;
+  int num_heads, block_size, partition_size, num_partitions, table_width;
+  float scale_log2;  // softmax_scale * k_scale * log2(e)
+  float v_scale;
+};
+
+template <int QT, int KV, int D>
+__global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
+  constexpr int EPL = Unpack<KV>::EPL;        // elements per lane
+  constexpr int LPT = D / EPL;                // lanes per token
+  constexpr int TPL = 64 / LPT;               // tokens per wave-wide load
+  constexpr int NG = kTile / TPL;             // loads per tile and per K/V
+  static_assert(LPT >= 2 && LPT <= 32 && NG >= 1, "unsupported head size");
+  constexpr int KV_ELEM_B = (KV == KV_FP8) ? 1 : 2;
+
+  const int head = blockIdx.x;
+  const int part = blockIdx.y;
+  const int seq = blockIdx.z;
+  const int lane = threadIdx.x;
+  const int tl = lane / LPT;  // token row of this lane
+  const int dl = lane % LPT;  // 16-byte chunk of the head vector
+
+  const int seq_len = a.seq_lens[seq];
+  const int start = part * a.partition_size;
+  if (start >= seq_len && !(part == 0 && seq_len <= 0)) return;
+  const int end = min(seq_len, start + a.partition_size);
+  const int n_tiles = (end > start) ? (end - start + kTile - 1) / kTile : 0;
+
+  // query fragment of this lane, fp32
+  float qf[EPL];
+  {
+    const uint16_t* qp = (const uint16_t*)a.q + (int64_t)seq * a.q_stride + (int64_t)head * D + dl * EPL;
+#pragma unroll
+    for (int i = 0; i < EPL; i += 8) {
+      const u32x4 r = *(const u32x4*)(qp + i);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        qf[i + 2 * j] = q_to_f32<QT>((uint16_t)(r[j] & 0xffffu));
+        qf[i + 2 * j + 1] = q_to_f32<QT>((uint16_t)(r[j] >> 16));
+      }
+    }
+  }
+
+  // block ids (and types) of this partition: lane j holds logical block first_blk + j
+  const int first_blk = start / a.block_size;
+  const int n_blk = (end > start) ? (end - 1) / a.block_size - first_blk + 1 : 0;
+  int my_blk = -1;
+  int my_type = 0;
+  if (lane < n_blk && first_blk + lane < a.table_width) {
+    my_blk = a.block_tables[(int64_t)seq * a.table_stride + first_blk + lane];
+    if (a.block_types) my_type = a.block_types[(int64_t)seq * a.types_stride + first_blk + lane];
+  }
+
+  const int64_t row_b = (int64_t)a.num_heads * D * KV_ELEM_B;       // one token, all heads
+  const int64_t lane_off = (int64_t)head * D * KV_ELEM_B + dl * 16;  // this lane's chunk in a token row
+
+  float m = -INFINITY, l = 0.f;
+  float acc[EPL];
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) acc[i] = 0.f;
+
+  u32x4 kA[NG], vA[NG], kB[NG], vB[NG];
+
+  // Issue the loads of tile t into (kr, vr); returns false if the tile's block is unusable.
+  auto load_tile = [&](int t, u32x4(&kr)[NG], u32x4(&vr)[NG]) -> bool {
+    const int tok0 = start + t * kTile;
+    const int bi = tok0 / a.block_size - first_blk;
+    const int blk = __builtin_amdgcn_readlane(my_blk, bi);
+    const int type = __builtin_amdgcn_readlane(my_type, bi);
+    const bool ws = type != 0;
+    const int64_t nblk = ws ? a.num_ws_blocks : a.num_cache_blocks;
+    if (blk < 0 || blk >= nblk) return false;
+    const int64_t base = (int64_t)blk * (ws ? a.ws_block_stride_b : a.cache_block_stride_b) +
+                         (int64_t)(tok0 % a.block_size + tl) * row_b + lane_off;
+    const char* kp = (ws ? a.ws_k_cache : a.k_cache) + base;
+    const char* vp = (ws ? a.ws_v_cache : a.v_cache) + base;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      kr[g] = __builtin_nontemporal_load((const u32x4*)(kp + (int64_t)g * TPL * row_b));
+      vr[g] = __builtin_nontemporal_load((const u32x4*)(vp + (int64_t)g * TPL * row_b));
+    }
+    return true;
+  };
+
+  auto consume_tile = [&](int t, bool ok, const u32x4(&kr)[NG], const u32x4(&vr)[NG]) {
+    if (!ok) return;
+    const int tok0 = start + t * kTile;
+    const bool partial = tok0 + kTile > end;
+    float s[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      float kf[EPL];
+      Unpack<KV>::run(kr[g], kf);
+      float d = 0.f;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) d = fmaf(qf[i], kf[i], d);
+      d = group_sum<LPT>(d) * a.scale_log2;
+      s[g] = (tok0 + g * TPL + tl < end) ? d : -INFINITY;
+    }
+    float m_new = m;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) m_new = fmaxf(m_new, s[g]);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+    float p[NG];
+    float psum = 0.f;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      p[g] = __builtin_amdgcn_exp2f(s[g] - m_use);
+      psum += p[g];
+    }
+    l = l * alpha + psum;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) acc[i] *= alpha;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      float vf[EPL];
+      Unpack<KV>::run(vr[g], vf);
+      if (partial) {  // slots past the end of the sequence may hold anything, NaN included
+        const bool live = tok0 + g * TPL + tl < end;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) vf[i] = live ? vf[i] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) acc[i] = fmaf(p[g], vf[i], acc[i]);
+    }
+    m = m_new;
+  };
+
+  bool okA = false, okB = false;
+  if (n_tiles > 0) okA = load_tile(0, kA, vA);
+  for (int t = 0; t < n_tiles; t += 2) {
+    if (t + 1 < n_tiles) okB = load_tile(t + 1, kB, vB);
+    consume_tile(t, okA, kA, vA);
+    if (t + 2 < n_tiles) okA = load_tile(t + 2, kA, vA);
+    if (t + 1 < n_tiles) consume_tile(t + 1, okB, kB, vB);
+  }
+
+  // merge the TPL token rows (lanes that share dl)
+#pragma unroll
+  for (int off = LPT; off < 64; off <<= 1) {
+    const float m_o = __shfl_xor(m, off);
+    const float l_o = __shfl_xor(l, off);
+    const float m_n = fmaxf(m, m_o);
+    const float m_u = (m_n == -INFINITY) ? 0.f : m_n;
+    const float wa = __builtin_amdgcn_exp2f(m - m_u), wb = __builtin_amdgcn_exp2f(m_o - m_u);
+    l = l * wa + l_o * wb;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) acc[i] = acc[i] * wa + __shfl_xor(acc[i], off) * wb;
+    m = m_n;
+  }
+
+  if (tl != 0) return;
+  const float inv = (l > 0.f) ? a.v_scale / l : 0.f;
+  if (a.num_partitions == 1) {
+    uint16_t* op = (uint16_t*)a.out + (int64_t)seq * a.out_stride + (int64_t)head * D + dl * EPL;
+#pragma unroll
+    for (int i = 0; i < EPL; i += 8) {
+      u32x4 r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        r[j] = (uint32_t)f32_to_q<QT>(acc[i + 2 * j] * inv) |
+               ((uint32_t)f32_to_q<QT>(acc[i + 2 * j + 1] * inv) << 16);
+      *(u32x4*)(op + i) = r;
+    }
+  } else {
+    const int64_t ph = ((int64_t)seq * a.num_heads + head) * a.num_partitions + part;
+    float* po = a.part_out + ph * D + dl * EPL;
+#pragma unroll
+    for (int i = 0; i < EPL; i += 4) {
+      float4 r = make_float4(acc[i] * inv, acc[i + 1] * inv, acc[i + 2] * inv, acc[i + 3] * inv);
+      *(float4*)(po + i) = r;
+    }
+    if (dl == 0) a.part_lse[ph] = (l > 0.f) ? m + log2f(l) : -INFINITY;
+  }
+}
+
+// out[b,h,:] = sum_p w_p * part_out[b,h,p,:] / sum_p w_p,  w_p = 2^(lse_p - max lse)
+template <int QT>
+__global__ __launch_bounds__(256) void combine_partitions_kernel(void* out, const float* part_out,
+                                                                const float* part_lse, const int32_t* seq_lens,
+                                                                int64_t out_stride, int num_heads, int head_size,
+                                                                int num_partitions, int partition_size) {
+  const int head = blockIdx.x, seq = blockIdx.y;
+  const int seq_len = seq_lens[seq];
+  int np = (seq_len + partition_size - 1) / partition_size;
+  if (np < 1) np = 1;
+  if (np > num_partitions) np = num_partitions;
+  const int64_t ph = ((int64_t)seq * num_heads + head) * num_partitions;
+  float mx = -INFINITY;
+  for (int p = 0; p < np; ++p) mx = fmaxf(mx, part_lse[ph + p]);
+  uint16_t* op = (uint16_t*)out + (int64_t)seq * out_stride + (int64_t)head * head_size;
+  for (int d = threadIdx.x; d < head_size; d += blockDim.x) {
+    float num = 0.f, den = 0.f;
+    if (mx != -INFINITY) {
+      for (int p = 0; p < np; ++p) {
+        const float w = __builtin_amdgcn_exp2f(part_lse[ph + p] - mx);
+        num = fmaf(w, part_out[(ph + p) * head_size + d], num);
+        den += w;
+      }
+    }
+    op[d] = f32_to_q<QT>(den > 0.f ? num / den : 0.f);
+  }
+}
+
+template <int QT, int KV>
+int launch_decode(const AttnArgs& a, int head_size, int64_t batch, hipStream_t s) {
+  const dim3 grid((unsigned)a.num_heads, (unsigned)a.num_partitions, (unsigned)batch);
+  switch (head_size) {
+    case 64: hipLaunchKernelGGL((paged_decode_kernel<QT, KV, 64>), grid, dim3(64), 0, s, a); break;
+    case 128: hipLaunchKernelGGL((paged_decode_kernel<QT, KV, 128>), grid, dim3(64), 0, s, a); break;
+    case 256: hipLaunchKernelGGL((paged_decode_kernel<QT, KV, 256>), grid, dim3(64), 0, s, a); break;
+    case 32:
+      if constexpr (KV == KV_FP8) return APS_ERR_UNSUPPORTED;
+      else hipLaunchKernelGGL((paged_decode_kernel<QT, KV, 32>), grid, dim3(64), 0, s, a);
+      break;
+    default: return APS_ERR_UNSUPPORTED;
+  }
+  int st = launch_status();
+  if (st != APS_OK || a.num_partitions == 1) return st;
+  const int threads = head_size >= 256 ? 256 : (head_size + 63) / 64 * 64;
+  hipLaunchKernelGGL((combine_partitions_kernel<QT>), dim3((unsigned)a.num_heads, (unsigned)batch), dim3(threads), 0,
+                     s, a.out, a.part_out, a.part_lse, a.seq_lens, a.out_stride, a.num_heads, head_size,
+                     a.num_partitions, a.partition_size);
+  return launch_status();
+}
+
+inline int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
+
+}  // namespace
+}  // namespace aps
+
+using namespace aps;
+
+extern "C" {
+
+int aps_decode_attention_partition_size(int64_t batch, int num_heads, int64_t max_seq_len, int block_size) {
+  if (batch <= 0 || num_heads <= 0 || max_seq_len <= 0 || block_size <= 0) return 256;
+  // Aim for a few thousand wavefronts (256 compute units x 8-16 resident waves);
+  // shorten the partitions of small batches, never below two tiles.
+  int64_t part = 256;
+  while (part > 32 && batch * num_heads * ((max_seq_len + part - 1) / part) < 4096) part >>= 1;
+  if (part % block_size != 0) part = (part + block_size - 1) / block_size * block_size;
+  return (int)part;
+}
+
+int64_t aps_decode_attention_workspace_bytes(int64_t batch, int num_heads, int head_size, int64_t max_seq_len,
+                                             int partition_size) {
+  if (batch <= 0 || num_heads <= 0 || head_size <= 0 || max_seq_len <= 0 || partition_size <= 0) return 0;
+  const int64_t np = (max_seq_len + partition_size - 1) / partition_size;
+  if (np <= 1) return 0;
+  const int64_t n = batch * num_heads * np;
+  return align_up(n * head_size * 4, 256) + align_up(n * 4, 256);
+}
+
+int aps_paged_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
+                               const void* ws_k_cache, const void* ws_v_cache, const int32_t* block_tables,
+                               const uint8_t* block_types, const int32_t* seq_lens, int64_t batch, int num_heads,
+                               int head_size, int block_size, int64_t table_width, int64_t table_stride,
+                               int64_t types_stride, int64_t q_stride, int64_t out_stride,
+                               int64_t cache_block_stride, int64_t num_cache_blocks, int64_t ws_block_stride,
+                               int64_t num_ws_blocks, int64_t max_seq_len, int partition_size, float softmax_scale,
+                               int q_dtype, int kv_dtype, float k_scale, float v_scale, void* workspace,
+                               int64_t workspace_bytes, aps_stream_t stream) {
+  if (batch < 0 || num_heads <= 0 || head_size <= 0 || block_size <= 0 || table_width < 0) return APS_ERR_INVALID_ARG;
+  if (batch == 0) return APS_OK;
+  if (!out || !q || !seq_lens) return APS_ERR_INVALID_ARG;
+  if (max_seq_len > 0 && (!k_cache || !v_cache || !block_tables)) return APS_ERR_INVALID_ARG;
+  if (block_types && (!ws_k_cache || !ws_v_cache)) return APS_ERR_INVALID_ARG;
+  if (block_size % kTile != 0) return APS_ERR_UNSUPPORTED;
+  if (q_dtype != APS_F16 && q_dtype != APS_BF16) return APS_ERR_UNSUPPORTED;
+  if (kv_dtype != q_dtype && kv_dtype != APS_FP8_E4M3) return APS_ERR_UNSUPPORTED;
+  if (q_stride < (int64_t)num_heads * head_size || out_stride < (int64_t)num_heads * head_size)
+    return APS_ERR_INVALID_ARG;
+  const int kv_b = kv_dtype == APS_FP8_E4M3 ? 1 : 2;
+  const int64_t row = (int64_t)num_heads * head_size;
+  if (cache_block_stride < row * block_size || (block_types && ws_block_stride < row * block_size))
+    return APS_ERR_INVALID_ARG;
+  if (common_vec_bytes({addr(q), addr(out), (uint64_t)q_stride * 2, (uint64_t)out_stride * 2, addr(k_cache),
+                        addr(v_cache), addr(ws_k_cache), addr(ws_v_cache), (uint64_t)cache_block_stride * kv_b,
+                        (uint64_t)ws_block_stride * kv_b, (uint64_t)head_size * kv_b}) != 16)
+    return APS_ERR_UNSUPPORTED;
+  if (max_seq_len < 1) max_seq_len = 1;
+  if (partition_size <= 0)
+    partition_size = aps_decode_attention_partition_size(batch, num_heads, max_seq_len, block_size);
+  if (partition_size % block_size != 0 || partition_size / block_size > 64) return APS_ERR_INVALID_ARG;
+  const int64_t np = (max_seq_len + partition_size - 1) / partition_size;
+  if (np > 65535 || batch > 65535) return APS_ERR_UNSUPPORTED;
+
+  AttnArgs a;
+  a.out = out;
+  a.q = q;
+  a.k_cache = (const char*)k_cache; a.v_cache = (const char*)v_cache;
+  a.ws_k_cache = (const char*)ws_k_cache; a.ws_v_cache = (const char*)ws_v_cache;
+  a.block_tables = block_tables; a.block_types = block_types; a.seq_lens = seq_lens;
+  a.q_stride = q_stride; a.out_stride = out_stride; a.table_stride = table_stride; a.types_stride = types_stride;
+  a.cache_block_stride_b = cache_block_stride * kv_b; a.ws_block_stride_b = ws_block_stride * kv_b;
+  a.num_cache_blocks = num_cache_blocks; a.num_ws_blocks = num_ws_blocks;
+  a.num_heads = num_heads; a.block_size = block_size; a.partition_size = partition_size;
+  a.num_partitions = (int)np; a.table_width = (int)table_width;
+  const float ks = kv_dtype == APS_FP8_E4M3 ? k_scale : 1.f;
+  a.scale_log2 = softmax_scale * ks * kLog2e;
+  a.v_scale = kv_dtype == APS_FP8_E4M3 ? v_scale : 1.f;
+  a.part_out = nullptr; a.part_lse = nullptr;
+  if (np > 1) {
+    const int64_t need = aps_decode_attention_workspace_bytes(batch, num_heads, head_size, max_seq_len, partition_size);
+    if (!workspace || workspace_bytes < need || (addr(workspace) & 15)) return APS_ERR_WORKSPACE;
+    const int64_t n = batch * num_heads * np;
+    a.part_out = (float*)workspace;
+    a.part_lse = (float*)((char*)workspace + align_up(n * head_size * 4, 256));
+  }
+  hipStream_t s = (hipStream_t)stream;
+  if (q_dtype == APS_F16) {
+    return kv_dtype == APS_FP8_E4M3 ? launch_decode<APS_F16, KV_FP8>(a, head_size, batch, s)
+                                    : launch_decode<APS_F16, KV_F16>(a, head_size, batch, s);
+  }
+  return kv_dtype == APS_FP8_E4M3 ? launch_decode<APS_BF16, KV_FP8>(a, head_size, batch, s)
+                                  : launch_decode<APS_BF16, KV_BF16>(a, head_size, batch, s);
+}
+
+}  // extern "C"

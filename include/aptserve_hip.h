@@ -142,6 +142,106 @@ int aps_mixed_kv_to_cache(const void* key, const void* value, void* k_cache,
                           int64_t num_shared_blocks, int elem_size,
                           unsigned flags, aps_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * Paged decode attention (one query token per sequence) over a hybrid cache.
+ * ------------------------------------------------------------------------ */
+
+/* Partition length (tokens) the library would choose for this problem; a
+ * sequence longer than one partition is split and recombined (split-KV). */
+int aps_decode_attention_partition_size(int64_t batch, int num_heads,
+                                        int64_t max_seq_len, int block_size);
+
+/* Bytes of scratch aps_paged_decode_attention needs (0 if every sequence
+ * fits one partition).  The caller owns the scratch. */
+int64_t aps_decode_attention_workspace_bytes(int64_t batch, int num_heads,
+                                             int head_size,
+                                             int64_t max_seq_len,
+                                             int partition_size);
+
+/* ref: third-party vllm_flash_attn.flash_attn_with_kvcache as called at
+ * attention/backends/aptserve_flash_attn.py:452-461 (private cache) and
+ * :464-473 (shared cache):  for sequence b, head h, L = seq_lens[b]:
+ *   out[b,h,:] = softmax_j(softmax_scale * <q[b,h,:], K_j>) V,  j in [0,L)
+ *   K_j / V_j  = cache[block_tables[b, j/BS], j%BS, h, :]
+ * in fp32, result rounded to q's dtype.  seq_lens[b] <= 0 gives zeros.
+ *
+ * Hybrid extension: block_types (nullable, uint8 [batch, >=table_width],
+ * row stride types_stride) selects per logical block the persistent cache
+ * (0) or the re-projection workspace caches ws_k_cache/ws_v_cache (!= 0),
+ * which share the [blocks, BS, H, D] layout and kv_dtype.
+ *
+ * q/out: [batch, H, D] f16 or bf16, row strides q_stride/out_stride.
+ * kv_dtype: equal to q_dtype, or APS_FP8_E4M3 (K = code*k_scale, V = code*
+ * v_scale).  head_size in {32,64,128,256} (no 32 with fp8); block_size a
+ * multiple of 16.  block ids outside [0, num_*_blocks) contribute nothing.
+ * max_seq_len: host-side upper bound of seq_lens (sizes the partition grid).
+ * partition_size: 0 = library default, else a multiple of block_size with
+ * at most 64 blocks. */
+int aps_paged_decode_attention(
+    void* out, const void* q, const void* k_cache, const void* v_cache,
+    const void* ws_k_cache, const void* ws_v_cache,
+    const int32_t* block_tables, const uint8_t* block_types,
+    const int32_t* seq_lens, int64_t batch, int num_heads, int head_size,
+    int block_size, int64_t table_width, int64_t table_stride,
+    int64_t types_stride, int64_t q_stride, int64_t out_stride,
+    int64_t cache_block_stride, int64_t num_cache_blocks,
+    int64_t ws_block_stride, int64_t num_ws_blocks, int64_t max_seq_len,
+    int partition_size, float softmax_scale, int q_dtype, int kv_dtype,
+    float k_scale, float v_scale, void* workspace, int64_t workspace_bytes,
+    aps_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Ragged-batch metadata, built on the GPU from a per-sequence description.
+ * ref: worker/aptserve_model_runner.py:240-842 (_prepare_model_input), hybrid
+ * parts :256-304, :410-437, :516-564, :601-668, :707-733, :772-785.
+ * Inputs are int32 device arrays of one entry per sequence (use_hidden: 0/1)
+ * and 0-padded block tables; outputs are caller-allocated with the given
+ * capacities (entries beyond a capacity are dropped, never written).
+ * totals (nullable, int64[4]) receives {rows, hidden rows, hidden sequences,
+ * K/V rows or sequences} as computed on the device.
+ * ------------------------------------------------------------------------ */
+
+/* Decode step (:525-539, :554-564, :617-645).  Row space "tot": a hidden-cached
+ * sequence contributes seq_len rows (its whole context is re-projected), a
+ * K/V-cached one a single row.
+ *   slot_mapping[row]        private slot of token j (hidden) / of the new token (K/V)
+ *   slot_mapping_shared[i]   slot of token j in the shared (workspace) table, hidden rows only
+ *   hidden_cache_use_tot / kv_cache_use_tot    rows by cache type, ascending
+ *   hidden_holder_upd[b]     row of sequence b's newest token; hidden_holder_pull = the rest
+ *   hidden_cache_use_input   batch positions of hidden sequences
+ *   hidden_cache_store_tot   their newest rows
+ *   block_tables_out[b,:]    shared table for hidden sequences, private otherwise (:415-418)
+ *   seq_start_loc / query_start_loc int32 cumulative sums with leading 0;
+ *   context_lens = seq_len-1; input_positions = seq_len-1. */
+int aps_build_decode_metadata(
+    const int32_t* seq_lens, const int32_t* use_hidden,
+    const int32_t* block_tables, int64_t table_stride, int64_t table_width,
+    const int32_t* block_tables_shared, int64_t shared_stride,
+    int64_t shared_width, int64_t batch, int block_size, int64_t* slot_mapping,
+    int64_t* slot_mapping_shared, int64_t* hidden_cache_use_tot,
+    int64_t* kv_cache_use_tot, int64_t* hidden_cache_use_input,
+    int64_t* hidden_cache_store_tot, int64_t* hidden_holder_upd,
+    int64_t* hidden_holder_pull, int64_t cap_rows, int64_t cap_hidden_rows,
+    int64_t cap_hidden_seqs, int64_t cap_kv_seqs, int32_t* block_tables_out,
+    int64_t out_stride, int64_t out_width, int32_t* seq_start_loc,
+    int32_t* query_start_loc, int32_t* context_lens, int64_t* input_positions,
+    int64_t* totals, aps_stream_t stream);
+
+/* Prompt step (:542-552, :648-666).  Row space = token space; token i of a
+ * sequence (i in [context_len, seq_len)) gets slot table[i/BS]*BS + i%BS, or
+ * -1 when table_width is 0.  hidden_cache_use_input = tokens of hidden-cached
+ * prompts (it also serves as hidden_cache_use_tot and hidden_cache_store_tot),
+ * kv_cache_use_tot = the other tokens.  context_lens_in may be NULL (= 0). */
+int aps_build_prefill_metadata(
+    const int32_t* seq_lens, const int32_t* context_lens_in,
+    const int32_t* use_hidden, const int32_t* block_tables,
+    int64_t table_stride, int64_t table_width, int64_t batch, int block_size,
+    int64_t* slot_mapping, int64_t* input_positions,
+    int64_t* hidden_cache_use_input, int64_t* kv_cache_use_tot,
+    int64_t cap_tokens, int64_t cap_hidden_tokens, int64_t cap_kv_tokens,
+    int32_t* seq_start_loc, int32_t* query_start_loc, int32_t* context_lens,
+    int64_t* totals, aps_stream_t stream);
+
 /* Plain device copy of nbytes (16-byte aligned pointers): the known-size
  * kernel that hardware counters of the kernels above are scaled against. */
 int aps_copy_bytes(void* dst, const void* src, int64_t nbytes,
