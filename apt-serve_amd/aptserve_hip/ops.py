@@ -136,6 +136,35 @@ def hybrid_decode_gather(holder, hidden_states, paged_cache, slot_mapping, hidde
     _lib.check(st, "hybrid_decode_gather")
 
 
+def gather_hidden_rows(holder, hidden_states, paged_cache, holder_src, slot_mapping, hidden_cache_use_input,
+                       hidden_cache_store_tot) -> None:
+    """``hybrid_decode_gather`` with the row sources resolved by the metadata builder
+    (``HybridAttentionMetadata.holder_src``): same result, one index load per chunk."""
+    dev = holder.device
+    for n, t in (("holder", holder), ("hidden_states", hidden_states), ("paged_cache", paged_cache)):
+        _check_data(n, t, dev)
+    _need(holder.dim() == 2 and hidden_states.dim() == 2, "holder and hidden_states must be 2-D")
+    _need(holder.size(1) == hidden_states.size(1), "holder and hidden_states widths differ")
+    _need(holder.dtype == hidden_states.dtype == paged_cache.dtype, "dtypes differ")
+    _check_paged(paged_cache, holder.size(1))
+    for n, t in (("holder_src", holder_src), ("slot_mapping", slot_mapping),
+                 ("hidden_cache_use_input", hidden_cache_use_input),
+                 ("hidden_cache_store_tot", hidden_cache_store_tot)):
+        _check_index(n, t, dev)
+    _need(holder_src.numel() == holder.size(0), "holder_src must have one entry per holder row")
+    _need(slot_mapping.numel() == holder.size(0), "slot_mapping must have one entry per holder row")
+    _need(hidden_cache_use_input.numel() == hidden_cache_store_tot.numel(), "store index lengths differ")
+    slot_stride = paged_cache.stride(2)
+    with torch.cuda.device(dev):
+        st = _lib.load().aps_gather_hidden_rows(
+            holder.data_ptr(), hidden_states.data_ptr(), paged_cache.data_ptr(), _ptr(holder_src), holder.size(0),
+            _ptr(slot_mapping), _ptr(hidden_cache_use_input), _ptr(hidden_cache_store_tot),
+            hidden_cache_store_tot.numel(), hidden_states.size(0), holder.size(1), holder.stride(0),
+            hidden_states.stride(0), slot_stride, paged_cache.numel() // slot_stride, holder.element_size(),
+            _stream(holder))
+    _lib.check(st, "gather_hidden_rows")
+
+
 # --------------------------------------------------------------------- a3 / a4
 
 def _check_kv_cache(name: str, c: torch.Tensor, heads: int, head_size: int) -> None:

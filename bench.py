@@ -1,0 +1,261 @@
+#!/usr/bin/env python3
+"""Benchmark of the hybrid-cache hot path on one MI355X.
+
+A "step" is one pass of the per-layer cache traffic of a decode step at OPT-13B
+shapes (256 sequences, half of them hidden-cached, lognormal context lengths):
+store the new hidden rows, write the new K/V rows, and gather every hidden
+context row into the contiguous holder that feeds the K/V re-projection.
+``value`` is the algorithmic GB/s of that step with all inputs resident in HBM.
+The line also reports decode-attention tokens/s (fp16 and fp8 caches) and, when
+built, the re-projection TFLOP/s, each with its own roofline fraction, plus a
+CPU baseline of the same step timed on this host's cores with the oracle.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for p in (ROOT, ROOT / "apt-serve_amd"):
+    if str(p) not in sys.path:
+        sys.path.insert(0, str(p))
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip attention / re-projection figures")
+    return ap.parse_args()
+
+
+def median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def event_times(torch, fn, n, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return [a.elapsed_time(b) for a, b in evs]
+
+
+def attention_figures(torch, ops, workloads, np, dev, seed, fp8):
+    """Config 4: 128 sequences, 40x128, 65536-block pool, each block from the workspace with p=0.5."""
+    H, D, BS, B, POOL = 40, 128, 16, 128, 65536
+    rng = np.random.default_rng(seed)
+    lens = workloads.lognormal_lengths(rng, B)
+    nblk = [-(-int(l) // BS) for l in lens]
+    W = max(nblk)
+    ids = rng.permutation(POOL)[:sum(nblk)]
+    bt = np.zeros((B, W), dtype=np.int32)
+    p = 0
+    for b, n in enumerate(nblk):
+        bt[b, :n] = ids[p:p + n]
+        p += n
+    types = (rng.random((B, W)) < 0.5).astype(np.uint8)
+    g = torch.Generator(device=dev).manual_seed(seed)
+
+    def pool():
+        x = torch.empty(POOL, BS, H, D, dtype=torch.uint8 if fp8 else torch.float16, device=dev)
+        for i in range(0, POOL, 8192):
+            r = torch.randn(8192, BS, H, D, generator=g, dtype=torch.float32, device=dev)
+            x[i:i + 8192] = (torch.clamp(r / 0.04, -448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+                             if fp8 else r.to(torch.float16))
+        return x
+    kc, vc, wk, wv = pool(), pool(), pool(), pool()
+    q = torch.randn(B, H, D, generator=g, dtype=torch.float32, device=dev).half()
+    d_bt, d_ty = torch.from_numpy(bt).to(dev), torch.from_numpy(types).to(dev)
+    d_sl = torch.from_numpy(lens.astype(np.int32)).to(dev)
+    out = torch.empty_like(q)
+    max_len = int(lens.max())
+    fn = lambda: ops.paged_decode_attention(q, kc, vc, d_bt, d_sl, D ** -0.5, block_types=d_ty, ws_k_cache=wk,
+                                            ws_v_cache=wv, k_scale=0.04, v_scale=0.04, max_seq_len=max_len, out=out)
+    ms = median(event_times(torch, fn, 30))
+    total = int(lens.sum())
+    nbytes = total * 2 * H * D * (1 if fp8 else 2)
+    gbs = nbytes / ms / 1e6
+    return {"workload": "config4 paged hybrid decode attention, B=128, 40x128, sum(L)=%d, %s cache" %
+                        (total, "fp8-e4m3" if fp8 else "fp16"),
+            "tokens_per_s": B / (ms * 1e-3), "ms": ms, "algorithmic_bytes": nbytes,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+    from aptserve_hip import metadata, ops, workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    H, D, BS = 40, 128, 16
+    Hd = H * D
+
+    # ---- workload: BASELINE.json configs[1]
+    batch = workloads.decode_batch_opt13b(args.seed)
+    md = metadata.build_from_batch(batch, dev, check_totals=True)
+    N, B, T = batch.num_blocks, len(batch.seq_lens), md.num_tot_tokens
+    n_hidden_rows = md.hidden_cache_use_tot.numel()
+    n_hidden_seqs = md.num_hidden_cache_tokens
+    n_kv_seqs = B - n_hidden_seqs
+    g = torch.Generator(device=dev).manual_seed(args.seed)
+    cache = torch.empty(2, N, BS, H, D, dtype=torch.float16, device=dev)
+    for i in range(0, N, 4096):
+        cache[:, i:i + 4096] = torch.randn(2, min(4096, N - i), BS, H, D, generator=g, device=dev).half()
+    hs = torch.randn(B, Hd, generator=g, device=dev).half()
+    kv = torch.randn(B, 2 * Hd, generator=g, device=dev).half()
+    key, value = (x.view(B, H, D) for x in kv.chunk(2, -1))
+    holder = torch.empty(T, Hd, dtype=torch.float16, device=dev)
+    kv_seq_idx = torch.tensor([i for i, h in enumerate(batch.use_hidden) if not h], dtype=torch.int64, device=dev)
+    new_slots = torch.full((B,), -1, dtype=torch.int64, device=dev)
+    new_slots[kv_seq_idx] = md.slot_mapping[md.kv_cache_use_tot]
+
+    write_bytes = n_kv_seqs * 2 * (2 * Hd * 2) + n_hidden_seqs * 2 * (Hd * 2)   # read + write of each new row
+    gather_bytes = n_hidden_rows * 2 * (Hd * 2)                                 # read + write of each context row
+    step_bytes = write_bytes + gather_bytes
+
+    gather_events = []
+
+    def step(timed=False):
+        # new K/V rows of the K/V-cached sequences -> private cache
+        ops.reshape_and_cache_flash(key, value, cache[0], cache[1], new_slots, "auto", token_idx=kv_seq_idx)
+        # new hidden rows -> hidden blocks, and the holder of every row that is re-projected
+        if timed:
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+        ops.gather_hidden_rows(holder, hs, cache, md.holder_src, md.slot_mapping, md.hidden_cache_use_input,
+                               md.hidden_cache_store_tot)
+        if timed:
+            b.record()
+            gather_events.append((a, b))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(timed=True)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    step_gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
+    gather_ms = sum(a.elapsed_time(b) for a, b in gather_events) / len(gather_events)
+    # the gather launch also carries the B newest rows (upd) and the hidden stores; count only what 8(d) counts
+    gather_alg = gather_bytes + n_hidden_seqs * 2 * (Hd * 2)
+    achieved = gather_alg / gather_ms / 1e6
+
+    result = {
+        "metric": "hybrid-cache write/gather GB/s + decode attn tokens/s, OPT-13B shapes, 1 MI355X",
+        "value": step_gbs, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: hybrid cache write + hidden-block gather, OPT-13B 40x128, "
+                               "decode batch 256 (128 K/V + 128 hidden), lognormal(6.2,0.8) contexts in [16,2048]",
+                   "seed": args.seed, "hidden_rows_gathered": n_hidden_rows, "rows_total": T,
+                   "step_bytes": step_bytes, "write_bytes": write_bytes, "gather_bytes": gather_bytes,
+                   "launches_per_step": 2},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "row_mover<16,ResolvedGatherOp>",
+                     "algorithmic_bytes_per_launch": gather_alg, "avg_launch_ms": gather_ms},
+    }
+
+    if not args.no_extras:
+        extras = {}
+        del holder
+        for fp8 in (False, True):
+            torch.cuda.empty_cache()
+            extras["decode_attention_fp8" if fp8 else "decode_attention_f16"] = attention_figures(
+                torch, ops, workloads, np, dev, args.seed, fp8)
+        # metadata build, GPU vs the list-based host algorithm
+        t = []
+        for _ in range(10):
+            torch.cuda.synchronize()
+            a = time.perf_counter()
+            metadata.build_from_batch(batch, dev)
+            torch.cuda.synchronize()
+            t.append((time.perf_counter() - a) * 1e6)
+        extras["metadata_build_us"] = median(t)
+        if hasattr(ops, "kv_reproject"):
+            extras.update(reproject_figures(torch, ops, dev, args.seed))
+        result["extras"] = extras
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, np, batch, md, cache, hs, key, value, kv_seq_idx, new_slots,
+                                              step_bytes, T, Hd)
+    print(json.dumps(result))
+
+
+def reproject_figures(torch, ops, dev, seed):
+    out = {}
+    Hd = 5120
+    g = torch.Generator(device=dev).manual_seed(seed)
+    w = (torch.randn(2 * Hd, Hd, generator=g, device=dev) * 0.02).half()
+    bias = torch.randn(2 * Hd, generator=g, device=dev).half()
+    for T in (4096, 16384):
+        x = torch.randn(T, Hd, generator=g, device=dev).half()
+        y = torch.empty(T, 2 * Hd, dtype=torch.float16, device=dev)
+        ms = median(event_times(torch, lambda: ops.kv_reproject(x, w, bias, out=y), 20))
+        flops = 2.0 * T * Hd * 2 * Hd
+        tf = flops / ms / 1e9
+        out["kv_reproject_T%d" % T] = {
+            "workload": "config3 [T,5120]x[5120,10240] f16, f32 accumulate, T=%d" % T, "ms": ms, "tflops": tf,
+            "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": None}}
+    return out
+
+
+def cpu_baseline(torch, np, batch, md, cache, hs, key, value, kv_seq_idx, new_slots, step_bytes, T, Hd):
+    """The same step with the oracle (PyTorch-CPU index_put_/index_select) on this host's cores."""
+    from oracle import cache_ops as OC
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    c_cache, c_hs = cache.cpu(), hs.cpu()
+    c_key, c_val = key.cpu(), value.cpu()
+    idx = {k: getattr(md, k).cpu() for k in ("slot_mapping", "hidden_holder_upd", "hidden_cache_use_tot",
+                                             "hidden_cache_use_input", "hidden_cache_store_tot")}
+    c_seq, c_slots = kv_seq_idx.cpu(), new_slots.cpu()[kv_seq_idx.cpu()]
+
+    def step():
+        OC.reshape_and_cache_flash(c_key[c_seq], c_val[c_seq], c_cache[0], c_cache[1], c_slots, "auto")
+        OC.hidden_to_cache(c_hs, c_cache, idx["slot_mapping"], idx["hidden_cache_use_input"],
+                           idx["hidden_cache_store_tot"])
+        return OC.assemble_hidden_holder(c_hs, c_cache, idx["slot_mapping"], T, idx["hidden_holder_upd"],
+                                         idx["hidden_cache_use_tot"])
+    ts = []
+    for i in range(7):
+        a = time.perf_counter()
+        step()
+        if i >= 2:
+            ts.append(time.perf_counter() - a)
+    s = median(ts)
+    return {"value": step_bytes / s / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "host_cpus": threads,
+            "sample": "the full configs[1] step (same batch, seed and bytes as the GPU leg), 2 warm-ups, "
+                      "median of 5 runs, %.3f s per step" % s}
+
+
+if __name__ == "__main__":
+    main()

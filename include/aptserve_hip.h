@@ -101,6 +101,24 @@ int aps_hybrid_decode_gather(void* holder, const void* hidden_states,
                              int64_t num_tot_tokens, int elem_size,
                              aps_stream_t stream);
 
+/* Same result as aps_hybrid_decode_gather with the source of every holder row
+ * resolved beforehand (aps_build_decode_metadata writes holder_src):
+ *   holder_src[t] >= 0        holder[t] = cache slot holder_src[t]
+ *   holder_src[t] = -(b+1)    holder[t] = hidden_states[b], b < num_inputs
+ *   anything else             holder[t] = 0 (padding slot)
+ * plus the n_store stores of the newest hidden rows into the cache.  One
+ * dependent index load per chunk instead of two. */
+int aps_gather_hidden_rows(void* holder, const void* hidden_states,
+                           void* paged_cache, const int64_t* holder_src,
+                           int64_t n_rows, const int64_t* slot_mapping,
+                           const int64_t* hidden_cache_use_input,
+                           const int64_t* hidden_cache_store_tot,
+                           int64_t n_store, int64_t num_inputs,
+                           int64_t hidden_size, int64_t holder_stride,
+                           int64_t hidden_stride, int64_t slot_stride,
+                           int64_t num_slots, int elem_size,
+                           aps_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * K/V row scatter into [num_blocks, block_size, H, D] caches.
  * ------------------------------------------------------------------------ */
@@ -210,6 +228,8 @@ int aps_paged_decode_attention(
  *   hidden_holder_upd[b]     row of sequence b's newest token; hidden_holder_pull = the rest
  *   hidden_cache_use_input   batch positions of hidden sequences
  *   hidden_cache_store_tot   their newest rows
+ *   holder_src[row]          (nullable, not in the reference) resolved source of the row for
+ *                            aps_gather_hidden_rows: slot, -(b+1) for the newest row, INT64_MIN for padding
  *   block_tables_out[b,:]    shared table for hidden sequences, private otherwise (:415-418)
  *   seq_start_loc / query_start_loc int32 cumulative sums with leading 0;
  *   context_lens = seq_len-1; input_positions = seq_len-1. */
@@ -221,7 +241,8 @@ int aps_build_decode_metadata(
     int64_t* slot_mapping_shared, int64_t* hidden_cache_use_tot,
     int64_t* kv_cache_use_tot, int64_t* hidden_cache_use_input,
     int64_t* hidden_cache_store_tot, int64_t* hidden_holder_upd,
-    int64_t* hidden_holder_pull, int64_t cap_rows, int64_t cap_hidden_rows,
+    int64_t* hidden_holder_pull, int64_t* holder_src, int64_t cap_rows,
+    int64_t cap_hidden_rows,
     int64_t cap_hidden_seqs, int64_t cap_kv_seqs, int32_t* block_tables_out,
     int64_t out_stride, int64_t out_width, int32_t* seq_start_loc,
     int32_t* query_start_loc, int32_t* context_lens, int64_t* input_positions,

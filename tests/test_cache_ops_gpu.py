@@ -163,6 +163,46 @@ def test_hybrid_decode_gather_zero_fills_padding_rows(dev):
     assert holder[1].abs().sum() == 0
 
 
+@pytest.mark.parametrize("seed,frac", [(0, 0.5), (1, 0.3), (2, 1.0), (3, 0.0)])
+@pytest.mark.parametrize("H,D", [(2, 4), (12, 64), (40, 128)])
+def test_resolved_gather_equals_reference_sequence(dev, seed, frac, H, D):
+    """gather_hidden_rows driven by the metadata builder's holder_src."""
+    from aptserve_hip import metadata
+    N, BS = 64, 16
+    b = workloads.small_decode_batch(seed, 9, 90, frac, N)
+    md = oracle_metadata(b)
+    gmd = metadata.build_from_batch(b, dev)
+    B, T, Hd = len(b.seq_lens), md["num_tot_tokens"], H * D
+    hs = randn((B, Hd), seed)
+    cache = sentinel_cache((2, N, BS, H, D))
+    ref = cache.clone()
+    sm = t64(md["slot_mapping"])
+    O.hidden_to_cache(hs, ref, sm, t64(md["hidden_cache_use_input"]), t64(md["hidden_cache_store_tot"]))
+    holder_ref = O.assemble_hidden_holder(hs, ref, sm, T, t64(md["hidden_holder_upd"]),
+                                          t64(md["hidden_cache_use_tot"]))
+    g = cache.to(dev)
+    holder = sentinel_cache((T, Hd), seed=5).to(dev)
+    ops.gather_hidden_rows(holder, hs.to(dev), g, gmd.holder_src, gmd.slot_mapping, gmd.hidden_cache_use_input,
+                           gmd.hidden_cache_store_tot)
+    assert bits_equal(holder, holder_ref)
+    assert bits_equal(g, ref)
+
+
+def test_resolved_gather_zero_fills_padding_rows(dev):
+    H, D, N, BS = 1, 8, 4, 16
+    sm = t64([4, -1, 6, 40], dev)
+    src = t64([4, -(1 << 63), -1, -2], dev)
+    hs = randn((2, 8), 0)
+    cache = sentinel_cache((2, N, BS, H, D))
+    g = cache.to(dev)
+    holder = sentinel_cache((4, 8), seed=5).to(dev)
+    ops.gather_hidden_rows(holder, hs.to(dev), g, src, sm, t64([0], dev), t64([2], dev))
+    h = holder.cpu()
+    assert torch.equal(h[0], cache.view(-1, 8)[4]) and h[1].abs().sum() == 0
+    assert torch.equal(h[2], hs[0]) and torch.equal(h[3], hs[1])
+    assert torch.equal(g.cpu().view(-1, 8)[6], hs[0])
+
+
 # ---------------------------------------------------------------- K/V writes
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
@@ -306,7 +346,13 @@ def test_config2_write_and_gather_opt13b_full_size(dev):
                              idx(md, "hidden_holder_pull", dev), idx(md, "hidden_cache_use_input", dev),
                              idx(md, "hidden_cache_store_tot", dev))
     assert torch.equal(holder2, holder)
-    del holder2, holder
+    from aptserve_hip import metadata
+    gmd = metadata.build_from_batch(b, dev)
+    holder3 = torch.empty(T, Hd, dtype=torch.float16, device=dev)
+    ops.gather_hidden_rows(holder3, dhs, g2, gmd.holder_src, gmd.slot_mapping, gmd.hidden_cache_use_input,
+                           gmd.hidden_cache_store_tot)
+    assert torch.equal(holder3, holder)
+    del holder2, holder, holder3
     assert torch.equal(g2, g)
     del g2
     # checksum of the whole cache instead of shipping 4 GB back
