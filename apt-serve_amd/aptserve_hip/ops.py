@@ -377,3 +377,48 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, block_table=None, cache_seqlens
     _need(block_table is not None and cache_seqlens is not None, "a paged cache needs block_table and cache_seqlens")
     o = paged_decode_attention(q[:, 0], k_cache, v_cache, block_table, cache_seqlens, softmax_scale, **kw)
     return o.unsqueeze(1)
+
+
+# --------------------------------------------------------------------- a5 / a6
+
+def linear_nt(x, weight, bias=None, out=None, out_row_map=None):
+    """``out = x @ weight.T + bias`` on the matrix cores (f16/bf16, fp32 accumulation).
+
+    ``x [M, K]`` and ``weight [N, K]`` may be row-strided views (a row slice of the fused
+    QKV weight, a ``chunk`` of activations); ``N % 256 == 0`` and ``K % 64 == 0``.
+    ``out_row_map`` (int64 ``[M]``) scatters result row ``m`` to ``out[out_row_map[m]]``.
+    """
+    dev = x.device
+    _check_data("x", x, dev)
+    _check_data("weight", weight, dev)
+    _need(x.dim() == 2 and weight.dim() == 2 and x.size(1) == weight.size(1), "x [M,K] and weight [N,K] expected")
+    _need(x.dtype == weight.dtype and x.dtype in (torch.float16, torch.bfloat16), "f16 or bf16 operands expected")
+    M, K = x.shape
+    N = weight.size(0)
+    if bias is not None:
+        _check_data("bias", bias, dev)
+        _need(bias.dim() == 1 and bias.numel() == N and bias.dtype == x.dtype and bias.is_contiguous(),
+              "bias must be a contiguous [N] vector of the operand dtype")
+    if out is None:
+        _need(out_row_map is None, "a row map needs a destination")
+        out = torch.empty(M, N, dtype=x.dtype, device=dev)
+    _check_data("out", out, dev)
+    _need(out.dim() == 2 and out.size(1) >= N and out.dtype == x.dtype, "out must be [rows, >=N] of the operand dtype")
+    if out_row_map is not None:
+        _check_index("out_row_map", out_row_map, dev)
+        _need(out_row_map.numel() == M, "one destination row per input row expected")
+    else:
+        _need(out.size(0) >= M, "out has fewer rows than x")
+    with torch.cuda.device(dev):
+        st = _lib.load().aps_linear_nt(
+            x.data_ptr() if M else None, weight.data_ptr(), None if bias is None else bias.data_ptr(),
+            out.data_ptr() if out.numel() else None, M, N, K, x.stride(0), weight.stride(0), out.stride(0),
+            None if out_row_map is None else _ptr(out_row_map), out.size(0), _DTYPE_CODE[x.dtype], _stream(x))
+    _lib.check(st, "linear_nt")
+    return out
+
+
+def kv_reproject(x, w_kv, b_kv=None, out=None):
+    """K/V re-projection of gathered hidden rows: ``[T,Hd] x w_kv[2Hd,Hd]^T + b_kv -> [T,2Hd]``
+    (``k, v = out.chunk(2, -1)``), additional_designs/model_executor/models/aptserve_opt.py:123-124."""
+    return linear_nt(x, w_kv, b_kv, out=out)

@@ -263,6 +263,26 @@ int aps_build_prefill_metadata(
     int32_t* seq_start_loc, int32_t* query_start_loc, int32_t* context_lens,
     int64_t* totals, aps_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * q-only / kv-only projection on the matrix cores.
+ * ref: model_executor/layers/aptserve_linear.py:102-132 (UnquantizedLinearMethod
+ * .apply with q_only / kv_only = F.linear on a row slice of the fused QKV
+ * weight), called at model_executor/models/aptserve_opt.py:116 and :123-124.
+ *   out[m, n] = sum_k x[m, k] * weight[n, k] + bias[n]
+ * x [m, k] and weight [n, k] are K-contiguous with row strides x_stride /
+ * w_stride (pass weight + slice*w_stride for a row slice); bias nullable;
+ * f16 or bf16 operands, fp32 accumulation, result rounded once to the operand
+ * dtype.  n must be a multiple of 256 and k of 64.
+ * out_row_map (nullable): row m is stored at row out_row_map[m] of out (rows of
+ * out_stride elements; negative or >= out_rows: skipped) — the epilogue that
+ * writes re-projected K/V rows straight into [blocks, BS, H, D] tiles by slot.
+ * ------------------------------------------------------------------------ */
+int aps_linear_nt(const void* x, const void* weight, const void* bias,
+                  void* out, int64_t m, int64_t n, int64_t k, int64_t x_stride,
+                  int64_t w_stride, int64_t out_stride,
+                  const int64_t* out_row_map, int64_t out_rows, int dtype,
+                  aps_stream_t stream);
+
 /* Plain device copy of nbytes (16-byte aligned pointers): the known-size
  * kernel that hardware counters of the kernels above are scaled against. */
 int aps_copy_bytes(void* dst, const void* src, int64_t nbytes,

@@ -1,0 +1,125 @@
+"""MFMA q-only / kv-only projection against the oracle (exact fp32 product of the
+fp16-rounded operands, rounded once).
+
+Tolerances: 1e-3 relative on the fp32-accumulated value is the stated bar; the
+kernel rounds its fp32 accumulator once to fp16, so against the oracle's fp16
+result an element may differ by one fp16 ulp (2^-10 relative) plus the
+accumulation-order noise — checked as |d| <= 1e-3*|ref| + 2e-3 and, for the
+stated absolute bar of an fp16 output, |d| <= 2e-2.
+"""
+import numpy as np
+import pytest
+import torch
+
+from aptserve_hip import layers, ops
+from oracle import reproject as OR
+from util import randn
+
+pytestmark = pytest.mark.gpu
+
+
+def check(out, ref32, dtype=torch.float16):
+    out = out.float().cpu()
+    d = (out - ref32).abs()
+    assert d.max().item() <= 2e-2, f"max abs error {d.max().item()}"
+    ulp = 2 ** -10 if dtype == torch.float16 else 2 ** -7
+    bound = (1e-3 + ulp) * ref32.abs() + 2e-3
+    bad = (d > bound).sum().item()
+    assert bad == 0, f"{bad} elements outside tolerance, worst {d.max().item()}"
+
+
+@pytest.mark.parametrize("M", [1, 7, 255, 256, 257, 700])
+@pytest.mark.parametrize("N,K", [(256, 64), (512, 192), (1536, 768)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_linear_nt_small(dev, M, N, K, dtype):
+    x = randn((M, K), M, dtype)
+    w = (randn((N, K), N) * 0.05).to(dtype)
+    b = randn((N,), 3, dtype)
+    ref = OR._linear_fp32(x, w, b)
+    out = ops.linear_nt(x.to(dev), w.to(dev), b.to(dev))
+    check(out, ref, dtype)
+    out2 = ops.linear_nt(x.to(dev), w.to(dev), None)
+    check(out2, OR._linear_fp32(x, w, None), dtype)
+
+
+def test_identity_and_one_hot_weights_are_exact(dev):
+    """W = I reproduces x bit for bit; a one-hot row picks one input column."""
+    K = N = 256
+    x = randn((300, K), 0)
+    w = torch.eye(N, K, dtype=torch.float16)
+    out = ops.linear_nt(x.to(dev), w.to(dev)).cpu()
+    assert torch.equal(out, x)
+    w2 = torch.zeros(N, K, dtype=torch.float16); w2[:, 17] = 1
+    out = ops.linear_nt(x.to(dev), w2.to(dev)).cpu()
+    assert torch.equal(out, x[:, 17:18].expand(300, N))
+
+
+def test_qkv_proj_q_only_and_kv_only_on_weight_slices(dev):
+    """The reference slices the fused weight in place (aptserve_linear.py:115-130);
+    the kernel reads the row slice through its stride, no copy."""
+    Hd, T = 768, 130
+    w = (randn((3 * Hd, Hd), 1) * 0.03).half()
+    b = randn((3 * Hd,), 2)
+    x = randn((T, Hd), 3)
+    proj = layers.QKVLinear(w.to(dev), b.to(dev))
+    q, none = proj(x.to(dev), q_only=True)
+    assert none is None
+    check(q, OR.q_only(x, w, b, keep_fp32=True))
+    kv, _ = proj(x.to(dev), kv_only=True)
+    check(kv, OR.kv_only(x, w, b, keep_fp32=True))
+    k, v = kv.chunk(2, dim=-1)
+    kr, vr = OR.kv_reproject(x, w[Hd:], b[Hd:], keep_fp32=True)
+    check(k, kr); check(v, vr)
+    full, _ = proj(x.to(dev))
+    check(full, OR._linear_fp32(x, w, b))
+    with pytest.raises(NotImplementedError):
+        proj(x.to(dev), q_only=True, kv_only=True)
+
+
+def test_strided_activations_and_row_scatter_epilogue(dev):
+    K, N, M = 128, 256, 77
+    wide = randn((M, 3 * K), 0)
+    x = wide[:, K:2 * K]
+    w = (randn((N, K), 1) * 0.1).half()
+    ref = OR._linear_fp32(x, w, None)
+    out = ops.linear_nt(wide.to(dev)[:, K:2 * K], w.to(dev))
+    check(out, ref)
+    # scatter: row m -> dest[perm[m]], rows mapped to -1 are dropped, untouched rows keep their content
+    rng = np.random.default_rng(0)
+    rows = 200
+    perm = torch.from_numpy(rng.permutation(rows)[:M].astype(np.int64)); perm[5] = -1
+    dest = torch.full((rows, N), 7.0, dtype=torch.float16, device=dev)
+    ops.linear_nt(wide.to(dev)[:, K:2 * K], w.to(dev), out=dest, out_row_map=perm.to(dev))
+    dest = dest.cpu()
+    keep = perm >= 0
+    check(dest[perm[keep]], ref[keep])
+    untouched = torch.ones(rows, dtype=torch.bool); untouched[perm[keep]] = False
+    assert (dest[untouched] == 7).all()
+
+
+def test_unsupported_shapes_raise(dev):
+    x = torch.zeros(4, 64, dtype=torch.float16, device=dev)
+    with pytest.raises(RuntimeError):
+        ops.linear_nt(x, torch.zeros(100, 64, dtype=torch.float16, device=dev))     # N not a multiple of 256
+    with pytest.raises(RuntimeError):
+        ops.linear_nt(torch.zeros(4, 40, dtype=torch.float16, device=dev),
+                      torch.zeros(256, 40, dtype=torch.float16, device=dev))        # K not a multiple of 64
+    with pytest.raises(ValueError):
+        ops.linear_nt(x.float(), torch.zeros(256, 64, device=dev))
+
+
+def test_config3_kv_reprojection_opt13b(dev):
+    """[T,5120] x W_kv[10240,5120]^T, W ~ N(0,0.02), X ~ N(0,1).  T=4096 against the full
+    oracle product; T=16384 on 384 sampled rows (every row is an independent product)."""
+    Hd = 5120
+    w = (randn((2 * Hd, Hd), 1, torch.float32) * 0.02).half()
+    b = randn((2 * Hd,), 2)
+    dw, db = w.to(dev), b.to(dev)
+    x = randn((4096, Hd), 3)
+    out = ops.kv_reproject(x.to(dev), dw, db)
+    torch.set_num_threads(16)
+    check(out, OR._linear_fp32(x, w, b))
+    x2 = randn((16384, Hd), 4)
+    out2 = ops.kv_reproject(x2.to(dev), dw, db)
+    rows = torch.from_numpy(np.random.default_rng(0).choice(16384, 384, replace=False))
+    check(out2[rows.to(dev)], OR._linear_fp32(x2[rows], w, b))
