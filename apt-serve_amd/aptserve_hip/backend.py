@@ -1,0 +1,203 @@
+"""Attention backend and decoder-attention orchestration over the hybrid cache.
+
+Host-side mirrors of the reference classes on the hot path:
+
+* ``HybridCacheBackend``   <- ``FlashAttentionBackend``
+  (additional_designs/attention/backends/aptserve_flash_attn.py:15-65)
+* ``allocate_caches``      <- ``CacheEngine._allocate_kv_cache``
+  (additional_designs/worker/aptserve_cache_engine.py:61-86)
+* ``HybridAttentionImpl``  <- ``FlashAttentionImpl.forward`` (``aptserve_flash_attn.py:290-478``)
+* ``HybridOPTAttention``   <- ``OPTAttention.forward``
+  (additional_designs/model_executor/models/aptserve_opt.py:99-134)
+
+Two data flows are offered for a decode batch that mixes cache types:
+
+``literal=True`` replays the reference's operator sequence: ``mixed_kv_to_cache`` with the
+mirror range, then one attention call over the shared cache for every sequence.  In the
+reference the mirror region (shared blocks ``0..N-1``) only ever receives the newest token
+of the current layer, so K/V-cached sequences of a mixed batch attend over stale history;
+that is kept only so the two flows can be compared where they must agree (all-hidden and
+no-hidden batches).
+
+``literal=False`` (default) removes the mirror: K/V-cached sequences read their private
+cache, hidden-cached sequences read the re-projected K/V in the shared workspace, selected
+per block inside one attention launch.
+"""
+
+from __future__ import annotations
+
+from typing import Callable, List, Optional, Tuple
+
+import torch
+
+from . import ops
+from .layers import QKVLinear
+from .metadata import HybridAttentionMetadata
+
+
+class HybridCacheBackend:
+    @staticmethod
+    def get_supported_head_sizes() -> List[int]:
+        return [32, 64, 128, 256]
+
+    @staticmethod
+    def get_name() -> str:
+        return "hybrid-cache-hip"
+
+    @staticmethod
+    def get_impl_cls():
+        return HybridAttentionImpl
+
+    @staticmethod
+    def make_metadata(*args, **kwargs) -> HybridAttentionMetadata:
+        return HybridAttentionMetadata(*args, **kwargs)
+
+    @staticmethod
+    def get_kv_cache_shape(num_blocks: int, block_size: int, num_kv_heads: int, head_size: int) -> Tuple[int, ...]:
+        if block_size % 16 != 0:
+            raise ValueError("Block size must be a multiple of 16.")
+        return (2, num_blocks, block_size, num_kv_heads, head_size)
+
+
+def allocate_caches(num_layers: int, num_blocks: int, block_size: int, num_kv_heads: int, head_size: int,
+                    dtype: torch.dtype, device) -> Tuple[List[torch.Tensor], torch.Tensor]:
+    """One zeroed ``(2, N, BS, H, D)`` cache per layer and ONE ``(2, 2N, BS, H, D)`` shared
+    cache for all layers (blocks ``N..2N-1`` are the per-step K/V workspace)."""
+    shape = HybridCacheBackend.get_kv_cache_shape(num_blocks, block_size, num_kv_heads, head_size)
+    kv = [torch.zeros(shape, dtype=dtype, device=device) for _ in range(num_layers)]
+    shared = torch.zeros((shape[0], 2 * shape[1]) + shape[2:], dtype=dtype, device=device)
+    return kv, shared
+
+
+class HybridAttentionImpl:
+    def __init__(self, num_heads: int, head_size: int, scale: float, num_kv_heads: Optional[int] = None,
+                 alibi_slopes=None, sliding_window=None, kv_cache_dtype: str = "auto", *, literal: bool = False,
+                 prefill_attention: Optional[Callable] = None) -> None:
+        if alibi_slopes is not None:
+            raise ValueError("alibi_slopes is not supported (OPT has none)")
+        if sliding_window is not None:
+            raise ValueError("Sliding window is not supported.")     # aptserve_flash_attn.py:277-282
+        if num_kv_heads not in (None, num_heads):
+            raise ValueError("grouped-query attention is outside the OPT path")
+        if head_size not in HybridCacheBackend.get_supported_head_sizes():
+            raise ValueError(f"Head size {head_size} is not supported. "
+                             f"Supported head sizes are: {HybridCacheBackend.get_supported_head_sizes()}.")
+        self.num_heads, self.head_size, self.scale = num_heads, head_size, float(scale)
+        self.num_kv_heads = num_heads
+        self.kv_cache_dtype = kv_cache_dtype
+        self.literal = literal
+        self.prefill_attention = prefill_attention
+
+    def forward(self, query, key, value, kv_cache, shared_cache, attn_metadata: HybridAttentionMetadata,
+                kv_scale: float = 1.0) -> torch.Tensor:
+        """``query [tokens, H*D]``, ``key``/``value [rows, H*D]`` (rows = tokens, or the 'tot' rows of a
+        decode batch with hidden-cached sequences) -> ``[tokens, H*D]``."""
+        assert kv_scale == 1.0, "kv_scale is not supported"            # :312
+        md = attn_metadata
+        num_tokens, hidden_size = query.shape
+        H, D = self.num_heads, self.head_size
+        query = query.view(-1, H, D)
+        key = key.view(-1, H, D)
+        value = value.view(-1, H, D)
+        n_hidden, n_prefill, n_decode = md.num_hidden_cache_tokens, md.num_prefill_tokens, md.num_decode_tokens
+        if n_hidden == 0:
+            assert key.shape[0] == n_prefill + n_decode and value.shape[0] == n_prefill + n_decode
+
+        mixed = False
+        if kv_cache is not None:
+            key_cache, value_cache = kv_cache[0], kv_cache[1]
+            if n_hidden == 0:                                                       # :334-345
+                ops.reshape_and_cache_flash(key, value, key_cache, value_cache, md.slot_mapping,
+                                            self.kv_cache_dtype)
+            elif n_prefill != 0:                                                    # :347-355, without the gather copies
+                ops.reshape_and_cache_flash(key, value, key_cache, value_cache, md.slot_mapping,
+                                            self.kv_cache_dtype, token_idx=md.kv_cache_use_tot)
+            else:
+                shared_k, shared_v = shared_cache[0], shared_cache[1]
+                mixed = md.num_tot_tokens != md.slot_mapping_shared.numel()         # :359
+                if mixed:
+                    ops.mixed_kv_to_cache(key, value, key_cache, value_cache, shared_k, shared_v, md.slot_mapping,
+                                          md.slot_mapping_shared, md.kv_cache_use_tot, md.hidden_cache_use_tot,
+                                          skip_mirror=not self.literal)
+                else:                                                               # :376-385
+                    ops.reshape_and_cache_flash(key, value, shared_k, shared_v, md.slot_mapping_shared,
+                                                self.kv_cache_dtype)
+
+        output = torch.empty_like(query)
+        decode_query = query[n_prefill:]
+        if md.prefill_metadata is not None:
+            pm = md.prefill_metadata
+            if self.prefill_attention is None:
+                raise NotImplementedError(
+                    "prompt attention (flash_attn_varlen_func, aptserve_flash_attn.py:405-447) is not part of "
+                    "this library: pass prefill_attention=callable(q, k, v, cu_seqlens, max_seqlen, scale)")
+            output[:n_prefill] = self.prefill_attention(query[:n_prefill], key[:n_prefill], value[:n_prefill],
+                                                        pm.seq_start_loc, pm.max_prefill_seq_len, self.scale)
+        if md.decode_metadata is not None:
+            dm = md.decode_metadata
+            max_len = dm.max_decode_seq_len or None
+            if n_hidden == 0:                                                       # :451-461
+                ops.paged_decode_attention(decode_query, key_cache, value_cache, dm.block_tables,
+                                           dm.seq_lens_tensor, self.scale, max_seq_len=max_len,
+                                           out=output[n_prefill:])
+            elif self.literal or not mixed:                                         # :464-473
+                ops.paged_decode_attention(decode_query, shared_k, shared_v, dm.block_tables, dm.seq_lens_tensor,
+                                           self.scale, max_seq_len=max_len, out=output[n_prefill:])
+            else:
+                ops.paged_decode_attention(decode_query, key_cache, value_cache, dm.block_tables,
+                                           dm.seq_lens_tensor, self.scale, block_types=dm.block_types,
+                                           ws_k_cache=shared_k, ws_v_cache=shared_v, max_seq_len=max_len,
+                                           out=output[n_prefill:])
+        return output.view(num_tokens, hidden_size)
+
+
+class HybridOPTAttention:
+    """Self-attention of one OPT decoder layer over the hybrid cache.
+
+    ``fused=False`` issues the reference's operator sequence (``hidden_to_cache``,
+    ``torch.zeros`` holder, index_put, ``cache_to_hidden``); ``fused=True`` replaces it by
+    one ``gather_hidden_rows`` launch into an uninitialised holder.  Results are identical.
+    """
+
+    def __init__(self, embed_dim: int, num_heads: int, qkv_weight, qkv_bias, out_weight, out_bias, *,
+                 fused: bool = True, literal: bool = False, prefill_attention: Optional[Callable] = None) -> None:
+        self.embed_dim, self.num_heads = embed_dim, num_heads
+        self.head_dim = embed_dim // num_heads
+        self.scaling = self.head_dim ** -0.5
+        self.qkv_proj = QKVLinear(qkv_weight, qkv_bias)
+        self.out_weight, self.out_bias = out_weight, out_bias
+        self.fused = fused
+        self.attn = HybridAttentionImpl(num_heads, self.head_dim, self.scaling, literal=literal,
+                                        prefill_attention=prefill_attention)
+
+    def forward(self, hidden_states, kv_cache, shared_cache, attn_metadata: HybridAttentionMetadata):
+        md = attn_metadata
+        if md.num_hidden_cache_tokens != 0:
+            if md.num_decode_tokens != 0:
+                if self.fused and md.holder_src is not None:
+                    holder = torch.empty(md.num_tot_tokens, hidden_states.shape[1], device=hidden_states.device,
+                                         dtype=hidden_states.dtype)
+                    ops.gather_hidden_rows(holder, hidden_states, kv_cache, md.holder_src, md.slot_mapping,
+                                           md.hidden_cache_use_input, md.hidden_cache_store_tot)
+                else:                                                               # aptserve_opt.py:108-121
+                    ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
+                                        md.hidden_cache_store_tot)
+                    holder = torch.zeros(md.num_tot_tokens, hidden_states.shape[1], device=hidden_states.device,
+                                         dtype=hidden_states.dtype)
+                    holder[md.hidden_holder_upd] = hidden_states
+                    ops.cache_to_hidden(holder, kv_cache, md.slot_mapping, md.hidden_cache_use_tot)
+                q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
+                kv, _ = self.qkv_proj(holder, q_only=False, kv_only=True)
+                k, v = kv.chunk(chunks=2, dim=-1)
+            else:                                                                   # :125-127
+                ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
+                                    md.hidden_cache_store_tot)
+                qkv, _ = self.qkv_proj(hidden_states)
+                q, k, v = qkv.chunk(chunks=3, dim=-1)
+        else:                                                                       # :128-130
+            qkv, _ = self.qkv_proj(hidden_states)
+            q, k, v = qkv.chunk(chunks=3, dim=-1)
+        attn_output = self.attn.forward(q, k, v, kv_cache, shared_cache, md)
+        return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
+
+    __call__ = forward

@@ -26,6 +26,10 @@ kv_reproject / q_only   float64 numpy matmul; identity / one-hot weights
 paged decode attention  float64 textbook softmax on dense K/V; L=1; equal
                         keys -> mean of V; block permutation invariance;
                         all-K/V vs all-hidden equivalence
+layer.opt_attention     composition of the functions above; all-hidden vs
+                        all-K/V caches built from the same hidden states agree;
+                        decode after prefill equals the last row of a longer
+                        prefill
 build_metadata          the invariants the reference's own commented checks
                         list; brute force from an independent per-row
                         definition on tiny batches
@@ -38,4 +42,4 @@ their outputs are covered by the stated tolerances instead (1e-3 relative with
 fp32 accumulation, 2e-2 absolute for fp16 outputs).
 """
 
-from . import cache_ops, fp8, reproject, attention, metadata  # noqa: F401
+from . import cache_ops, fp8, reproject, attention, metadata, layer  # noqa: F401
