@@ -23,6 +23,9 @@ for p in (ROOT, ROOT / "apt-serve_amd"):
         sys.path.insert(0, str(p))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (seed 0 workloads), scaled by what the
+# same counters read for the 1 GiB copy kernel (x2.000 and x1.000); summary in profiles/bench_step_hbm_counters.txt
+PMC_TRAFFIC_BYTES = {"gather": 1804.9e6, "attention_f16": 1800.4e6, "attention_fp8": 905.3e6}
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 
 
@@ -34,6 +37,8 @@ def parse():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip attention / re-projection figures")
+    ap.add_argument("--pmc-calibrate", action="store_true",
+                    help="first run the plain copy kernel on 1 GiB three times (known traffic for counter scaling)")
     return ap.parse_args()
 
 
@@ -94,7 +99,8 @@ def attention_figures(torch, ops, workloads, np, dev, seed, fp8):
                         (total, "fp8-e4m3" if fp8 else "fp16"),
             "tokens_per_s": B / (ms * 1e-3), "ms": ms, "algorithmic_bytes": nbytes,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
+                         "frac": gbs / HBM_PEAK_GBS,
+                         "traffic": PMC_TRAFFIC_BYTES["attention_fp8" if fp8 else "attention_f16"] if seed == 0 else None}}
 
 
 def main():
@@ -152,6 +158,14 @@ def main():
             b.record()
             gather_events.append((a, b))
 
+    if args.pmc_calibrate:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            ops.copy_bytes(dst, src)
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -178,7 +192,9 @@ def main():
                    "step_bytes": step_bytes, "write_bytes": write_bytes, "gather_bytes": gather_bytes,
                    "launches_per_step": 2},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "row_mover<16,ResolvedGatherOp>",
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": PMC_TRAFFIC_BYTES["gather"] if args.seed == 0 else None,
+                     "kernel": "row_mover<16,ResolvedGatherOp>",
                      "algorithmic_bytes_per_launch": gather_alg, "avg_launch_ms": gather_ms},
     }
 
