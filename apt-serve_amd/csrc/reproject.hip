@@ -7,15 +7,25 @@
 // Tiling: one 256-thread workgroup (4 wavefronts, 2 x 2) owns a 256 x 256 tile
 // of C; each wavefront owns 128 x 128 = 4 x 4 MFMA 32x32x16 tiles (256 fp32
 // accumulator registers per lane).  The K loop moves BK = 64 at a time through
-// a two-stage LDS ring (2 x (32 + 32) KiB of the 160 KiB per CU): tile t+1 is
+// a two-stage LDS ring (2 x (32 + 32) KiB of the 160 KiB per CU; 136 KiB with the epilogue images): tile t+1 is
 // copied global -> LDS by buffer_load ... lds (no VGPR round trip) while the
 // matrix cores consume tile t.
 //
 // LDS layout: a tile is [256 rows][8 chunks of 16 B]; chunk c of row r lives at
-// position c ^ (r % 8), so that the 128-bit fragment reads of 8 consecutive rows
-// touch 8 different 16-byte bank groups.  The DMA writes 1 KiB per wavefront in
-// lane order, so the swizzle is applied on the global side: lane l of a
-// wave-wide load fetches chunk (l%8) ^ (l/8) of row l/8.
+// position c ^ ((r >> 1) % 8).  The LDS of gfx950 serves a 128-bit read to 16
+// lanes per cycle over 64 banks, so the 16 consecutive rows those lanes read
+// (2 rows x 8 chunks per 256 B of banks) must all land in different 16-byte
+// bank groups; with an 8-row swizzle half of all LDS cycles were conflicts
+// (SQ_LDS_BANK_CONFLICT).  The DMA writes 1 KiB per wavefront in lane order,
+// so the swizzle is applied on the global side: lane l of a wave-wide load
+// fetches chunk (l%8) ^ ((row>>1)%8) of row l/8 of its 8-row group.
+//
+// Schedule: fragments live in two register sets; while the matrix cores work
+// on k-step s the 8 ds_read_b128 of k-step s+1 are in flight (2 MFMA : 1 read).
+// Before the last k-step of a tile every wave has its fragments in registers,
+// so after one barrier the stage can be refilled with tile t+2 while the last
+// k-step runs and the first fragments of tile t+1 stream in.  Waits and the
+// barrier are written as asm so that no fence forces all DMA traffic to drain.
 //
 // Workgroups are renumbered so that the 32 workgroups an XCD runs together
 // form an 8 x 4 block of tiles and share their A and W panels in that XCD's L2.
@@ -34,7 +44,9 @@ constexpr int kThreads = 256;
 constexpr int kTileBytes = BM * BK * 2;          // 32 KiB, same for A and W tiles
 constexpr int kStageBytes = 2 * kTileBytes;      // A + W
 constexpr int kStages = 2;
-constexpr int kLdsBytes = kStages * kStageBytes;  // 128 KiB
+constexpr int kEpiPitch = 128 * 2 + 16;           // bytes per row of a wave's epilogue image
+constexpr int kEpiWaveBytes = 128 * kEpiPitch;    // 34 KiB
+constexpr int kLdsBytes = 4 * kEpiWaveBytes > kStages * kStageBytes ? 4 * kEpiWaveBytes : kStages * kStageBytes;
 constexpr int kNumXcd = 8;
 constexpr int kGroupM = 8;
 
@@ -46,6 +58,7 @@ struct GemmArgs {
   // optional row scatter of the epilogue: row t of C goes to row_map[t] (rows of ldc elements), <0 skipped
   const int64_t* row_map;
   int64_t row_map_limit;
+  int c_aligned16;  // out pointer and row pitch allow 128-bit stores
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
@@ -71,8 +84,14 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
   return (uint16_t)(u >> 16);
 }
 
+// Hand-placed wait points: a __syncthreads() would add fences that wait for every outstanding DMA load.
+#define APS_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
+#define APS_WAIT_LGKM0() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
+#define APS_BARRIER() asm volatile("s_barrier" ::: "memory")
+
 template <bool BF16>
-__global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const GemmArgs g) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_nt_kernel(
+    const GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -99,23 +118,25 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const GemmArgs g) 
   const int64_t row0 = (int64_t)pid_m * BM, col0 = (int64_t)pid_n * BN;
   const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(g.a + row0 * g.lda_b, (g.m - row0) * g.lda_b);
   const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(g.w + col0 * g.ldw_b, (g.n - col0) * g.ldw_b);
-  const int lrow = lane >> 3;                       // row within the 8-row group of a wave-wide load
-  const int lchunk = (lane & 7) ^ lrow;             // swizzled 16-byte chunk this lane fetches
-  const uint32_t voff_a = (uint32_t)(lrow * g.lda_b + lchunk * 16);
-  const uint32_t voff_w = (uint32_t)(lrow * g.ldw_b + lchunk * 16);
+  const int lrow = lane >> 3;  // row within the 8-row group of a wave-wide load
+  // (row >> 1) % 8 of row 8*i + lane/8 is 4*(i&1) + lane/16: two swizzles, for even and odd groups
+  const int lchunk0 = (lane & 7) ^ ((lane >> 4) & 7);
+  const int lchunk1 = (lane & 7) ^ ((4 + (lane >> 4)) & 7);
+  const uint32_t voff_a0 = (uint32_t)(lrow * g.lda_b + lchunk0 * 16), voff_a1 = (uint32_t)(lrow * g.lda_b + lchunk1 * 16);
+  const uint32_t voff_w0 = (uint32_t)(lrow * g.ldw_b + lchunk0 * 16), voff_w1 = (uint32_t)(lrow * g.ldw_b + lchunk1 * 16);
   const uint32_t grp_a = (uint32_t)(8 * g.lda_b), grp_w = (uint32_t)(8 * g.ldw_b);
 
-  auto issue_loads = [&](int kt, int stage) {
-    char* sa = lds + stage * kStageBytes;
+  auto issue_loads = [&](int kt) {
+    char* sa = lds + (kt & 1) * kStageBytes;
     char* sw = sa + kTileBytes;
     const uint32_t koff = (uint32_t)kt * (BK * 2);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int i = wave * 8 + j;  // 8-row group of the tile handled by this wave-wide load
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(sa + i * 1024), 16,
-                                               voff_a, koff + i * grp_a, 0, 0);
+                                               (j & 1) ? voff_a1 : voff_a0, koff + i * grp_a, 0, 0);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (__attribute__((address_space(3))) void*)(sw + i * 1024), 16,
-                                               voff_w, koff + i * grp_w, 0, 0);
+                                               (j & 1) ? voff_w1 : voff_w0, koff + i * grp_w, 0, 0);
     }
   };
 
@@ -125,7 +146,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const GemmArgs g) 
   const uint32_t w_row_off = (uint32_t)((wn * 128 + frow) * (BK * 2));
   uint32_t chunk_off[4];
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) chunk_off[ks] = (uint32_t)(((2 * ks + fhalf) ^ (frow & 7)) * 16);
+  for (int ks = 0; ks < 4; ++ks) chunk_off[ks] = (uint32_t)(((2 * ks + fhalf) ^ ((frow >> 1) & 7)) * 16);
 
   float16v acc[4][4];
 #pragma unroll
@@ -135,54 +156,113 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const GemmArgs g) 
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int nk = (int)(g.k / BK);
-  issue_loads(0, 0);
-  for (int kt = 0; kt < nk; ++kt) {
-    const int stage = kt & 1;
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of tile kt has landed in LDS
-    __syncthreads();                      // everyone's part has landed; everyone is done with the other stage
-    if (kt + 1 < nk) issue_loads(kt + 1, stage ^ 1);
-    const char* sa = lds + stage * kStageBytes;
+  auto read_frags = [&](int kt, int ks, u32x4(&af)[4], u32x4(&wf)[4]) {
+    const char* sa = lds + (kt & 1) * kStageBytes;
     const char* sw = sa + kTileBytes;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      u32x4 af[4], wf[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        af[i] = *(const u32x4*)(sa + a_row_off + i * (32 * BK * 2) + chunk_off[ks]);
-        wf[i] = *(const u32x4*)(sw + w_row_off + i * (32 * BK * 2) + chunk_off[ks]);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = mfma32<BF16>(af[i], wf[j], acc[i][j]);
+    for (int i = 0; i < 4; ++i) {
+      af[i] = *(const u32x4*)(sa + a_row_off + i * (32 * BK * 2) + chunk_off[ks]);
+      wf[i] = *(const u32x4*)(sw + w_row_off + i * (32 * BK * 2) + chunk_off[ks]);
     }
+  };
+  auto mfma16 = [&](const u32x4(&af)[4], const u32x4(&wf)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = mfma32<BF16>(af[i], wf[j], acc[i][j]);
+  };
+  auto interleave = [&]() {  // scheduling hint: 2 MFMA, then 1 LDS read, eight times
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+  };
+
+  const int nk = (int)(g.k / BK);
+  u32x4 a0[4], w0[4], a1[4], w1[4];
+  issue_loads(0);
+  if (nk > 1) {
+    issue_loads(1);
+    APS_WAIT_VM(16);  // tile 0 has landed, tile 1 may still be in flight
+  } else {
+    APS_WAIT_VM(0);
+  }
+  APS_BARRIER();
+  read_frags(0, 0, a0, w0);
+  int kt = 0;
+  for (; kt + 2 < nk; ++kt) {  // steady state: a tile kt+2 exists, the body has no branches
+    read_frags(kt, 1, a1, w1); mfma16(a0, w0); interleave();
+    read_frags(kt, 2, a0, w0); mfma16(a1, w1); interleave();
+    read_frags(kt, 3, a1, w1); mfma16(a0, w0); interleave();
+    APS_WAIT_LGKM0();  // every fragment of tile kt is in registers: its stage is free
+    APS_WAIT_VM(0);    // tile kt+1 has landed (this wave's part; the barrier covers the others)
+    APS_BARRIER();
+    issue_loads(kt + 2);
+    read_frags(kt + 1, 0, a0, w0); mfma16(a1, w1); interleave();
+  }
+  for (; kt < nk; ++kt) {  // last two tiles: nothing left to issue
+    read_frags(kt, 1, a1, w1); mfma16(a0, w0); interleave();
+    read_frags(kt, 2, a0, w0); mfma16(a1, w1); interleave();
+    read_frags(kt, 3, a1, w1); mfma16(a0, w0); interleave();
+    APS_WAIT_LGKM0();
+    APS_WAIT_VM(0);
+    APS_BARRIER();
+    if (kt + 1 < nk) read_frags(kt + 1, 0, a0, w0);
+    mfma16(a1, w1);
   }
 
-  // ---- epilogue: bias, convert, store.  Lane l of a 32x32 result tile holds column l%32 and
-  // rows 8*(e/4) + 4*(l/32) + e%4, e = 0..15.
-  uint16_t* c = (uint16_t*)g.c;
+  // ---- epilogue: bias, round once, transpose through LDS, 128-bit row stores.
+  // Lane l of a 32x32 result tile holds column l%32 and rows 8*(e/4) + 4*(l/32) + e%4, e = 0..15.
+  // Each wave owns a [128 rows][128 cols] fp16 image (row pitch 272 B so that the two half-waves,
+  // four rows apart, use different banks).  Neighbouring lanes swap one value so that every lane
+  // writes a 32-bit pair; the image is then read back 16 bytes per lane, 16 lanes per row.
+  APS_WAIT_LGKM0();
+  APS_BARRIER();  // the main-loop tiles are dead; the LDS is reused for the images
+  char* img = lds + wave * kEpiWaveBytes;
+  const bool odd = lane & 1;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int64_t col = col0 + wn * 128 + j * 32 + frow;
+    const int col = j * 32 + frow;  // column inside the wave's 128-column strip
     float bv = 0.f;
     if (g.bias) {
-      const uint16_t bb = ((const uint16_t*)g.bias)[col];
+      const uint16_t bb = ((const uint16_t*)g.bias)[col0 + wn * 128 + col];
       bv = BF16 ? __uint_as_float((uint32_t)bb << 16) : (float)__builtin_bit_cast(_Float16, bb);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        int64_t row = row0 + wm * 128 + i * 32 + 8 * (e >> 2) + 4 * fhalf + (e & 3);
-        if (row >= g.m) continue;
-        if (g.row_map) {
-          row = g.row_map[row];
-          if (row < 0 || row >= g.row_map_limit) continue;
-        }
-        const float v = acc[i][j][e] + bv;
-        c[row * g.ldc + col] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+      for (int e = 0; e < 16; e += 2) {
+        const float v0 = acc[i][j][e] + bv, v1 = acc[i][j][e + 1] + bv;
+        const uint32_t h0 = BF16 ? f32_to_bf16_bits(v0) : f32_to_f16_bits(v0);
+        const uint32_t h1 = BF16 ? f32_to_bf16_bits(v1) : f32_to_f16_bits(v1);
+        // even lanes keep row e and receive the neighbour's row-e value; odd lanes keep row e+1
+        const uint32_t send = odd ? h0 : h1;
+        const uint32_t recv = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send, 0xB1, 0xf, 0xf, true);
+        const uint32_t pair = odd ? (recv | (h1 << 16)) : (h0 | (recv << 16));
+        const int row = i * 32 + 8 * (e >> 2) + 4 * fhalf + (e & 3) + (odd ? 1 : 0);
+        *(uint32_t*)(img + row * kEpiPitch + (col & ~1) * 2) = pair;
       }
+    }
+  }
+  // same wave wrote and reads: only the LDS counter has to drain
+  uint16_t* c = (uint16_t*)g.c;
+  const int rrow = lane >> 4, rchunk = lane & 15;
+#pragma unroll 4
+  for (int it = 0; it < 32; ++it) {
+    const int lr = it * 4 + rrow;
+    const u32x4 v = *(const u32x4*)(img + lr * kEpiPitch + rchunk * 16);
+    int64_t row = row0 + wm * 128 + lr;
+    if (row >= g.m) continue;
+    if (g.row_map) {
+      row = g.row_map[row];
+      if (row < 0 || row >= g.row_map_limit) continue;
+    }
+    if (g.c_aligned16)
+      *(u32x4*)(c + row * g.ldc + col0 + wn * 128 + rchunk * 8) = v;
+    else {
+      uint32_t* d = (uint32_t*)(c + row * g.ldc + col0 + wn * 128 + rchunk * 8);
+      d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
     }
   }
 }
@@ -205,6 +285,7 @@ int aps_linear_nt(const void* x, const void* weight, const void* bias, void* out
   if (x_stride < k || w_stride < k || out_stride < n) return APS_ERR_INVALID_ARG;
   if (common_vec_bytes({addr(x), addr(weight), (uint64_t)x_stride * 2, (uint64_t)w_stride * 2}) != 16)
     return APS_ERR_UNSUPPORTED;
+  if (common_vec_bytes({addr(out), (uint64_t)out_stride * 2}) < 4) return APS_ERR_UNSUPPORTED;
   // one tile's rows must be addressable with 32-bit byte offsets
   if ((int64_t)BM * x_stride * 2 >= ((int64_t)1 << 31) || (int64_t)BN * w_stride * 2 >= ((int64_t)1 << 31))
     return APS_ERR_UNSUPPORTED;
@@ -214,6 +295,7 @@ int aps_linear_nt(const void* x, const void* weight, const void* bias, void* out
   g.m = m; g.n = n; g.k = k;
   g.tiles_m = (int)((m + BM - 1) / BM); g.tiles_n = (int)(n / BN);
   g.row_map = out_row_map; g.row_map_limit = out_rows;
+  g.c_aligned16 = common_vec_bytes({addr(out), (uint64_t)out_stride * 2}) == 16;
   const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
   if (total >= ((int64_t)1 << 30)) return APS_ERR_UNSUPPORTED;
   const int64_t per_xcd = (total + kNumXcd - 1) / kNumXcd;
