@@ -128,21 +128,24 @@ struct AttnArgs {
   float v_scale;
 };
 
-template <int QT, int KV, int D>
+// HPW adjacent heads share a wavefront: the LPT lanes of head h+1 sit next to those of head h, so one
+// token contributes HPW*D contiguous elements to a wave-wide load (longer DRAM bursts per token row).
+template <int QT, int KV, int D, int HPW>
 __global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
   constexpr int EPL = Unpack<KV>::EPL;        // elements per lane
-  constexpr int LPT = D / EPL;                // lanes per token
-  constexpr int TPL = 64 / LPT;               // tokens per wave-wide load
+  constexpr int LPT = D / EPL;                // lanes per (token, head)
+  constexpr int LPR = LPT * HPW;              // lanes per token row of the wave
+  constexpr int TPL = 64 / LPR;               // tokens per wave-wide load
   constexpr int NG = kTile / TPL;             // loads per tile and per K/V
-  static_assert(LPT >= 2 && LPT <= 32 && NG >= 1, "unsupported head size");
+  static_assert(LPT >= 2 && LPR <= 32 && NG >= 1, "unsupported head size");
   constexpr int KV_ELEM_B = (KV == KV_FP8) ? 1 : 2;
 
-  const int head = blockIdx.x;
   const int part = blockIdx.y;
   const int seq = blockIdx.z;
   const int lane = threadIdx.x;
-  const int tl = lane / LPT;  // token row of this lane
-  const int dl = lane % LPT;  // 16-byte chunk of the head vector
+  const int tl = lane / LPR;                            // token row of this lane
+  const int head = blockIdx.x * HPW + (lane % LPR) / LPT;
+  const int dl = lane % LPT;                            // 16-byte chunk of the head vector
 
   const int seq_len = a.seq_lens[seq];
   const int start = part * a.partition_size;
@@ -262,7 +265,7 @@ __global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
 
   // merge the TPL token rows (lanes that share dl)
 #pragma unroll
-  for (int off = LPT; off < 64; off <<= 1) {
+  for (int off = LPR; off < 64; off <<= 1) {
     const float m_o = __shfl_xor(m, off);
     const float l_o = __shfl_xor(l, off);
     const float m_n = fmaxf(m, m_o);
@@ -327,16 +330,40 @@ __global__ __launch_bounds__(256) void combine_partitions_kernel(void* out, cons
   }
 }
 
+#ifndef APS_HPW_F16
+#define APS_HPW_F16 1
+#endif
+#ifndef APS_HPW_FP8
+#define APS_HPW_FP8 2
+#endif
+
+// Heads per wavefront: adjacent heads of one token are contiguous in memory, so HPW heads per wave make
+// the contiguous piece a wave-wide load takes from one token row HPW times longer.
+template <int QT, int KV, int D>
+void launch_head_size(const AttnArgs& a, int64_t batch, hipStream_t s) {
+  constexpr int kWant = (KV == KV_FP8) ? APS_HPW_FP8 : APS_HPW_F16;
+  constexpr int LPT = D / Unpack<KV>::EPL;
+  constexpr int HPW = (LPT * kWant <= 32) ? kWant : 1;
+  if constexpr (HPW > 1) {
+    if (a.num_heads % HPW == 0) {
+      const dim3 grid((unsigned)(a.num_heads / HPW), (unsigned)a.num_partitions, (unsigned)batch);
+      hipLaunchKernelGGL((paged_decode_kernel<QT, KV, D, HPW>), grid, dim3(64), 0, s, a);
+      return;
+    }
+  }
+  const dim3 grid((unsigned)a.num_heads, (unsigned)a.num_partitions, (unsigned)batch);
+  hipLaunchKernelGGL((paged_decode_kernel<QT, KV, D, 1>), grid, dim3(64), 0, s, a);
+}
+
 template <int QT, int KV>
 int launch_decode(const AttnArgs& a, int head_size, int64_t batch, hipStream_t s) {
-  const dim3 grid((unsigned)a.num_heads, (unsigned)a.num_partitions, (unsigned)batch);
   switch (head_size) {
-    case 64: hipLaunchKernelGGL((paged_decode_kernel<QT, KV, 64>), grid, dim3(64), 0, s, a); break;
-    case 128: hipLaunchKernelGGL((paged_decode_kernel<QT, KV, 128>), grid, dim3(64), 0, s, a); break;
-    case 256: hipLaunchKernelGGL((paged_decode_kernel<QT, KV, 256>), grid, dim3(64), 0, s, a); break;
+    case 64: launch_head_size<QT, KV, 64>(a, batch, s); break;
+    case 128: launch_head_size<QT, KV, 128>(a, batch, s); break;
+    case 256: launch_head_size<QT, KV, 256>(a, batch, s); break;
     case 32:
       if constexpr (KV == KV_FP8) return APS_ERR_UNSUPPORTED;
-      else hipLaunchKernelGGL((paged_decode_kernel<QT, KV, 32>), grid, dim3(64), 0, s, a);
+      else launch_head_size<QT, KV, 32>(a, batch, s);
       break;
     default: return APS_ERR_UNSUPPORTED;
   }
