@@ -16,6 +16,7 @@ that scales with the number of cached tokens.
 
 from __future__ import annotations
 
+import itertools
 from dataclasses import dataclass
 from typing import List, Optional, Sequence
 
@@ -142,11 +143,20 @@ def _stage(device, n: int):
     return st, i, host
 
 
-def _pack_tables(tables: Sequence[Sequence[int]], width: int, out: np.ndarray) -> None:
-    for i, t in enumerate(tables):
-        n = min(len(t), width)
-        if n:
-            out[i, :n] = t[:n]
+def _table_lens(tables: Sequence[Sequence[int]]) -> np.ndarray:
+    return np.fromiter(map(len, tables), dtype=np.int64, count=len(tables))
+
+
+def _pack_tables(tables: Sequence[Sequence[int]], lens: np.ndarray, out: np.ndarray) -> None:
+    """Ragged lists -> 0-padded ``out[B, W]`` with one flat copy instead of a Python loop per row."""
+    total = int(lens.sum())
+    if total == 0:
+        return
+    flat = np.fromiter(itertools.chain.from_iterable(tables), dtype=np.int32, count=total)
+    starts = np.cumsum(lens) - lens
+    rows = np.repeat(np.arange(len(tables)), lens)
+    cols = np.arange(total) - np.repeat(starts, lens)
+    out[rows, cols] = flat
 
 
 def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequence[bool],
@@ -171,12 +181,12 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
     if np.any(lens <= 0):
         raise ValueError("sequence lengths must be positive")
     need_blocks = -(-lens // block_size)
-    have_tables = any(len(t) for t in block_tables)
-    W = max(len(t) for t in block_tables) if have_tables else 0
-    if have_tables:
-        for b in range(B):
-            if len(block_tables[b]) < need_blocks[b]:
-                raise ValueError(f"sequence {b}: private block table shorter than ceil(seq_len/block_size)")
+    bt_lens = _table_lens(block_tables)
+    have_tables = bool(bt_lens.any())
+    W = int(bt_lens.max()) if have_tables else 0
+    if have_tables and np.any(bt_lens < need_blocks):
+        b = int(np.nonzero(bt_lens < need_blocks)[0][0])
+        raise ValueError(f"sequence {b}: private block table shorter than ceil(seq_len/block_size)")
     lib = _lib.load()
     i64 = dict(dtype=torch.int64, device=device)
     i32 = dict(dtype=torch.int32, device=device)
@@ -184,26 +194,27 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
     if not is_prompt:
         if len(block_tables_4_shared) != B:
             raise ValueError("block_tables_4_shared must have one entry per sequence")
-        for b in np.nonzero(hid)[0]:
-            if have_tables and len(block_tables_4_shared[b]) < need_blocks[b]:
-                raise ValueError(f"sequence {b}: shared block table shorter than ceil(seq_len/block_size)")
+        bts_lens = _table_lens(block_tables_4_shared) * hid      # tables of K/V-cached sequences are ignored
+        if have_tables and np.any(bts_lens[hid] < need_blocks[hid]):
+            b = int(np.nonzero(hid & (bts_lens < need_blocks))[0][0])
+            raise ValueError(f"sequence {b}: shared block table shorter than ceil(seq_len/block_size)")
         n_hs = int(hid.sum())
         n_kv = B - n_hs
         n_hr = int(lens[hid].sum())
         num_tot = n_hr + n_kv
-        Ws = max((len(block_tables_4_shared[b]) for b in np.nonzero(hid)[0]), default=0) if have_tables else 0
+        Ws = int(bts_lens.max()) if (have_tables and n_hs) else 0
         # width of the table handed to attention: the longest *selected* table (:601-609)
-        Wo = max((len(block_tables_4_shared[b]) if hid[b] else len(block_tables[b]) for b in range(B)),
-                 default=0) if have_tables else 0
+        Wo = int(np.where(hid, bts_lens, bt_lens).max()) if have_tables else 0
         # one packed upload: lens | flags | private tables | shared tables
         stg, slot, host = _stage(device, 2 * B + B * W + B * Ws)
         hv = host.numpy()
         hv[:B] = lens
         hv[B:2 * B] = hid
         if W:
-            _pack_tables(block_tables, W, hv[2 * B:2 * B + B * W].reshape(B, W))
+            _pack_tables(block_tables, bt_lens, hv[2 * B:2 * B + B * W].reshape(B, W))
         if Ws:
-            _pack_tables(block_tables_4_shared, Ws, hv[2 * B + B * W:].reshape(B, Ws))
+            shared = [t if h else () for t, h in zip(block_tables_4_shared, hid)]
+            _pack_tables(shared, bts_lens, hv[2 * B + B * W:].reshape(B, Ws))
         packed = stg.upload(slot, host, device)
         d_lens, d_hid = packed[:B], packed[B:2 * B]
         d_bt = packed[2 * B:2 * B + B * W].view(B, W)
@@ -258,7 +269,7 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
     hv[B:2 * B] = hid
     hv[2 * B:3 * B] = ctxs
     if W:
-        _pack_tables(block_tables, W, hv[3 * B:].reshape(B, W))
+        _pack_tables(block_tables, bt_lens, hv[3 * B:].reshape(B, W))
     packed = stg.upload(slot, host, device)
     d_lens, d_hid, d_ctx_in = packed[:B], packed[B:2 * B], packed[2 * B:3 * B]
     d_bt = packed[3 * B:].view(B, W)

@@ -214,6 +214,18 @@ def main():
             torch.cuda.synchronize()
             t.append((time.perf_counter() - a) * 1e6)
         extras["metadata_build_us"] = median(t)
+        if not args.no_cpu:
+            # the reference's approach to the same metadata: Python lists per cached token, then tensors
+            from oracle.metadata import SeqRecord, build_metadata as list_build
+            recs = [SeqRecord(False, h, l, l - 1, bt, bts) for l, h, bt, bts in
+                    zip(batch.seq_lens, batch.use_hidden, batch.block_tables, batch.block_tables_4_shared)]
+            t = []
+            for _ in range(3):
+                a = time.perf_counter()
+                list_build(recs, batch.block_size)
+                t.append((time.perf_counter() - a) * 1e6)
+            extras["metadata_build_us_cpu_list_algorithm"] = median(t)
+        extras["kv_write_prefill_16384"] = write_figures(torch, ops, dev, args.seed)
         if hasattr(ops, "kv_reproject"):
             extras.update(reproject_figures(torch, ops, dev, args.seed))
         result["extras"] = extras
@@ -222,6 +234,26 @@ def main():
         result["cpu_baseline"] = cpu_baseline(torch, np, batch, md, cache, hs, key, value, kv_seq_idx, new_slots,
                                               step_bytes, T, Hd)
     print(json.dumps(result))
+
+
+def write_figures(torch, ops, dev, seed):
+    """The cache write at a shape that can saturate HBM: a 16 384-token prompt batch at OPT-13B width,
+    K and V rows scattered by slot_mapping (the decode-step write of configs[1] moves 7.9 MB and is
+    bounded by launch latency, not bandwidth)."""
+    H, D, BS, T = 40, 128, 16, 16384
+    N = T // BS + 64
+    g = torch.Generator(device=dev).manual_seed(seed)
+    kv = torch.randn(T, 2 * H * D, generator=g, device=dev).half()
+    key, value = (x.view(T, H, D) for x in kv.chunk(2, -1))
+    cache = torch.zeros(2, N, BS, H, D, dtype=torch.float16, device=dev)
+    slots = torch.randperm(N * BS, generator=g, device=dev)[:T].contiguous()
+    ms = median(event_times(torch, lambda: ops.reshape_and_cache_flash(key, value, cache[0], cache[1], slots, "auto"), 30))
+    nbytes = T * 2 * (2 * H * D * 2)
+    gbs = nbytes / ms / 1e6
+    return {"workload": "K/V cache write of 16384 tokens, 40x128 f16, random slots", "ms": ms,
+            "algorithmic_bytes": nbytes,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
 
 
 def reproject_figures(torch, ops, dev, seed):
