@@ -127,12 +127,15 @@ class HybridAttentionImpl:
         decode_query = query[n_prefill:]
         if md.prefill_metadata is not None:
             pm = md.prefill_metadata
-            if self.prefill_attention is None:
-                raise NotImplementedError(
-                    "prompt attention (flash_attn_varlen_func, aptserve_flash_attn.py:405-447) is not part of "
-                    "this library: pass prefill_attention=callable(q, k, v, cu_seqlens, max_seqlen, scale)")
-            output[:n_prefill] = self.prefill_attention(query[:n_prefill], key[:n_prefill], value[:n_prefill],
-                                                        pm.seq_start_loc, pm.max_prefill_seq_len, self.scale)
+            if self.prefill_attention is not None:       # caller-supplied prompt attention
+                output[:n_prefill] = self.prefill_attention(query[:n_prefill], key[:n_prefill], value[:n_prefill],
+                                                            pm.seq_start_loc, pm.max_prefill_seq_len, self.scale)
+            else:                                        # aptserve_flash_attn.py:414-426
+                ops.flash_attn_varlen_func(
+                    q=query[:n_prefill], k=key[:n_prefill], v=value[:n_prefill], cu_seqlens_q=pm.seq_start_loc,
+                    cu_seqlens_k=pm.seq_start_loc, max_seqlen_q=pm.max_prefill_seq_len,
+                    max_seqlen_k=pm.max_prefill_seq_len, softmax_scale=self.scale, causal=True,
+                    out=output[:n_prefill])
         if md.decode_metadata is not None:
             dm = md.decode_metadata
             max_len = dm.max_decode_seq_len or None

@@ -422,3 +422,46 @@ def kv_reproject(x, w_kv, b_kv=None, out=None):
     """K/V re-projection of gathered hidden rows: ``[T,Hd] x w_kv[2Hd,Hd]^T + b_kv -> [T,2Hd]``
     (``k, v = out.chunk(2, -1)``), additional_designs/model_executor/models/aptserve_opt.py:123-124."""
     return linear_nt(x, w_kv, b_kv, out=out)
+
+
+# ------------------------------------------------------------------ prompt attention
+
+def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=None, max_seqlen_k=None,
+                           softmax_scale=None, causal: bool = True, window_size=None, alibi_slopes=None, out=None):
+    """Prompt-step case of the third-party function with the keywords used at
+    additional_designs/attention/backends/aptserve_flash_attn.py:414-426: q, k and v are the
+    packed, freshly projected ``[tokens, H, D]`` tensors of the same sequences
+    (``cu_seqlens_q is cu_seqlens_k``), causal.  Returns ``[tokens, H, D]``."""
+    dev = q.device
+    _need(causal, "only causal attention is provided")
+    _need(alibi_slopes is None, "alibi_slopes is not supported")
+    _need(window_size in (None, (-1, -1)), "sliding windows are not supported")
+    _need(cu_seqlens_q is not None, "cu_seqlens_q is required")
+    _need(cu_seqlens_k is None or cu_seqlens_k is cu_seqlens_q or torch.equal(cu_seqlens_k, cu_seqlens_q),
+          "prompt attention needs identical query and key sequence boundaries")
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        _check_data(n, t, dev)
+        _need(t.dim() == 3 and t.shape == q.shape, f"{n} must be [tokens, heads, head_dim] like q")
+        _need(t.stride(2) == 1 and t.stride(1) == t.size(2), f"{n}: heads of one token must be contiguous")
+        _need(t.dtype == q.dtype, "q, k, v dtypes differ")
+    _need(q.dtype in (torch.float16, torch.bfloat16), "f16 or bf16 expected")
+    _check_index("cu_seqlens_q", cu_seqlens_q, dev, torch.int32)
+    T, H, D = q.shape
+    n_seq = cu_seqlens_q.numel() - 1
+    _need(n_seq >= 0, "cu_seqlens must have a leading 0")
+    max_len = int(max_seqlen_q if max_seqlen_q is not None else (max_seqlen_k if max_seqlen_k is not None else T))
+    if softmax_scale is None:
+        softmax_scale = D ** -0.5
+    if out is None:
+        out = torch.empty(T, H, D, dtype=q.dtype, device=dev)
+    else:
+        _check_data("out", out, dev)
+        _need(out.shape == q.shape and out.dtype == q.dtype and out.stride(2) == 1 and out.stride(1) == D,
+              "out must look like q")
+    with torch.cuda.device(dev):
+        st = _lib.load().aps_varlen_prefill_attention(
+            out.data_ptr() if T else None, q.data_ptr() if T else None, k.data_ptr() if T else None,
+            v.data_ptr() if T else None, _ptr(cu_seqlens_q), n_seq if T else 0, max_len, H, D, q.stride(0),
+            k.stride(0), v.stride(0), out.stride(0), float(softmax_scale), _DTYPE_CODE[q.dtype], _stream(q))
+    _lib.check(st, "flash_attn_varlen_func")
+    return out

@@ -1,0 +1,246 @@
+// Causal attention over freshly projected, packed (varlen) q/k/v for gfx950 — the prompt step.
+//
+// One 256-thread workgroup owns 128 consecutive queries of one (sequence, head); each of its four
+// wavefronts owns 32 of them.  Keys/values are consumed 64 at a time through LDS.
+//
+// The score tile is computed transposed, S^T = K Q^T, with v_mfma_f32_32x32x16: in the result layout
+// a lane owns ONE query (column lane%32) and 16 of the 32 keys of a tile, so the running max / sum of
+// the online softmax are per-lane scalars plus one exchange with lane^32.  The same registers, rounded
+// to the operand dtype, are directly the B operand (k = keys) of O^T = V^T P^T, provided V^T is laid
+// out in LDS in the key order the result layout produces:
+//     position (key/16)*16 + ((key%8)/4)*8 + (key%16/8)*4 + key%4   holds   key.
+// V is transposed while it is staged (16-byte global loads, 16-bit LDS stores); K is staged row-major
+// with its 16-byte chunks XOR-swizzled by key%16 so the fragment reads do not collide in the 64 banks.
+#include "aps_common.h"
+
+#include <math.h>
+
+namespace aps {
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int BQ = 128;   // queries per workgroup
+constexpr int BKV = 64;   // keys per iteration
+constexpr int kThreads = 256;
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct PrefillArgs {
+  const char* q; const char* k; const char* v; char* out;
+  const int32_t* cu_seqlens;
+  int64_t q_stride_b, k_stride_b, v_stride_b, out_stride_b;  // token row strides in bytes
+  int num_heads;
+  float scale_log2;
+};
+
+template <bool BF16>
+__device__ __forceinline__ float16v mfma32(const u32x4& a, const u32x4& b, const float16v& c) {
+  if constexpr (BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                   0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0,
+                                                  0);
+}
+
+template <bool BF16>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  if constexpr (BF16) {
+    auto cv = [](float x) -> uint32_t {
+      uint32_t u = __float_as_uint(x);
+      if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40;
+      u += 0x7fffu + ((u >> 16) & 1u);
+      return u >> 16;
+    };
+    return cv(a) | (cv(b) << 16);
+  } else {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)a) |
+           ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)b) << 16);
+  }
+}
+
+__device__ __forceinline__ int vt_pos(int key) {  // see the file comment
+  return (key & ~15) + ((key & 7) >> 2) * 8 + ((key & 15) >> 3) * 4 + (key & 3);
+}
+
+template <bool BF16, int D>
+__global__ __launch_bounds__(kThreads) void prefill_attention_kernel(const PrefillArgs a) {
+  constexpr int KS = D / 16;          // k-steps of the score product
+  constexpr int DT = D / 32;          // 32-row tiles of O^T
+  constexpr int KROW = D * 2;         // bytes per key row in LDS
+  constexpr int KCH = KROW / 16;      // 16-byte chunks per key row
+  constexpr int VPITCH = BKV * 2 + 16;  // bytes per d-row of V^T (padding keeps rows off the same banks)
+  __shared__ __attribute__((aligned(16))) char k_lds[BKV * KROW];
+  __shared__ __attribute__((aligned(16))) char vt_lds[D * VPITCH];
+
+  const int seq = blockIdx.z, head = blockIdx.y;
+  const int s0 = a.cu_seqlens[seq], s1 = a.cu_seqlens[seq + 1];
+  const int len = s1 - s0;
+  const int q0 = blockIdx.x * BQ;
+  if (q0 >= len) return;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int qcol = lane & 31, half = lane >> 5;
+  const int my_q = q0 + wave * 32 + qcol;      // query index inside the sequence (may be >= len)
+  const bool q_live = my_q < len;
+
+  // Q^T fragments: B operand, lane = (query, 8 consecutive d of each 16-wide k-step)
+  u32x4 qf[KS];
+  {
+    const char* qp = a.q + (int64_t)(s0 + (q_live ? my_q : len - 1)) * a.q_stride_b + (int64_t)head * D * 2;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) qf[s] = *(const u32x4*)(qp + (16 * s + 8 * half) * 2);
+  }
+
+  float16v o[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[t][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  const int kv_end = min(len, q0 + BQ);  // causal: keys beyond the tile's last query are never needed
+  for (int kv0 = 0; kv0 < kv_end; kv0 += BKV) {
+    __syncthreads();  // previous tile fully consumed
+    // ---- stage K (row-major, swizzled) and V (transposed)
+    for (int c = tid; c < BKV * KCH; c += kThreads) {
+      const int key = c / KCH, ch = c % KCH;
+      const int gk = min(kv0 + key, len - 1);
+      const u32x4 kvv = *(const u32x4*)(a.k + (int64_t)(s0 + gk) * a.k_stride_b + (int64_t)head * D * 2 + ch * 16);
+      *(u32x4*)(k_lds + key * KROW + ((ch ^ (key & (KCH - 1) & 15)) * 16)) = kvv;
+    }
+    for (int c = tid; c < BKV * KCH; c += kThreads) {
+      const int key = c % BKV, ch = c / BKV;   // consecutive lanes -> consecutive keys of one d-chunk
+      const int gk = min(kv0 + key, len - 1);
+      const u32x4 vv = *(const u32x4*)(a.v + (int64_t)(s0 + gk) * a.v_stride_b + (int64_t)head * D * 2 + ch * 16);
+      const int pos = vt_pos(key);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t w = vv[i];
+        *(uint16_t*)(vt_lds + (ch * 8 + 2 * i) * VPITCH + pos * 2) = (uint16_t)(w & 0xffffu);
+        *(uint16_t*)(vt_lds + (ch * 8 + 2 * i + 1) * VPITCH + pos * 2) = (uint16_t)(w >> 16);
+      }
+    }
+    __syncthreads();
+
+    // ---- S^T = K Q^T for the two 32-key tiles
+    float16v st[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) st[t][e] = 0.f;
+      const int key = t * 32 + qcol;  // A operand row of this lane
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int ch = 2 * s + half;
+        const u32x4 kf = *(const u32x4*)(k_lds + key * KROW + ((ch ^ (key & (KCH - 1) & 15)) * 16));
+        st[t] = mfma32<BF16>(kf, qf[s], st[t]);
+      }
+    }
+    // ---- online softmax for this lane's query (its 32 keys here, the other 32 in lane^32)
+    float mx = m_run;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int key = kv0 + t * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+        const float sc = (key <= my_q && key < len) ? st[t][e] * a.scale_log2 : -INFINITY;
+        st[t][e] = sc;
+        mx = fmaxf(mx, sc);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_use = (mx == -INFINITY) ? 0.f : mx;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float p = __builtin_amdgcn_exp2f(st[t][e] - m_use);
+        st[t][e] = p;
+        psum += p;
+      }
+    psum += __shfl_xor(psum, 32);
+    l_run = l_run * alpha + psum;
+    m_run = mx;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
+    // ---- O^T += V^T P^T : four k-steps of 16 keys; P^T fragment = 8 consecutive result registers
+#pragma unroll
+    for (int t32 = 0; t32 < 2; ++t32)
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        u32x4 pf;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pf[i] = pack2<BF16>(st[t32][8 * ks + 2 * i], st[t32][8 * ks + 2 * i + 1]);
+        const int kpos = (t32 * 2 + ks) * 16 + half * 8;  // this lane's 8 keys of the step, in stored order
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+          const u32x4 vf = *(const u32x4*)(vt_lds + (t * 32 + qcol) * VPITCH + kpos * 2);
+          o[t] = mfma32<BF16>(vf, pf, o[t]);
+        }
+      }
+  }
+
+  // ---- normalise and store: lane owns query my_q, rows d = 32 t + 8 (e/4) + 4 half + e%4
+  if (!q_live) return;
+  const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+  char* op = a.out + (int64_t)(s0 + my_q) * a.out_stride_b + (int64_t)head * D * 2;
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int d = 32 * t + 8 * g + 4 * half;
+      uint2 w;
+      w.x = pack2<BF16>(o[t][4 * g] * inv, o[t][4 * g + 1] * inv);
+      w.y = pack2<BF16>(o[t][4 * g + 2] * inv, o[t][4 * g + 3] * inv);
+      *(uint2*)(op + d * 2) = w;
+    }
+}
+
+}  // namespace
+}  // namespace aps
+
+using namespace aps;
+
+extern "C" {
+
+int aps_varlen_prefill_attention(void* out, const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
+                                 int64_t num_seqs, int64_t max_seqlen, int num_heads, int head_size,
+                                 int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t out_stride,
+                                 float softmax_scale, int dtype, aps_stream_t stream) {
+  if (num_seqs < 0 || max_seqlen < 0 || num_heads <= 0 || head_size <= 0) return APS_ERR_INVALID_ARG;
+  if (num_seqs == 0 || max_seqlen == 0) return APS_OK;
+  if (!out || !q || !k || !v || !cu_seqlens) return APS_ERR_INVALID_ARG;
+  if (dtype != APS_F16 && dtype != APS_BF16) return APS_ERR_UNSUPPORTED;
+  if (head_size != 64 && head_size != 128) return APS_ERR_UNSUPPORTED;
+  const int64_t row = (int64_t)num_heads * head_size;
+  if (q_stride < row || k_stride < row || v_stride < row || out_stride < row) return APS_ERR_INVALID_ARG;
+  if (common_vec_bytes({addr(q), addr(k), addr(v), (uint64_t)q_stride * 2, (uint64_t)k_stride * 2,
+                        (uint64_t)v_stride * 2}) != 16 ||
+      common_vec_bytes({addr(out), (uint64_t)out_stride * 2}) < 8)
+    return APS_ERR_UNSUPPORTED;
+  if (num_seqs > 65535 || num_heads > 65535) return APS_ERR_UNSUPPORTED;
+  PrefillArgs a;
+  a.q = (const char*)q; a.k = (const char*)k; a.v = (const char*)v; a.out = (char*)out;
+  a.cu_seqlens = cu_seqlens;
+  a.q_stride_b = q_stride * 2; a.k_stride_b = k_stride * 2; a.v_stride_b = v_stride * 2; a.out_stride_b = out_stride * 2;
+  a.num_heads = num_heads;
+  a.scale_log2 = softmax_scale * kLog2e;
+  const dim3 grid((unsigned)((max_seqlen + BQ - 1) / BQ), (unsigned)num_heads, (unsigned)num_seqs);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == APS_F16) {
+    if (head_size == 64) hipLaunchKernelGGL((prefill_attention_kernel<false, 64>), grid, dim3(kThreads), 0, s, a);
+    else hipLaunchKernelGGL((prefill_attention_kernel<false, 128>), grid, dim3(kThreads), 0, s, a);
+  } else {
+    if (head_size == 64) hipLaunchKernelGGL((prefill_attention_kernel<true, 64>), grid, dim3(kThreads), 0, s, a);
+    else hipLaunchKernelGGL((prefill_attention_kernel<true, 128>), grid, dim3(kThreads), 0, s, a);
+  }
+  return launch_status();
+}
+
+}  // extern "C"

@@ -209,6 +209,26 @@ int aps_paged_decode_attention(
     aps_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Prompt-step attention on freshly projected q/k/v (no cache read).
+ * ref: third-party vllm_flash_attn.flash_attn_varlen_func with causal=True as
+ * called at attention/backends/aptserve_flash_attn.py:414-426.  Sequences are
+ * packed along the token dimension and delimited by cu_seqlens (int32
+ * [num_seqs+1], leading 0); query i of a sequence attends to keys 0..i of the
+ * same sequence; softmax in fp32; result in the operand dtype.
+ * q/k/v/out: [tokens, H, D] with token-row strides (elements), heads
+ * contiguous; f16 or bf16; D in {64, 128}.  max_seqlen: host-side bound of
+ * the sequence lengths (sizes the grid).
+ * ------------------------------------------------------------------------ */
+int aps_varlen_prefill_attention(void* out, const void* q, const void* k,
+                                 const void* v, const int32_t* cu_seqlens,
+                                 int64_t num_seqs, int64_t max_seqlen,
+                                 int num_heads, int head_size,
+                                 int64_t q_stride, int64_t k_stride,
+                                 int64_t v_stride, int64_t out_stride,
+                                 float softmax_scale, int dtype,
+                                 aps_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Ragged-batch metadata, built on the GPU from a per-sequence description.
  * ref: worker/aptserve_model_runner.py:240-842 (_prepare_model_input), hybrid
  * parts :256-304, :410-437, :516-564, :601-668, :707-733, :772-785.

@@ -104,10 +104,12 @@ def test_prefill_layer_cache_writes_and_output(dev, frac):
     close(out, ref)
     close(d_kv, ref_kv)
     assert torch.equal(d_sh.cpu(), sh)        # prompts never touch the shared cache
-    # without a prompt-attention callable the layer refuses instead of falling back
-    bare = backend.HybridOPTAttention(Hd, H, *(w.to(dev) for w in W))
-    with pytest.raises(NotImplementedError):
-        bare(hs.to(dev), kv.to(dev), sh.to(dev), metadata.build_from_batch(batch, dev))
+    # the library's own prompt attention gives the same answer as the injected one
+    own = backend.HybridOPTAttention(Hd, H, *(w.to(dev) for w in W))
+    d_kv2 = kv.to(dev)
+    out2 = own(hs.to(dev), d_kv2, sh.to(dev), metadata.build_from_batch(batch, dev))
+    close(out2, ref)
+    assert torch.equal(d_kv2, d_kv)
 
 
 def test_decode_follows_prefill_through_the_hip_path(dev):
@@ -120,7 +122,7 @@ def test_decode_follows_prefill_through_the_hip_path(dev):
     hid = workloads.pick_hidden(rng, len(lens), 0.5)
     full = workloads.allocate_blocks(rng, [l + 1 for l in lens], hid, N, BS, is_prompt=True)
     xs = [randn((l + 1, Hd), 30 + i) for i, l in enumerate(lens)]
-    layer = backend.HybridOPTAttention(Hd, H, *dW, prefill_attention=torch_prefill_attention)
+    layer = backend.HybridOPTAttention(Hd, H, *dW)      # prompt and decode attention both from the library
     kv1, sh1 = backend.allocate_caches(1, N, BS, H, D, torch.float16, dev)
     md = metadata.build_metadata(True, [l + 1 for l in lens], hid, full.block_tables, full.block_tables_4_shared, BS, dev)
     out_full = layer(torch.cat(xs).to(dev), kv1[0], sh1, md)
