@@ -228,6 +228,8 @@ def main():
         extras["kv_write_prefill_16384"] = write_figures(torch, ops, dev, args.seed)
         if hasattr(ops, "kv_reproject"):
             extras.update(reproject_figures(torch, ops, dev, args.seed))
+        torch.cuda.empty_cache()
+        extras["opt13b_step_loop"] = step_loop_figures(torch, dev, args.seed)
         result["extras"] = extras
 
     if not args.no_cpu:
@@ -254,6 +256,36 @@ def write_figures(torch, ops, dev, seed):
             "algorithmic_bytes": nbytes,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
+
+
+def step_loop_figures(torch, dev, seed, max_steps=48):
+    """BASELINE configs[4]: OPT-13B (random-init fp16, 40 layers) serving steps on the hybrid cache with
+    synthetic arrivals (3 req/s, CV 1) and lognormal prompt/output lengths; half of the requests hidden-cached."""
+    from aptserve_hip import backend, opt_model, step_loop
+    cfg = opt_model.OPTConfig.opt_13b()
+    N, BS = 6144, 16
+    w = opt_model.random_weights(cfg, seed, dev)
+    model = opt_model.HybridOPTModel(cfg, w)
+    kv, shared = backend.allocate_caches(cfg.num_hidden_layers, N, BS, cfg.num_attention_heads,
+                                         cfg.hidden_size // cfg.num_attention_heads, torch.float16, dev)
+    reqs = step_loop.synth_requests(seed, 64, rate=3.0, cv=1.0, hidden_fraction=0.5)
+    loop = step_loop.StepLoop(lambda ids, pos, md: model(ids, pos, kv, shared, md), model.next_tokens, reqs, N, BS, dev)
+    loop.run(4)                      # warm-up steps (allocator, kernels)
+    log = loop.run(max_steps)[4:]
+    dec = [e for e in log if e["kind"] == "decode"]
+    pre = [e for e in log if e["kind"] == "prefill"]
+    mean = lambda xs: sum(xs) / len(xs) if xs else None
+    return {"workload": "OPT-13B 40 layers fp16 random-init, eager; gamma arrivals 3 req/s cv 1; prompts "
+                        "lognormal(5.5,1.0) in [4,2048]; outputs lognormal(5.0,0.9) in [4,1024]; 50% hidden-cached",
+            "steps": len(log), "decode_steps": len(dec), "prefill_steps": len(pre),
+            "decode_ms_per_step": mean([e["model_ms"] for e in dec]),
+            "decode_seqs_per_step": mean([e["seqs"] for e in dec]),
+            "decode_rows_per_step": mean([e["rows"] for e in dec]),
+            "prefill_ms_per_step": mean([e["model_ms"] for e in pre]),
+            "prefill_tokens_per_step": mean([e["tokens"] for e in pre]),
+            "metadata_ms_per_step": mean([e["metadata_ms"] for e in log]),
+            "decode_tokens_per_s": (sum(e["seqs"] for e in dec) / (sum(e["model_ms"] + e["metadata_ms"] for e in dec) * 1e-3)
+                                    if dec else None)}
 
 
 def reproject_figures(torch, ops, dev, seed):

@@ -42,4 +42,4 @@ their outputs are covered by the stated tolerances instead (1e-3 relative with
 fp32 accumulation, 2e-2 absolute for fp16 outputs).
 """
 
-from . import cache_ops, fp8, reproject, attention, metadata, layer  # noqa: F401
+from . import cache_ops, fp8, reproject, attention, metadata, layer, model  # noqa: F401
