@@ -381,12 +381,14 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, block_table=None, cache_seqlens
 
 # --------------------------------------------------------------------- a5 / a6
 
-def linear_nt(x, weight, bias=None, out=None, out_row_map=None):
+def linear_nt(x, weight, bias=None, out=None, out_row_map=None, workspace=None, split_k: bool = True):
     """``out = x @ weight.T + bias`` on the matrix cores (f16/bf16, fp32 accumulation).
 
     ``x [M, K]`` and ``weight [N, K]`` may be row-strided views (a row slice of the fused
     QKV weight, a ``chunk`` of activations); ``N % 256 == 0`` and ``K % 64 == 0``.
     ``out_row_map`` (int64 ``[M]``) scatters result row ``m`` to ``out[out_row_map[m]]``.
+    With ``split_k`` (default) a problem of few output tiles is split along K through an fp32
+    ``workspace`` (allocated here when not given) so that enough workgroups stream the weights.
     """
     dev = x.device
     _check_data("x", x, dev)
@@ -409,11 +411,17 @@ def linear_nt(x, weight, bias=None, out=None, out_row_map=None):
         _need(out_row_map.numel() == M, "one destination row per input row expected")
     else:
         _need(out.size(0) >= M, "out has fewer rows than x")
+    lib = _lib.load()
+    need = lib.aps_linear_nt_workspace_bytes(M, N, K) if split_k else 0
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)     # scratch is host-side plumbing
+    ws_ptr = workspace.data_ptr() if need else None
     with torch.cuda.device(dev):
-        st = _lib.load().aps_linear_nt(
+        st = lib.aps_linear_nt(
             x.data_ptr() if M else None, weight.data_ptr(), None if bias is None else bias.data_ptr(),
             out.data_ptr() if out.numel() else None, M, N, K, x.stride(0), weight.stride(0), out.stride(0),
-            None if out_row_map is None else _ptr(out_row_map), out.size(0), _DTYPE_CODE[x.dtype], _stream(x))
+            None if out_row_map is None else _ptr(out_row_map), out.size(0), _DTYPE_CODE[x.dtype], ws_ptr,
+            workspace.numel() * workspace.element_size() if need else 0, _stream(x))
     _lib.check(st, "linear_nt")
     return out
 

@@ -59,6 +59,10 @@ struct GemmArgs {
   const int64_t* row_map;
   int64_t row_map_limit;
   int c_aligned16;  // out pointer and row pitch allow 128-bit stores
+  // split-K (small M): workgroup (tile, z) handles k-tiles [z*kt_per_split, ...) and stores its fp32
+  // partial tile to partial[z][m][n]; a second kernel adds the splits and the bias
+  float* partial;
+  int kt_per_split;
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
@@ -126,10 +130,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   const uint32_t voff_w0 = (uint32_t)(lrow * g.ldw_b + lchunk0 * 16), voff_w1 = (uint32_t)(lrow * g.ldw_b + lchunk1 * 16);
   const uint32_t grp_a = (uint32_t)(8 * g.lda_b), grp_w = (uint32_t)(8 * g.ldw_b);
 
+  const int kt_base_ = g.partial ? (int)blockIdx.y * g.kt_per_split : 0;
   auto issue_loads = [&](int kt) {
     char* sa = lds + (kt & 1) * kStageBytes;
     char* sw = sa + kTileBytes;
-    const uint32_t koff = (uint32_t)kt * (BK * 2);
+    const uint32_t koff = (uint32_t)(kt_base_ + kt) * (BK * 2);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int i = wave * 8 + j;  // 8-row group of the tile handled by this wave-wide load
@@ -179,7 +184,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     }
   };
 
-  const int nk = (int)(g.k / BK);
+  const int nk_total = (int)(g.k / BK);
+  const int kt_base = g.partial ? blockIdx.y * g.kt_per_split : 0;
+  const int nk = g.partial ? min(g.kt_per_split, nk_total - kt_base) : nk_total;
   u32x4 a0[4], w0[4], a1[4], w1[4];
   issue_loads(0);
   if (nk > 1) {
@@ -217,6 +224,21 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // Each wave owns a [128 rows][128 cols] fp16 image (row pitch 272 B so that the two half-waves,
   // four rows apart, use different banks).  Neighbouring lanes swap one value so that every lane
   // writes a 32-bit pair; the image is then read back 16 bytes per lane, 16 lanes per row.
+  if (g.partial) {  // split-K: raw fp32 partial sums, lanes of a half-wave write 128 contiguous bytes
+    float* pz = g.partial + (int64_t)blockIdx.y * g.m * g.n;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t col = col0 + wn * 128 + j * 32 + frow;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int64_t row = row0 + wm * 128 + i * 32 + 8 * (e >> 2) + 4 * fhalf + (e & 3);
+          if (row < g.m) pz[row * g.n + col] = acc[i][j][e];
+        }
+    }
+    return;
+  }
   APS_WAIT_LGKM0();
   APS_BARRIER();  // the main-loop tiles are dead; the LDS is reused for the images
   char* img = lds + wave * kEpiWaveBytes;
@@ -267,6 +289,35 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   }
 }
 
+// out[m][n] = sum_z partial[z][m][n] + bias[n], rounded once; 4 columns per thread
+template <bool BF16>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, const void* bias,
+                                                            uint16_t* out, int64_t m, int64_t n, int64_t ldc,
+                                                            int splits, const int64_t* row_map,
+                                                            int64_t row_map_limit) {
+  const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (idx >= m * n) return;
+  const int64_t row = idx / n, col = idx - row * n;
+  float4 s = *(const float4*)(partial + idx);
+  for (int z = 1; z < splits; ++z) {
+    const float4 p = *(const float4*)(partial + (int64_t)z * m * n + idx);
+    s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
+  }
+  if (bias) {
+    const uint16_t* b = (const uint16_t*)bias + col;
+    auto cv = [](uint16_t v) { return BF16 ? __uint_as_float((uint32_t)v << 16) : (float)__builtin_bit_cast(_Float16, v); };
+    s.x += cv(b[0]); s.y += cv(b[1]); s.z += cv(b[2]); s.w += cv(b[3]);
+  }
+  int64_t orow = row;
+  if (row_map) {
+    orow = row_map[row];
+    if (orow < 0 || orow >= row_map_limit) return;
+  }
+  uint16_t* o = out + orow * ldc + col;
+  if (BF16) { o[0] = f32_to_bf16_bits(s.x); o[1] = f32_to_bf16_bits(s.y); o[2] = f32_to_bf16_bits(s.z); o[3] = f32_to_bf16_bits(s.w); }
+  else { o[0] = f32_to_f16_bits(s.x); o[1] = f32_to_f16_bits(s.y); o[2] = f32_to_f16_bits(s.z); o[3] = f32_to_f16_bits(s.w); }
+}
+
 }  // namespace
 }  // namespace aps
 
@@ -274,9 +325,26 @@ using namespace aps;
 
 extern "C" {
 
+int aps_linear_nt_splits(int64_t m, int64_t n, int64_t k) {
+  // Few tiles (a decode step's handful of tokens) cannot pull the weights at HBM speed with one workgroup
+  // per tile: split K until about two waves of workgroups exist, keeping at least 4 k-tiles per split.
+  if (m <= 0 || n <= 0 || k <= 0 || n % BN != 0 || k % BK != 0) return 1;
+  if (m > 2 * BM) return 1;  // beyond two row tiles the fp32 partials cost more than the extra workgroups gain
+  const int64_t tiles = ((m + BM - 1) / BM) * (n / BN);
+  const int64_t nk = k / BK;
+  int64_t s = 1;
+  while (tiles * s < 384 && nk / (s * 2) >= 4 && s < 32) s *= 2;
+  return (int)s;
+}
+
+int64_t aps_linear_nt_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+  const int s = aps_linear_nt_splits(m, n, k);
+  return s > 1 ? (int64_t)s * m * n * 4 : 0;
+}
+
 int aps_linear_nt(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n, int64_t k,
                   int64_t x_stride, int64_t w_stride, int64_t out_stride, const int64_t* out_row_map,
-                  int64_t out_rows, int dtype, aps_stream_t stream) {
+                  int64_t out_rows, int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream) {
   if (m < 0 || n <= 0 || k <= 0) return APS_ERR_INVALID_ARG;
   if (m == 0) return APS_OK;
   if (!x || !weight || !out) return APS_ERR_INVALID_ARG;
@@ -299,7 +367,16 @@ int aps_linear_nt(const void* x, const void* weight, const void* bias, void* out
   const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
   if (total >= ((int64_t)1 << 30)) return APS_ERR_UNSUPPORTED;
   const int64_t per_xcd = (total + kNumXcd - 1) / kNumXcd;
-  const dim3 grid((unsigned)(per_xcd * kNumXcd));
+  int splits = 1;
+  if (workspace) {
+    splits = aps_linear_nt_splits(m, n, k);
+    if (splits > 1 && (workspace_bytes < (int64_t)splits * m * n * 4 || (addr(workspace) & 15))) return APS_ERR_WORKSPACE;
+  }
+  const int64_t nk_all = k / BK;
+  g.partial = splits > 1 ? (float*)workspace : nullptr;
+  g.kt_per_split = (int)((nk_all + splits - 1) / splits);
+  if (splits > 1) splits = (int)((nk_all + g.kt_per_split - 1) / g.kt_per_split);  // no empty split
+  const dim3 grid((unsigned)(per_xcd * kNumXcd), (unsigned)splits);
   hipStream_t s = (hipStream_t)stream;
   // more than 64 KiB of dynamic LDS has to be allowed per function (and per device)
   const void* fn = dtype == APS_BF16 ? (const void*)gemm_nt_kernel<true> : (const void*)gemm_nt_kernel<false>;
@@ -309,6 +386,16 @@ int aps_linear_nt(const void* x, const void* weight, const void* bias, void* out
     hipLaunchKernelGGL(gemm_nt_kernel<true>, grid, dim3(kThreads), kLdsBytes, s, g);
   else
     hipLaunchKernelGGL(gemm_nt_kernel<false>, grid, dim3(kThreads), kLdsBytes, s, g);
+  int st = launch_status();
+  if (st != APS_OK || splits <= 1) return st;
+  const int64_t quads = (m * n + 3) / 4;
+  const dim3 rgrid((unsigned)((quads + 255) / 256));
+  if (dtype == APS_BF16)
+    hipLaunchKernelGGL(splitk_reduce_kernel<true>, rgrid, dim3(256), 0, s, (const float*)workspace, bias,
+                       (uint16_t*)out, m, n, out_stride, splits, out_row_map, out_rows);
+  else
+    hipLaunchKernelGGL(splitk_reduce_kernel<false>, rgrid, dim3(256), 0, s, (const float*)workspace, bias,
+                       (uint16_t*)out, m, n, out_stride, splits, out_row_map, out_rows);
   return launch_status();
 }
 

@@ -296,11 +296,19 @@ int aps_build_prefill_metadata(
  * out_row_map (nullable): row m is stored at row out_row_map[m] of out (rows of
  * out_stride elements; negative or >= out_rows: skipped) — the epilogue that
  * writes re-projected K/V rows straight into [blocks, BS, H, D] tiles by slot.
+ * workspace (nullable): fp32 scratch of aps_linear_nt_workspace_bytes(m,n,k)
+ * bytes, 16-byte aligned, owned by the caller.  With it, a problem of few
+ * output tiles (a decode step's handful of rows) is split along K into
+ * aps_linear_nt_splits(m,n,k) partial products that a second kernel adds (in
+ * fp32, then bias, then one rounding); without it one workgroup per tile runs.
  * ------------------------------------------------------------------------ */
+int aps_linear_nt_splits(int64_t m, int64_t n, int64_t k);
+int64_t aps_linear_nt_workspace_bytes(int64_t m, int64_t n, int64_t k);
 int aps_linear_nt(const void* x, const void* weight, const void* bias,
                   void* out, int64_t m, int64_t n, int64_t k, int64_t x_stride,
                   int64_t w_stride, int64_t out_stride,
                   const int64_t* out_row_map, int64_t out_rows, int dtype,
+                  void* workspace, int64_t workspace_bytes,
                   aps_stream_t stream);
 
 /* Plain device copy of nbytes (16-byte aligned pointers): the known-size
