@@ -47,6 +47,25 @@ __global__ __launch_bounds__(kMaxThreads) void row_mover(Op op, int64_t n_items,
 
 // ---------------------------------------------------------------- descriptors
 
+// slot -> (block, offset).  Block sizes are powers of two in practice: a shift instead of a 64-bit
+// division per 16-byte chunk.
+struct BlockSplit {
+  int block_size, shift;  // shift < 0: not a power of two
+  __host__ explicit BlockSplit(int bs) : block_size(bs), shift(-1) {
+    for (int s = 0; s < 31; ++s)
+      if ((1 << s) == bs) shift = s;
+  }
+  __device__ __forceinline__ void operator()(int64_t slot, int64_t& blk, int64_t& off) const {
+    if (shift >= 0) {
+      blk = slot >> shift;
+      off = slot & (block_size - 1);
+    } else {
+      blk = slot / block_size;
+      off = slot - blk * block_size;
+    }
+  }
+};
+
 struct HiddenToCacheOp {
   const char* hidden; char* cache;
   const int64_t* slot_mapping; const int64_t* src_idx; const int64_t* tgt_idx;
@@ -152,7 +171,7 @@ struct KvScatterOp {
   const char* key; const char* value; char* k_cache; char* v_cache;
   const int64_t* slot_mapping; const int64_t* token_idx;
   int64_t num_tokens, key_stride_b, value_stride_b, block_stride_b, row_b, num_blocks;
-  int block_size;
+  BlockSplit split;
   __device__ RowDesc operator()(int64_t item) const {
     RowDesc r{nullptr, nullptr};
     const int64_t t = item >> 1;
@@ -160,9 +179,10 @@ struct KvScatterOp {
     if (tok < 0 || tok >= num_tokens) return r;
     const int64_t slot = slot_mapping[tok];
     if (slot < 0) return r;
-    const int64_t blk = slot / block_size;
+    int64_t blk, in_blk;
+    split(slot, blk, in_blk);
     if (blk >= num_blocks) return r;
-    const int64_t off = blk * block_stride_b + (slot - blk * block_size) * row_b;
+    const int64_t off = blk * block_stride_b + in_blk * row_b;
     if (item & 1) { r.src = value + tok * value_stride_b; r.dst = v_cache + off; }
     else          { r.src = key + tok * key_stride_b;     r.dst = k_cache + off; }
     return r;
@@ -178,7 +198,7 @@ struct MixedKvOp {
   int64_t n_kv, n_hidden, num_tot;
   int64_t key_stride_b, value_stride_b, block_stride_b, shared_block_stride_b, row_b;
   int64_t num_blocks, num_shared_blocks;
-  int block_size; unsigned flags;
+  BlockSplit split; unsigned flags;
   __device__ RowDesc operator()(int64_t item) const {
     RowDesc r{nullptr, nullptr};
     const int64_t blk = item >> 1;
@@ -205,10 +225,10 @@ struct MixedKvOp {
       to_shared = true;
     }
     if (slot < 0) return r;
-    const int64_t b = slot / block_size;
+    int64_t b, in_blk;
+    split(slot, b, in_blk);
     if (b >= (to_shared ? num_shared_blocks : num_blocks)) return r;
-    const int64_t off_b = b * (to_shared ? shared_block_stride_b : block_stride_b) +
-                          (slot - b * block_size) * row_b;
+    const int64_t off_b = b * (to_shared ? shared_block_stride_b : block_stride_b) + in_blk * row_b;
     if (item & 1) { r.src = value + tok * value_stride_b; r.dst = (to_shared ? sv_cache : v_cache) + off_b; }
     else          { r.src = key + tok * key_stride_b;     r.dst = (to_shared ? sk_cache : k_cache) + off_b; }
     return r;
@@ -469,7 +489,7 @@ int aps_reshape_and_cache_flash(const void* key, const void* value, void* key_ca
     const int64_t e = in_b;
     KvScatterOp op{(const char*)key, (const char*)value, (char*)key_cache, (char*)value_cache, slot_mapping,
                    token_idx, num_tokens, key_stride * e, value_stride * e, block_stride * e, row * e, num_blocks,
-                   block_size};
+                   BlockSplit(block_size)};
     const int vb = common_vec_bytes({addr(key), addr(value), addr(key_cache), addr(value_cache),
                                      (uint64_t)(key_stride * e), (uint64_t)(value_stride * e),
                                      (uint64_t)(block_stride * e), (uint64_t)(row * e)});
@@ -517,7 +537,7 @@ int aps_mixed_kv_to_cache(const void* key, const void* value, void* k_cache, voi
   MixedKvOp op{(const char*)key, (const char*)value, (char*)k_cache, (char*)v_cache, (char*)shared_k_cache,
                (char*)shared_v_cache, slot_mapping, slot_mapping_shared, kv_cache_use_tot, hidden_cache_use_tot,
                n_kv, n_hidden, num_tot_tokens, key_stride * e, value_stride * e, block_stride * e,
-               shared_block_stride * e, row * e, num_blocks, num_shared_blocks, block_size, flags};
+               shared_block_stride * e, row * e, num_blocks, num_shared_blocks, BlockSplit(block_size), flags};
   const int vb = common_vec_bytes({addr(key), addr(value), addr(k_cache), addr(v_cache), addr(shared_k_cache),
                                    addr(shared_v_cache), (uint64_t)(key_stride * e), (uint64_t)(value_stride * e),
                                    (uint64_t)(block_stride * e), (uint64_t)(shared_block_stride * e),

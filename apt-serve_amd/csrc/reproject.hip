@@ -4,12 +4,16 @@
 // fused QKV weight [3*Hd, Hd] and the holder of gathered hidden rows [T, Hd]
 // are laid out.
 //
-// Tiling: one 256-thread workgroup (4 wavefronts, 2 x 2) owns a 256 x 256 tile
-// of C; each wavefront owns 128 x 128 = 4 x 4 MFMA 32x32x16 tiles (256 fp32
-// accumulator registers per lane).  The K loop moves BK = 64 at a time through
-// a two-stage LDS ring (2 x (32 + 32) KiB of the 160 KiB per CU; 136 KiB with the epilogue images): tile t+1 is
-// copied global -> LDS by buffer_load ... lds (no VGPR round trip) while the
-// matrix cores consume tile t.
+// Tiling: one 512-thread workgroup (8 wavefronts, 2 x 4) owns a 256 x 256 tile
+// of C; each wavefront owns 128 x 64 = 4 x 2 MFMA 32x32x16 tiles (128 fp32
+// accumulator registers per lane), so two wavefronts fit on every SIMD.  That
+// matters more than the larger per-wave tile it replaces: a wavefront issues in
+// order, and while it is held at a global load the matrix core of its SIMD is
+// only kept busy by the other wavefront (with one wavefront per SIMD the main
+// loop took 1.4x the cycles).  The K loop moves BK = 64 at a time through a
+// two-stage LDS ring (2 x (32 + 32) KiB of the 160 KiB per CU; 144 KiB with the
+// epilogue images): tile t+1 is copied global -> LDS by buffer_load ... lds (no
+// VGPR round trip) while the matrix cores consume tile t.
 //
 // LDS layout: a tile is [256 rows][8 chunks of 16 B]; chunk c of row r lives at
 // position c ^ ((r >> 1) % 8).  The LDS of gfx950 serves a 128-bit read to 16
@@ -21,7 +25,7 @@
 // fetches chunk (l%8) ^ ((row>>1)%8) of row l/8 of its 8-row group.
 //
 // Schedule: fragments live in two register sets; while the matrix cores work
-// on k-step s the 8 ds_read_b128 of k-step s+1 are in flight (2 MFMA : 1 read).
+// on k-step s the 6 ds_read_b128 of k-step s+1 are in flight (8 MFMA : 6 reads).
 // Before the last k-step of a tile every wave has its fragments in registers,
 // so after one barrier the stage can be refilled with tile t+2 while the last
 // k-step runs and the first fragments of tile t+1 stream in.  Waits and the
@@ -40,13 +44,16 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
+constexpr int kWaves = kThreads / 64;
+constexpr int WM = 128, WN = 64;                  // wavefront tile
 constexpr int kTileBytes = BM * BK * 2;          // 32 KiB, same for A and W tiles
 constexpr int kStageBytes = 2 * kTileBytes;      // A + W
 constexpr int kStages = 2;
-constexpr int kEpiPitch = 128 * 2 + 16;           // bytes per row of a wave's epilogue image
-constexpr int kEpiWaveBytes = 128 * kEpiPitch;    // 34 KiB
-constexpr int kLdsBytes = 4 * kEpiWaveBytes > kStages * kStageBytes ? 4 * kEpiWaveBytes : kStages * kStageBytes;
+constexpr int kEpiPitch = WN * 2 + 16;            // bytes per row of a wave's epilogue image
+constexpr int kEpiWaveBytes = WM * kEpiPitch;     // 18 KiB
+constexpr int kLdsBytes =
+    kWaves * kEpiWaveBytes > kStages * kStageBytes ? kWaves * kEpiWaveBytes : kStages * kStageBytes;
 constexpr int kNumXcd = 8;
 constexpr int kGroupM = 8;
 
@@ -94,12 +101,12 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
 #define APS_BARRIER() asm volatile("s_barrier" ::: "memory")
 
 template <bool BF16>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_nt_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_nt_kernel(
     const GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave >> 2, wn = wave & 3;
 
   // ---- tile assignment: XCD-contiguous, grouped 8 tiles along M
   int pid_m, pid_n;
@@ -136,8 +143,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     char* sw = sa + kTileBytes;
     const uint32_t koff = (uint32_t)(kt_base_ + kt) * (BK * 2);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int i = wave * 8 + j;  // 8-row group of the tile handled by this wave-wide load
+    for (int j = 0; j < 4; ++j) {
+      const int i = wave * 4 + j;  // 8-row group of the tile handled by this wave-wide load
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(sa + i * 1024), 16,
                                                (j & 1) ? voff_a1 : voff_a0, koff + i * grp_a, 0, 0);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (__attribute__((address_space(3))) void*)(sw + i * 1024), 16,
@@ -147,51 +154,51 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 
   // ---- LDS -> register fragment addressing (row = base + lane%32, chunk = 2*ks + lane/32, swizzled)
   const int frow = lane & 31, fhalf = lane >> 5;
-  const uint32_t a_row_off = (uint32_t)((wm * 128 + frow) * (BK * 2));
-  const uint32_t w_row_off = (uint32_t)((wn * 128 + frow) * (BK * 2));
+  const uint32_t a_row_off = (uint32_t)((wm * WM + frow) * (BK * 2));
+  const uint32_t w_row_off = (uint32_t)((wn * WN + frow) * (BK * 2));
   uint32_t chunk_off[4];
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) chunk_off[ks] = (uint32_t)(((2 * ks + fhalf) ^ ((frow >> 1) & 7)) * 16);
 
-  float16v acc[4][4];
+  float16v acc[4][2];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  auto read_frags = [&](int kt, int ks, u32x4(&af)[4], u32x4(&wf)[4]) {
+  auto read_frags = [&](int kt, int ks, u32x4(&af)[4], u32x4(&wf)[2]) {
     const char* sa = lds + (kt & 1) * kStageBytes;
     const char* sw = sa + kTileBytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      af[i] = *(const u32x4*)(sa + a_row_off + i * (32 * BK * 2) + chunk_off[ks]);
-      wf[i] = *(const u32x4*)(sw + w_row_off + i * (32 * BK * 2) + chunk_off[ks]);
-    }
+    for (int i = 0; i < 4; ++i) af[i] = *(const u32x4*)(sa + a_row_off + i * (32 * BK * 2) + chunk_off[ks]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) wf[i] = *(const u32x4*)(sw + w_row_off + i * (32 * BK * 2) + chunk_off[ks]);
   };
-  auto mfma16 = [&](const u32x4(&af)[4], const u32x4(&wf)[4]) {
+  auto mfma8 = [&](const u32x4(&af)[4], const u32x4(&wf)[2]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = mfma32<BF16>(af[i], wf[j], acc[i][j]);
+      for (int j = 0; j < 2; ++j) acc[i][j] = mfma32<BF16>(af[i], wf[j], acc[i][j]);
   };
-  auto interleave = [&]() {  // scheduling hint: 2 MFMA, then 1 LDS read, eight times
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
+  auto interleave = [&]() {  // scheduling hint: the 6 LDS reads spread over the 8 MFMA of a k-step
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
   };
 
   const int nk_total = (int)(g.k / BK);
   const int kt_base = g.partial ? blockIdx.y * g.kt_per_split : 0;
   const int nk = g.partial ? min(g.kt_per_split, nk_total - kt_base) : nk_total;
-  u32x4 a0[4], w0[4], a1[4], w1[4];
+  u32x4 a0[4], w0[2], a1[4], w1[2];
   issue_loads(0);
   if (nk > 1) {
     issue_loads(1);
-    APS_WAIT_VM(16);  // tile 0 has landed, tile 1 may still be in flight
+    APS_WAIT_VM(8);  // tile 0 has landed, tile 1 may still be in flight
   } else {
     APS_WAIT_VM(0);
   }
@@ -199,41 +206,40 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   read_frags(0, 0, a0, w0);
   int kt = 0;
   for (; kt + 2 < nk; ++kt) {  // steady state: a tile kt+2 exists, the body has no branches
-    read_frags(kt, 1, a1, w1); mfma16(a0, w0); interleave();
-    read_frags(kt, 2, a0, w0); mfma16(a1, w1); interleave();
-    read_frags(kt, 3, a1, w1); mfma16(a0, w0); interleave();
+    read_frags(kt, 1, a1, w1); mfma8(a0, w0); interleave();
+    read_frags(kt, 2, a0, w0); mfma8(a1, w1); interleave();
+    read_frags(kt, 3, a1, w1); mfma8(a0, w0); interleave();
     APS_WAIT_LGKM0();  // every fragment of tile kt is in registers: its stage is free
     APS_WAIT_VM(0);    // tile kt+1 has landed (this wave's part; the barrier covers the others)
     APS_BARRIER();
     issue_loads(kt + 2);
-    read_frags(kt + 1, 0, a0, w0); mfma16(a1, w1); interleave();
+    read_frags(kt + 1, 0, a0, w0); mfma8(a1, w1); interleave();
   }
   for (; kt < nk; ++kt) {  // last two tiles: nothing left to issue
-    read_frags(kt, 1, a1, w1); mfma16(a0, w0); interleave();
-    read_frags(kt, 2, a0, w0); mfma16(a1, w1); interleave();
-    read_frags(kt, 3, a1, w1); mfma16(a0, w0); interleave();
+    read_frags(kt, 1, a1, w1); mfma8(a0, w0); interleave();
+    read_frags(kt, 2, a0, w0); mfma8(a1, w1); interleave();
+    read_frags(kt, 3, a1, w1); mfma8(a0, w0); interleave();
     APS_WAIT_LGKM0();
     APS_WAIT_VM(0);
     APS_BARRIER();
     if (kt + 1 < nk) read_frags(kt + 1, 0, a0, w0);
-    mfma16(a1, w1);
+    mfma8(a1, w1);
   }
 
   // ---- epilogue: bias, round once, transpose through LDS, 128-bit row stores.
   // Lane l of a 32x32 result tile holds column l%32 and rows 8*(e/4) + 4*(l/32) + e%4, e = 0..15.
-  // Each wave owns a [128 rows][128 cols] fp16 image (row pitch 272 B so that the two half-waves,
-  // four rows apart, use different banks).  Neighbouring lanes swap one value so that every lane
-  // writes a 32-bit pair; the image is then read back 16 bytes per lane, 16 lanes per row.
+  // Each wave owns a [128 rows][64 cols] fp16 image (row pitch 144 B).  Neighbouring lanes swap one value
+  // so that every lane writes a 32-bit pair; the image is then read back 16 bytes per lane, 8 lanes per row.
   if (g.partial) {  // split-K: raw fp32 partial sums, lanes of a half-wave write 128 contiguous bytes
     float* pz = g.partial + (int64_t)blockIdx.y * g.m * g.n;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int64_t col = col0 + wn * 128 + j * 32 + frow;
+    for (int j = 0; j < 2; ++j) {
+      const int64_t col = col0 + wn * WN + j * 32 + frow;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const int64_t row = row0 + wm * 128 + i * 32 + 8 * (e >> 2) + 4 * fhalf + (e & 3);
+          const int64_t row = row0 + wm * WM + i * 32 + 8 * (e >> 2) + 4 * fhalf + (e & 3);
           if (row < g.m) pz[row * g.n + col] = acc[i][j][e];
         }
     }
@@ -244,11 +250,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   char* img = lds + wave * kEpiWaveBytes;
   const bool odd = lane & 1;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int col = j * 32 + frow;  // column inside the wave's 128-column strip
+  for (int j = 0; j < 2; ++j) {
+    const int col = j * 32 + frow;  // column inside the wave's 64-column strip
     float bv = 0.f;
     if (g.bias) {
-      const uint16_t bb = ((const uint16_t*)g.bias)[col0 + wn * 128 + col];
+      const uint16_t bb = ((const uint16_t*)g.bias)[col0 + wn * WN + col];
       bv = BF16 ? __uint_as_float((uint32_t)bb << 16) : (float)__builtin_bit_cast(_Float16, bb);
     }
 #pragma unroll
@@ -269,21 +275,21 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   }
   // same wave wrote and reads: only the LDS counter has to drain
   uint16_t* c = (uint16_t*)g.c;
-  const int rrow = lane >> 4, rchunk = lane & 15;
+  const int rrow = lane >> 3, rchunk = lane & 7;
 #pragma unroll 4
-  for (int it = 0; it < 32; ++it) {
-    const int lr = it * 4 + rrow;
+  for (int it = 0; it < WM / 8; ++it) {
+    const int lr = it * 8 + rrow;
     const u32x4 v = *(const u32x4*)(img + lr * kEpiPitch + rchunk * 16);
-    int64_t row = row0 + wm * 128 + lr;
+    int64_t row = row0 + wm * WM + lr;
     if (row >= g.m) continue;
     if (g.row_map) {
       row = g.row_map[row];
       if (row < 0 || row >= g.row_map_limit) continue;
     }
     if (g.c_aligned16)
-      *(u32x4*)(c + row * g.ldc + col0 + wn * 128 + rchunk * 8) = v;
+      *(u32x4*)(c + row * g.ldc + col0 + wn * WN + rchunk * 8) = v;
     else {
-      uint32_t* d = (uint32_t*)(c + row * g.ldc + col0 + wn * 128 + rchunk * 8);
+      uint32_t* d = (uint32_t*)(c + row * g.ldc + col0 + wn * WN + rchunk * 8);
       d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
     }
   }
