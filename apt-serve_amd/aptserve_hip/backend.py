@@ -91,20 +91,32 @@ class HybridAttentionImpl:
     def forward(self, query, key, value, kv_cache, shared_cache, attn_metadata: HybridAttentionMetadata,
                 kv_scale: float = 1.0) -> torch.Tensor:
         """``query [tokens, H*D]``, ``key``/``value [rows, H*D]`` (rows = tokens, or the 'tot' rows of a
-        decode batch with hidden-cached sequences) -> ``[tokens, H*D]``."""
+        decode batch with hidden-cached sequences) -> ``[tokens, H*D]``.
+
+        ``key = value = None`` (decode batches only): the caller has already put this step's K/V
+        into the caches (``ops.kv_reproject_to_cache``), only the attention runs."""
         assert kv_scale == 1.0, "kv_scale is not supported"            # :312
         md = attn_metadata
         num_tokens, hidden_size = query.shape
         H, D = self.num_heads, self.head_size
         query = query.view(-1, H, D)
-        key = key.view(-1, H, D)
-        value = value.view(-1, H, D)
         n_hidden, n_prefill, n_decode = md.num_hidden_cache_tokens, md.num_prefill_tokens, md.num_decode_tokens
-        if n_hidden == 0:
-            assert key.shape[0] == n_prefill + n_decode and value.shape[0] == n_prefill + n_decode
+        written = key is None
+        if written:
+            assert value is None and n_prefill == 0 and kv_cache is not None and not self.literal
+        else:
+            key = key.view(-1, H, D)
+            value = value.view(-1, H, D)
+            if n_hidden == 0:
+                assert key.shape[0] == n_prefill + n_decode and value.shape[0] == n_prefill + n_decode
 
         mixed = False
-        if kv_cache is not None:
+        if written:
+            key_cache, value_cache = kv_cache[0], kv_cache[1]
+            if n_hidden != 0:
+                shared_k, shared_v = shared_cache[0], shared_cache[1]
+                mixed = md.num_tot_tokens != md.slot_mapping_shared.numel()
+        elif kv_cache is not None:
             key_cache, value_cache = kv_cache[0], kv_cache[1]
             if n_hidden == 0:                                                       # :334-345
                 ops.reshape_and_cache_flash(key, value, key_cache, value_cache, md.slot_mapping,
@@ -160,16 +172,23 @@ class HybridOPTAttention:
     ``fused=False`` issues the reference's operator sequence (``hidden_to_cache``,
     ``torch.zeros`` holder, index_put, ``cache_to_hidden``); ``fused=True`` replaces it by
     one ``gather_hidden_rows`` launch into an uninitialised holder.  Results are identical.
+
+    ``fuse_kv_write=True`` (with ``fused`` and not ``literal``) lets the K/V re-projection write
+    its rows straight into the cache slots (``ops.kv_reproject_to_cache``): no ``[T, 2*Hd]``
+    intermediate and no ``mixed_kv_to_cache`` pass.  Results are identical again: the same
+    values are rounded once and land in the same slots.
     """
 
     def __init__(self, embed_dim: int, num_heads: int, qkv_weight, qkv_bias, out_weight, out_bias, *,
-                 fused: bool = True, literal: bool = False, prefill_attention: Optional[Callable] = None) -> None:
+                 fused: bool = True, literal: bool = False, prefill_attention: Optional[Callable] = None,
+                 fuse_kv_write: bool = True) -> None:
         self.embed_dim, self.num_heads = embed_dim, num_heads
         self.head_dim = embed_dim // num_heads
         self.scaling = self.head_dim ** -0.5
         self.qkv_proj = QKVLinear(qkv_weight, qkv_bias)
         self.out_weight, self.out_bias = out_weight, out_bias
         self.fused = fused
+        self.fuse_kv_write = fuse_kv_write and fused and not literal
         self.attn = HybridAttentionImpl(num_heads, self.head_dim, self.scaling, literal=literal,
                                         prefill_attention=prefill_attention)
 
@@ -190,8 +209,16 @@ class HybridOPTAttention:
                     holder[md.hidden_holder_upd] = hidden_states
                     ops.cache_to_hidden(holder, kv_cache, md.slot_mapping, md.hidden_cache_use_tot)
                 q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
-                kv, _ = self.qkv_proj(holder, q_only=False, kv_only=True)
-                k, v = kv.chunk(chunks=2, dim=-1)
+                if (self.fuse_kv_write and md.kv_dest is not None and kv_cache is not None
+                        and kv_cache.dtype == holder.dtype):
+                    w, b = self.qkv_proj.weight, self.qkv_proj.bias
+                    s = w.shape[0] // 3
+                    ops.kv_reproject_to_cache(holder, w[s:], None if b is None else b[s:], shared_cache[0],
+                                              shared_cache[1], kv_cache[0], kv_cache[1], md.kv_dest)
+                    k = v = None
+                else:
+                    kv, _ = self.qkv_proj(holder, q_only=False, kv_only=True)
+                    k, v = kv.chunk(chunks=2, dim=-1)
             else:                                                                   # :125-127
                 ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
                                     md.hidden_cache_store_tot)

@@ -432,6 +432,56 @@ def kv_reproject(x, w_kv, b_kv=None, out=None):
     return linear_nt(x, w_kv, b_kv, out=out)
 
 
+def kv_reproject_to_cache(x, w_kv, b_kv, ws_k_cache, ws_v_cache, k_cache, v_cache, kv_dest, workspace=None,
+                          split_k: bool = True) -> None:
+    """K/V re-projection whose epilogue writes every row straight into its ``[blocks, BS, H, D]``
+    cache slot; replaces the ``kv_only`` projection, the ``chunk`` and ``mixed_kv_to_cache``
+    (additional_designs/model_executor/models/aptserve_opt.py:123-124 and
+    additional_designs/attention/backends/aptserve_flash_attn.py:359-373) without materialising
+    ``[T, 2*Hd]``.  ``kv_dest[t] >= 0``: slot of the workspace caches; ``<= -2``: slot
+    ``-(kv_dest[t]+2)`` of the private caches; ``-1``: skipped.  Either cache pair may be ``None``
+    when no row goes there."""
+    dev = x.device
+    _check_data("x", x, dev)
+    _check_data("w_kv", w_kv, dev)
+    _need(x.dim() == 2 and w_kv.dim() == 2 and x.size(1) == w_kv.size(1), "x [T,K] and w_kv [2*Hd,K] expected")
+    _need(x.dtype == w_kv.dtype and x.dtype in (torch.float16, torch.bfloat16), "f16 or bf16 operands expected")
+    T, K = x.shape
+    _need(w_kv.size(0) % 2 == 0, "w_kv must stack the K and V projections")
+    Hd = w_kv.size(0) // 2
+    if b_kv is not None:
+        _check_data("b_kv", b_kv, dev)
+        _need(b_kv.dim() == 1 and b_kv.numel() == 2 * Hd and b_kv.dtype == x.dtype and b_kv.is_contiguous(),
+              "b_kv must be a contiguous [2*Hd] vector of the operand dtype")
+    _check_index("kv_dest", kv_dest, dev)
+    _need(kv_dest.numel() == T, "one destination per row expected")
+    slots = [0, 0]
+    stride = None
+    for i, (kc, vc, nm) in enumerate(((ws_k_cache, ws_v_cache, "workspace"), (k_cache, v_cache, "private"))):
+        _need((kc is None) == (vc is None), f"{nm} K and V caches must be given together")
+        if kc is None:
+            continue
+        for c in (kc, vc):
+            _check_data(f"{nm} cache", c, dev)
+            _need(c.dim() == 4 and c.is_contiguous() and c.dtype == x.dtype and c.size(2) * c.size(3) == Hd,
+                  f"{nm} caches must be contiguous [blocks, BS, H, D] of the operand dtype with H*D = Hd")
+        _need(kc.shape == vc.shape, f"{nm} K and V caches differ in shape")
+        slots[i] = kc.size(0) * kc.size(1)
+        stride = Hd
+    _need(stride is not None, "no destination cache given")
+    lib = _lib.load()
+    need = lib.aps_linear_nt_workspace_bytes(T, 2 * Hd, K) if split_k else 0
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)     # scratch is host-side plumbing
+    with torch.cuda.device(dev):
+        st = lib.aps_kv_reproject_to_cache(
+            x.data_ptr() if T else None, w_kv.data_ptr(), None if b_kv is None else b_kv.data_ptr(),
+            _ptr(ws_k_cache), _ptr(ws_v_cache), _ptr(k_cache), _ptr(v_cache), _ptr(kv_dest), T, Hd, K, x.stride(0),
+            w_kv.stride(0), stride, slots[0], slots[1], _DTYPE_CODE[x.dtype], workspace.data_ptr() if need else None,
+            workspace.numel() * workspace.element_size() if need else 0, _stream(x))
+    _lib.check(st, "kv_reproject_to_cache")
+
+
 # ------------------------------------------------------------------ prompt attention
 
 def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=None, max_seqlen_k=None,

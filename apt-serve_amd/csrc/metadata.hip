@@ -58,7 +58,7 @@ struct MetaArgs {
   int64_t* slot_mapping; int64_t* slot_mapping_shared;
   int64_t* hidden_cache_use_tot; int64_t* kv_cache_use_tot;
   int64_t* hidden_cache_use_input; int64_t* hidden_cache_store_tot;
-  int64_t* hidden_holder_upd; int64_t* hidden_holder_pull; int64_t* holder_src;
+  int64_t* hidden_holder_upd; int64_t* hidden_holder_pull; int64_t* holder_src; int64_t* kv_dest;
   int32_t* block_tables_out; int64_t out_stride; int out_width;
   int32_t* seq_start_loc; int32_t* query_start_loc; int32_t* context_lens_out; int64_t* input_positions;
   int64_t* totals;
@@ -95,8 +95,10 @@ __global__ __launch_bounds__(kThreads) void decode_metadata_kernel(const MetaArg
         // context rows come from their slot (padding: a value below every -(b+1)), the newest row from input b
         if (a.holder_src) a.holder_src[row0 + j] = (j == L - 1) ? -(int64_t)(b + 1) : (slot >= 0 ? slot : INT64_MIN);
       }
+      const int64_t shared_slot = slot_of(bts, a.shared_width, j, a.block_size);
+      if (a.kv_dest && row0 + j < a.cap_rows) a.kv_dest[row0 + j] = shared_slot >= 0 ? shared_slot : -1;
       if (h0 + j < a.cap_hidden_rows) {
-        a.slot_mapping_shared[h0 + j] = slot_of(bts, a.shared_width, j, a.block_size);
+        a.slot_mapping_shared[h0 + j] = shared_slot;
         a.hidden_cache_use_tot[h0 + j] = row0 + j;
       }
       if (j < L - 1 && pull0 + j < a.cap_rows - a.batch) a.hidden_holder_pull[pull0 + j] = row0 + j;
@@ -110,8 +112,10 @@ __global__ __launch_bounds__(kThreads) void decode_metadata_kernel(const MetaArg
     }
   } else if (threadIdx.x == 0) {
     if (row0 < a.cap_rows) {
-      a.slot_mapping[row0] = L > 0 ? slot_of(bt, a.table_width, L - 1, a.block_size) : -1;
+      const int64_t slot = L > 0 ? slot_of(bt, a.table_width, L - 1, a.block_size) : -1;
+      a.slot_mapping[row0] = slot;
       if (a.holder_src) a.holder_src[row0] = -(int64_t)(b + 1);
+      if (a.kv_dest) a.kv_dest[row0] = slot >= 0 ? -(slot + 2) : -1;
     }
     const int64_t kv_rank = b - pre.hidden_seqs;
     if (kv_rank < a.cap_kv) a.kv_cache_use_tot[kv_rank] = row0;
@@ -196,8 +200,8 @@ int aps_build_decode_metadata(const int32_t* seq_lens, const int32_t* use_hidden
                               int64_t* slot_mapping, int64_t* slot_mapping_shared, int64_t* hidden_cache_use_tot,
                               int64_t* kv_cache_use_tot, int64_t* hidden_cache_use_input,
                               int64_t* hidden_cache_store_tot, int64_t* hidden_holder_upd,
-                              int64_t* hidden_holder_pull, int64_t* holder_src, int64_t cap_rows,
-                              int64_t cap_hidden_rows,
+                              int64_t* hidden_holder_pull, int64_t* holder_src, int64_t* kv_dest,
+                              int64_t cap_rows, int64_t cap_hidden_rows,
                               int64_t cap_hidden_seqs, int64_t cap_kv_seqs, int32_t* block_tables_out,
                               int64_t out_stride, int64_t out_width, int32_t* seq_start_loc,
                               int32_t* query_start_loc, int32_t* context_lens, int64_t* input_positions,
@@ -225,7 +229,7 @@ int aps_build_decode_metadata(const int32_t* seq_lens, const int32_t* use_hidden
   a.slot_mapping = slot_mapping; a.slot_mapping_shared = slot_mapping_shared;
   a.hidden_cache_use_tot = hidden_cache_use_tot; a.kv_cache_use_tot = kv_cache_use_tot;
   a.hidden_cache_use_input = hidden_cache_use_input; a.hidden_cache_store_tot = hidden_cache_store_tot;
-  a.hidden_holder_upd = hidden_holder_upd; a.hidden_holder_pull = hidden_holder_pull; a.holder_src = holder_src;
+  a.hidden_holder_upd = hidden_holder_upd; a.hidden_holder_pull = hidden_holder_pull; a.holder_src = holder_src; a.kv_dest = kv_dest;
   a.block_tables_out = block_tables_out; a.out_stride = out_stride; a.out_width = (int)out_width;
   a.seq_start_loc = seq_start_loc; a.query_start_loc = query_start_loc; a.context_lens_out = context_lens;
   a.input_positions = input_positions; a.totals = totals;

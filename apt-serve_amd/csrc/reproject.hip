@@ -57,15 +57,42 @@ constexpr int kLdsBytes =
 constexpr int kNumXcd = 8;
 constexpr int kGroupM = 8;
 
+// Where a result row goes.  Plain: row t of C is row t (or map[t], negative skipped) of base[0], ld elements
+// apart.  Cache mode (n_split > 0): columns below n_split are the K part of the row and columns from n_split
+// on its V part; map[t] >= 0 is a slot of the workspace caches base[0] (K) / base[1] (V), map[t] <= -2 is
+// slot -(map[t]+2) of the private caches base[2] / base[3], -1 is skipped; a slot is ld elements.
+struct OutMap {
+  char* base[4];
+  int64_t ld;
+  int64_t n_split;
+  const int64_t* map;
+  int64_t limit0, limit1;  // rows (plain) or workspace slots; private slots
+  int aligned16;           // every base and the pitch allow 128-bit stores
+};
+
+// Start of result row `row` for the column half `half`; nullptr when the row is skipped.
+__device__ __forceinline__ uint16_t* out_row(const OutMap& o, int64_t row, int half) {
+  int64_t r = row;
+  char* base = half ? o.base[1] : o.base[0];
+  if (o.map) {
+    r = o.map[row];
+    if (o.n_split && r <= -2) {
+      r = -(r + 2);
+      if (r >= o.limit1) return nullptr;
+      base = half ? o.base[3] : o.base[2];
+    } else if (r < 0 || r >= o.limit0) {
+      return nullptr;
+    }
+  }
+  return base ? (uint16_t*)base + r * o.ld : nullptr;
+}
+
 struct GemmArgs {
-  const char* a; const char* w; const void* bias; char* c;
-  int64_t lda_b, ldw_b, ldc;  // lda/ldw in bytes, ldc in elements
+  const char* a; const char* w; const void* bias;
+  int64_t lda_b, ldw_b;  // bytes
   int64_t m, n, k;
   int tiles_m, tiles_n;
-  // optional row scatter of the epilogue: row t of C goes to row_map[t] (rows of ldc elements), <0 skipped
-  const int64_t* row_map;
-  int64_t row_map_limit;
-  int c_aligned16;  // out pointer and row pitch allow 128-bit stores
+  OutMap out;
   // split-K (small M): workgroup (tile, z) handles k-tiles [z*kt_per_split, ...) and stores its fp32
   // partial tile to partial[z][m][n]; a second kernel adds the splits and the bias
   float* partial;
@@ -274,22 +301,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
   }
   // same wave wrote and reads: only the LDS counter has to drain
-  uint16_t* c = (uint16_t*)g.c;
+  const int half = (g.out.n_split && col0 >= g.out.n_split) ? 1 : 0;  // a tile never straddles the split
+  const int64_t ocol = col0 - (half ? g.out.n_split : 0) + wn * WN;
   const int rrow = lane >> 3, rchunk = lane & 7;
 #pragma unroll 4
   for (int it = 0; it < WM / 8; ++it) {
     const int lr = it * 8 + rrow;
     const u32x4 v = *(const u32x4*)(img + lr * kEpiPitch + rchunk * 16);
-    int64_t row = row0 + wm * WM + lr;
+    const int64_t row = row0 + wm * WM + lr;
     if (row >= g.m) continue;
-    if (g.row_map) {
-      row = g.row_map[row];
-      if (row < 0 || row >= g.row_map_limit) continue;
-    }
-    if (g.c_aligned16)
-      *(u32x4*)(c + row * g.ldc + col0 + wn * WN + rchunk * 8) = v;
+    uint16_t* dst = out_row(g.out, row, half);
+    if (!dst) continue;
+    dst += ocol + rchunk * 8;
+    if (g.out.aligned16)
+      *(u32x4*)dst = v;
     else {
-      uint32_t* d = (uint32_t*)(c + row * g.ldc + col0 + wn * WN + rchunk * 8);
+      uint32_t* d = (uint32_t*)dst;
       d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
     }
   }
@@ -298,9 +325,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 // out[m][n] = sum_z partial[z][m][n] + bias[n], rounded once; 4 columns per thread
 template <bool BF16>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, const void* bias,
-                                                            uint16_t* out, int64_t m, int64_t n, int64_t ldc,
-                                                            int splits, const int64_t* row_map,
-                                                            int64_t row_map_limit) {
+                                                            const OutMap out, int64_t m, int64_t n, int splits) {
   const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (idx >= m * n) return;
   const int64_t row = idx / n, col = idx - row * n;
@@ -314,12 +339,10 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     auto cv = [](uint16_t v) { return BF16 ? __uint_as_float((uint32_t)v << 16) : (float)__builtin_bit_cast(_Float16, v); };
     s.x += cv(b[0]); s.y += cv(b[1]); s.z += cv(b[2]); s.w += cv(b[3]);
   }
-  int64_t orow = row;
-  if (row_map) {
-    orow = row_map[row];
-    if (orow < 0 || orow >= row_map_limit) return;
-  }
-  uint16_t* o = out + orow * ldc + col;
+  const int half = (out.n_split && col >= out.n_split) ? 1 : 0;
+  uint16_t* o = out_row(out, row, half);
+  if (!o) return;
+  o += col - (half ? out.n_split : 0);
   if (BF16) { o[0] = f32_to_bf16_bits(s.x); o[1] = f32_to_bf16_bits(s.y); o[2] = f32_to_bf16_bits(s.z); o[3] = f32_to_bf16_bits(s.w); }
   else { o[0] = f32_to_f16_bits(s.x); o[1] = f32_to_f16_bits(s.y); o[2] = f32_to_f16_bits(s.z); o[3] = f32_to_f16_bits(s.w); }
 }
@@ -348,28 +371,23 @@ int64_t aps_linear_nt_workspace_bytes(int64_t m, int64_t n, int64_t k) {
   return s > 1 ? (int64_t)s * m * n * 4 : 0;
 }
 
-int aps_linear_nt(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n, int64_t k,
-                  int64_t x_stride, int64_t w_stride, int64_t out_stride, const int64_t* out_row_map,
-                  int64_t out_rows, int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream) {
-  if (m < 0 || n <= 0 || k <= 0) return APS_ERR_INVALID_ARG;
-  if (m == 0) return APS_OK;
-  if (!x || !weight || !out) return APS_ERR_INVALID_ARG;
+static int launch_gemm(const void* x, const void* weight, const void* bias, const OutMap& om, int64_t m, int64_t n,
+                       int64_t k, int64_t x_stride, int64_t w_stride, int dtype, void* workspace,
+                       int64_t workspace_bytes, aps_stream_t stream) {
   if (dtype != APS_F16 && dtype != APS_BF16) return APS_ERR_UNSUPPORTED;
   if (n % BN != 0 || k % BK != 0) return APS_ERR_UNSUPPORTED;
-  if (x_stride < k || w_stride < k || out_stride < n) return APS_ERR_INVALID_ARG;
+  if (x_stride < k || w_stride < k) return APS_ERR_INVALID_ARG;
   if (common_vec_bytes({addr(x), addr(weight), (uint64_t)x_stride * 2, (uint64_t)w_stride * 2}) != 16)
     return APS_ERR_UNSUPPORTED;
-  if (common_vec_bytes({addr(out), (uint64_t)out_stride * 2}) < 4) return APS_ERR_UNSUPPORTED;
   // one tile's rows must be addressable with 32-bit byte offsets
   if ((int64_t)BM * x_stride * 2 >= ((int64_t)1 << 31) || (int64_t)BN * w_stride * 2 >= ((int64_t)1 << 31))
     return APS_ERR_UNSUPPORTED;
   GemmArgs g{};
-  g.a = (const char*)x; g.w = (const char*)weight; g.bias = bias; g.c = (char*)out;
-  g.lda_b = x_stride * 2; g.ldw_b = w_stride * 2; g.ldc = out_stride;
+  g.a = (const char*)x; g.w = (const char*)weight; g.bias = bias;
+  g.lda_b = x_stride * 2; g.ldw_b = w_stride * 2;
   g.m = m; g.n = n; g.k = k;
   g.tiles_m = (int)((m + BM - 1) / BM); g.tiles_n = (int)(n / BN);
-  g.row_map = out_row_map; g.row_map_limit = out_rows;
-  g.c_aligned16 = common_vec_bytes({addr(out), (uint64_t)out_stride * 2}) == 16;
+  g.out = om;
   const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
   if (total >= ((int64_t)1 << 30)) return APS_ERR_UNSUPPORTED;
   const int64_t per_xcd = (total + kNumXcd - 1) / kNumXcd;
@@ -397,12 +415,50 @@ int aps_linear_nt(const void* x, const void* weight, const void* bias, void* out
   const int64_t quads = (m * n + 3) / 4;
   const dim3 rgrid((unsigned)((quads + 255) / 256));
   if (dtype == APS_BF16)
-    hipLaunchKernelGGL(splitk_reduce_kernel<true>, rgrid, dim3(256), 0, s, (const float*)workspace, bias,
-                       (uint16_t*)out, m, n, out_stride, splits, out_row_map, out_rows);
+    hipLaunchKernelGGL(splitk_reduce_kernel<true>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m, n,
+                       splits);
   else
-    hipLaunchKernelGGL(splitk_reduce_kernel<false>, rgrid, dim3(256), 0, s, (const float*)workspace, bias,
-                       (uint16_t*)out, m, n, out_stride, splits, out_row_map, out_rows);
+    hipLaunchKernelGGL(splitk_reduce_kernel<false>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m, n,
+                       splits);
   return launch_status();
+}
+
+int aps_linear_nt(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n, int64_t k,
+                  int64_t x_stride, int64_t w_stride, int64_t out_stride, const int64_t* out_row_map,
+                  int64_t out_rows, int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream) {
+  if (m < 0 || n <= 0 || k <= 0) return APS_ERR_INVALID_ARG;
+  if (m == 0) return APS_OK;
+  if (!x || !weight || !out) return APS_ERR_INVALID_ARG;
+  if (out_stride < n) return APS_ERR_INVALID_ARG;
+  const int align = common_vec_bytes({addr(out), (uint64_t)out_stride * 2});
+  if (align < 4) return APS_ERR_UNSUPPORTED;
+  OutMap om{};
+  om.base[0] = (char*)out; om.ld = out_stride; om.n_split = 0;
+  om.map = out_row_map; om.limit0 = out_rows; om.aligned16 = align == 16;
+  return launch_gemm(x, weight, bias, om, m, n, k, x_stride, w_stride, dtype, workspace, workspace_bytes, stream);
+}
+
+int aps_kv_reproject_to_cache(const void* x, const void* w_kv, const void* b_kv, void* ws_k_cache, void* ws_v_cache,
+                              void* k_cache, void* v_cache, const int64_t* kv_dest, int64_t m, int64_t hidden_size,
+                              int64_t k, int64_t x_stride, int64_t w_stride, int64_t slot_stride, int64_t ws_slots,
+                              int64_t cache_slots, int dtype, void* workspace, int64_t workspace_bytes,
+                              aps_stream_t stream) {
+  if (m < 0 || hidden_size <= 0 || k <= 0 || ws_slots < 0 || cache_slots < 0) return APS_ERR_INVALID_ARG;
+  if (m == 0) return APS_OK;
+  if (!x || !w_kv || !kv_dest) return APS_ERR_INVALID_ARG;
+  if ((ws_slots && (!ws_k_cache || !ws_v_cache)) || (cache_slots && (!k_cache || !v_cache))) return APS_ERR_INVALID_ARG;
+  if (slot_stride < hidden_size) return APS_ERR_INVALID_ARG;
+  if (hidden_size % BN != 0) return APS_ERR_UNSUPPORTED;  // a column tile must not straddle the K | V boundary
+  const int align = common_vec_bytes({addr(ws_k_cache), addr(ws_v_cache), addr(k_cache), addr(v_cache),
+                                      (uint64_t)slot_stride * 2});
+  if (align < 4) return APS_ERR_UNSUPPORTED;
+  OutMap om{};
+  om.base[0] = (char*)ws_k_cache; om.base[1] = (char*)ws_v_cache;
+  om.base[2] = (char*)k_cache; om.base[3] = (char*)v_cache;
+  om.ld = slot_stride; om.n_split = hidden_size; om.map = kv_dest;
+  om.limit0 = ws_slots; om.limit1 = cache_slots; om.aligned16 = align == 16;
+  return launch_gemm(x, w_kv, b_kv, om, m, 2 * hidden_size, k, x_stride, w_stride, dtype, workspace, workspace_bytes,
+                     stream);
 }
 
 }  // extern "C"

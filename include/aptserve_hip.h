@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define APS_ABI_VERSION 1
+#define APS_ABI_VERSION 2
 
 typedef void* aps_stream_t; /* a hipStream_t; NULL = the null stream */
 
@@ -250,6 +250,9 @@ int aps_varlen_prefill_attention(void* out, const void* q, const void* k,
  *   hidden_cache_store_tot   their newest rows
  *   holder_src[row]          (nullable, not in the reference) resolved source of the row for
  *                            aps_gather_hidden_rows: slot, -(b+1) for the newest row, INT64_MIN for padding
+ *   kv_dest[row]             (nullable, not in the reference) where the row's re-projected K/V go, for
+ *                            aps_kv_reproject_to_cache: shared slot (hidden rows), -(private slot + 2)
+ *                            (the new token of a K/V sequence), -1 for padding
  *   block_tables_out[b,:]    shared table for hidden sequences, private otherwise (:415-418)
  *   seq_start_loc / query_start_loc int32 cumulative sums with leading 0;
  *   context_lens = seq_len-1; input_positions = seq_len-1. */
@@ -261,8 +264,8 @@ int aps_build_decode_metadata(
     int64_t* slot_mapping_shared, int64_t* hidden_cache_use_tot,
     int64_t* kv_cache_use_tot, int64_t* hidden_cache_use_input,
     int64_t* hidden_cache_store_tot, int64_t* hidden_holder_upd,
-    int64_t* hidden_holder_pull, int64_t* holder_src, int64_t cap_rows,
-    int64_t cap_hidden_rows,
+    int64_t* hidden_holder_pull, int64_t* holder_src, int64_t* kv_dest,
+    int64_t cap_rows, int64_t cap_hidden_rows,
     int64_t cap_hidden_seqs, int64_t cap_kv_seqs, int32_t* block_tables_out,
     int64_t out_stride, int64_t out_width, int32_t* seq_start_loc,
     int32_t* query_start_loc, int32_t* context_lens, int64_t* input_positions,
@@ -310,6 +313,28 @@ int aps_linear_nt(const void* x, const void* weight, const void* bias,
                   const int64_t* out_row_map, int64_t out_rows, int dtype,
                   void* workspace, int64_t workspace_bytes,
                   aps_stream_t stream);
+
+/* K/V re-projection with the cache write fused into the epilogue: one pass that
+ * replaces the kv_only projection (model_executor/models/aptserve_opt.py:123-124),
+ * the chunk into key/value, and ranges (A) and (C) of mixed_kv_to_cache
+ * (mixed_cache_kernels/mixed_cache.cu:56-116, called at
+ * attention/backends/aptserve_flash_attn.py:359-373); the mirror range (B) has
+ * no reader and is not written.
+ *   kv[t, :] = x[t, :] * w_kv[2*hidden_size, k]^T + b_kv;  K = kv[t, :hidden_size], V = the rest
+ *   kv_dest[t] >= 0   K -> ws_k_cache slot kv_dest[t], V -> ws_v_cache (slots < ws_slots)
+ *   kv_dest[t] <= -2  K -> k_cache slot -(kv_dest[t]+2), V -> v_cache (slots < cache_slots)
+ *   kv_dest[t] == -1 or out of range: row not stored
+ * A slot is slot_stride elements (= heads*head_size of a [blocks, BS, H, D]
+ * cache); hidden_size must be a multiple of 256, k of 64.  The intermediate
+ * [m, 2*hidden_size] matrix is never materialised.  workspace as for
+ * aps_linear_nt with n = 2*hidden_size. */
+int aps_kv_reproject_to_cache(
+    const void* x, const void* w_kv, const void* b_kv, void* ws_k_cache,
+    void* ws_v_cache, void* k_cache, void* v_cache, const int64_t* kv_dest,
+    int64_t m, int64_t hidden_size, int64_t k, int64_t x_stride,
+    int64_t w_stride, int64_t slot_stride, int64_t ws_slots,
+    int64_t cache_slots, int dtype, void* workspace, int64_t workspace_bytes,
+    aps_stream_t stream);
 
 /* Plain device copy of nbytes (16-byte aligned pointers): the known-size
  * kernel that hardware counters of the kernels above are scaled against. */

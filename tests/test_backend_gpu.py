@@ -37,7 +37,7 @@ def close(a, b, tol=6e-3):
 
 
 @pytest.mark.parametrize("frac", [0.0, 0.4, 1.0])
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", [True, "gather-only", False])
 def test_decode_layer_matches_oracle(dev, frac, fused):
     W = weights(0)
     batch = workloads.small_decode_batch(3, 10, 150, frac, N)
@@ -48,7 +48,8 @@ def test_decode_layer_matches_oracle(dev, frac, fused):
     sh = randn((2, 2 * N, BS, H, D), 7)
     ref_kv, ref_sh = kv.clone(), sh.clone()
     ref = OL.opt_attention(hs, ref_kv, ref_sh, ref_md, *W, H)
-    layer = backend.HybridOPTAttention(Hd, H, *(w.to(dev) for w in W), fused=fused)
+    layer = backend.HybridOPTAttention(Hd, H, *(w.to(dev) for w in W), fused=bool(fused),
+                                       fuse_kv_write=fused is True)
     md = metadata.build_from_batch(batch, dev)
     d_kv, d_sh = kv.to(dev), sh.to(dev)
     out = layer(hs.to(dev), d_kv, d_sh, md)
@@ -61,6 +62,24 @@ def test_decode_layer_matches_oracle(dev, frac, fused):
     close(d_sh[:, N:], ref_sh[:, N:])
     # the mirror blocks 0..N-1 are not written by the default data flow
     assert torch.equal(d_sh[:, :N].cpu(), sh[:, :N])
+
+
+@pytest.mark.parametrize("frac", [0.4, 1.0])
+def test_fused_kv_write_is_bit_identical_to_the_operator_sequence(dev, frac):
+    """Projection with the cache write in its epilogue == projection, chunk, mixed_kv_to_cache."""
+    W = weights(1)
+    batch = workloads.small_decode_batch(4, 10, 150, frac, N)
+    hs = randn((len(batch.seq_lens), Hd), 8)
+    kv = randn((2, N, BS, H, D), 9)
+    sh = randn((2, 2 * N, BS, H, D), 10)
+    md = metadata.build_from_batch(batch, dev)
+    res = []
+    for fuse in (True, False):
+        layer = backend.HybridOPTAttention(Hd, H, *(w.to(dev) for w in W), fuse_kv_write=fuse)
+        d_kv, d_sh = kv.to(dev), sh.to(dev)
+        res.append((layer(hs.to(dev), d_kv, d_sh, md).cpu(), d_kv.cpu(), d_sh.cpu()))
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
 
 
 def test_literal_flow_agrees_where_the_reference_is_well_defined(dev):

@@ -24,6 +24,17 @@ def assert_same(md, ref):
         assert got.dtype == ref[f].dtype, (f, got.dtype, ref[f].dtype)
         assert got.shape == ref[f].shape, (f, got.shape, ref[f].shape)
         assert np.array_equal(got, ref[f]), f
+    if md.num_decode_tokens:
+        # the two resolved per-row vectors this implementation adds, restated from the reference's fields
+        src = ref["slot_mapping"].copy()
+        src[src < 0] = np.iinfo(np.int64).min
+        src[ref["hidden_holder_upd"]] = -(np.arange(len(ref["hidden_holder_upd"])) + 1)
+        assert np.array_equal(md.holder_src.cpu().numpy(), src)
+        dest = np.full(ref["num_tot_tokens"], -1, dtype=np.int64)
+        dest[ref["hidden_cache_use_tot"]] = ref["slot_mapping_shared"]
+        private = ref["slot_mapping"][ref["kv_cache_use_tot"]]
+        dest[ref["kv_cache_use_tot"]] = np.where(private >= 0, -(private + 2), -1)
+        assert np.array_equal(md.kv_dest.cpu().numpy(), dest)
 
 
 @pytest.mark.parametrize("seed", range(5))

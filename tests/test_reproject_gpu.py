@@ -97,6 +97,54 @@ def test_strided_activations_and_row_scatter_epilogue(dev):
     assert (dest[untouched] == 7).all()
 
 
+@pytest.mark.parametrize("T", [5, 300, 1100])          # split-K (few tiles) and the one-pass kernel
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_kv_reproject_into_cache_slots(dev, T, dtype):
+    """The fused epilogue puts K and V of every row into its slot: equal, bit for bit, to the
+    plain projection followed by an index_put; rows with -1 or an out-of-range slot are dropped;
+    every other slot keeps its content."""
+    H, D, BS, nblk = 4, 64, 16, 80
+    Hd = H * D
+    rng = np.random.default_rng(T)
+    x = randn((T, Hd), 1, dtype)
+    w = (randn((2 * Hd, Hd), 2) * 0.05).to(dtype)
+    b = randn((2 * Hd,), 3, dtype)
+    ws_slots, priv_slots = 2 * nblk * BS, nblk * BS
+    # a random third of the rows go to the private caches, the rest to the workspace; slots are distinct
+    to_priv = rng.random(T) < 0.33
+    dest = np.empty(T, dtype=np.int64)
+    dest[to_priv] = -(rng.permutation(priv_slots)[:to_priv.sum()] + 2)
+    dest[~to_priv] = rng.permutation(ws_slots)[:(~to_priv).sum()]
+    dropped = rng.choice(T, size=min(3, T - 1), replace=False)
+    dest[dropped[0]] = -1
+    if len(dropped) > 1:
+        dest[dropped[1]] = ws_slots + 5              # beyond the workspace
+    if len(dropped) > 2:
+        dest[dropped[2]] = -(priv_slots + 9 + 2)     # beyond the private cache
+    caches = [torch.full((n, BS, H, D), 3.0, dtype=dtype, device=dev) for n in (2 * nblk, 2 * nblk, nblk, nblk)]
+    ops.kv_reproject_to_cache(x.to(dev), w.to(dev), b.to(dev), *caches, torch.from_numpy(dest).to(dev))
+    plain = ops.linear_nt(x.to(dev), w.to(dev), b.to(dev)).cpu()
+    check(plain, OR._linear_fp32(x, w, b), dtype)
+    expect = [torch.full((n * BS, Hd), 3.0, dtype=dtype) for n in (2 * nblk, 2 * nblk, nblk, nblk)]
+    for t in range(T):
+        d = int(dest[t])
+        if 0 <= d < ws_slots:
+            expect[0][d], expect[1][d] = plain[t, :Hd], plain[t, Hd:]
+        elif d <= -2 and -(d + 2) < priv_slots:
+            expect[2][-(d + 2)], expect[3][-(d + 2)] = plain[t, :Hd], plain[t, Hd:]
+    for got, exp in zip(caches, expect):
+        assert torch.equal(got.cpu().view(-1, Hd), exp)
+    # one cache pair may be absent when no row goes there
+    only_ws = np.where(dest >= 0, dest, -1)
+    c2 = [torch.full((2 * nblk, BS, H, D), 3.0, dtype=dtype, device=dev) for _ in range(2)]
+    ops.kv_reproject_to_cache(x.to(dev), w.to(dev), b.to(dev), c2[0], c2[1], None, None,
+                              torch.from_numpy(only_ws).to(dev))
+    assert torch.equal(c2[0].cpu(), caches[0].cpu()) and torch.equal(c2[1].cpu(), caches[1].cpu())
+    with pytest.raises(ValueError):
+        ops.kv_reproject_to_cache(x.to(dev), w.to(dev), b.to(dev), None, None, None, None,
+                                  torch.from_numpy(dest).to(dev))
+
+
 def test_unsupported_shapes_raise(dev):
     x = torch.zeros(4, 64, dtype=torch.float16, device=dev)
     with pytest.raises(RuntimeError):
