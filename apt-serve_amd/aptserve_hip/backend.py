@@ -89,21 +89,22 @@ class HybridAttentionImpl:
         self.prefill_attention = prefill_attention
 
     def forward(self, query, key, value, kv_cache, shared_cache, attn_metadata: HybridAttentionMetadata,
-                kv_scale: float = 1.0) -> torch.Tensor:
+                kv_scale: float = 1.0, kv_written: bool = False) -> torch.Tensor:
         """``query [tokens, H*D]``, ``key``/``value [rows, H*D]`` (rows = tokens, or the 'tot' rows of a
         decode batch with hidden-cached sequences) -> ``[tokens, H*D]``.
 
-        ``key = value = None`` (decode batches only): the caller has already put this step's K/V
-        into the caches (``ops.kv_reproject_to_cache``), only the attention runs."""
+        ``kv_written``: the caller has already put this step's K/V into the caches
+        (``ops.kv_reproject_to_cache`` in a decode step, where ``key = value = None`` is then
+        allowed; ``ops.mixed_reshape_and_cache`` in a prompt step), only the attention runs."""
         assert kv_scale == 1.0, "kv_scale is not supported"            # :312
         md = attn_metadata
         num_tokens, hidden_size = query.shape
         H, D = self.num_heads, self.head_size
         query = query.view(-1, H, D)
         n_hidden, n_prefill, n_decode = md.num_hidden_cache_tokens, md.num_prefill_tokens, md.num_decode_tokens
-        written = key is None
-        if written:
-            assert value is None and n_prefill == 0 and kv_cache is not None and not self.literal
+        written = kv_written or key is None
+        if key is None:
+            assert value is None and n_prefill == 0
         else:
             key = key.view(-1, H, D)
             value = value.view(-1, H, D)
@@ -112,8 +113,9 @@ class HybridAttentionImpl:
 
         mixed = False
         if written:
+            assert kv_cache is not None and not self.literal
             key_cache, value_cache = kv_cache[0], kv_cache[1]
-            if n_hidden != 0:
+            if n_hidden != 0 and n_prefill == 0:
                 shared_k, shared_v = shared_cache[0], shared_cache[1]
                 mixed = md.num_tot_tokens != md.slot_mapping_shared.numel()
         elif kv_cache is not None:
@@ -215,10 +217,19 @@ class HybridOPTAttention:
                     s = w.shape[0] // 3
                     ops.kv_reproject_to_cache(holder, w[s:], None if b is None else b[s:], shared_cache[0],
                                               shared_cache[1], kv_cache[0], kv_cache[1], md.kv_dest)
-                    k = v = None
+                    attn_output = self.attn.forward(q, None, None, kv_cache, shared_cache, md, kv_written=True)
+                    return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
                 else:
                     kv, _ = self.qkv_proj(holder, q_only=False, kv_only=True)
                     k, v = kv.chunk(chunks=2, dim=-1)
+            elif (self.fuse_kv_write and md.token_is_hidden is not None and kv_cache is not None
+                  and kv_cache.dtype == hidden_states.dtype):
+                qkv, _ = self.qkv_proj(hidden_states)
+                q, k, v = qkv.chunk(chunks=3, dim=-1)
+                # hidden rows of hidden-cached prompts and K/V rows of the others, one launch
+                ops.mixed_reshape_and_cache(k, v, hidden_states, kv_cache, md.slot_mapping, md.token_is_hidden)
+                attn_output = self.attn.forward(q, k, v, kv_cache, shared_cache, md, kv_written=True)
+                return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
             else:                                                                   # :125-127
                 ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
                                     md.hidden_cache_store_tot)

@@ -58,6 +58,7 @@ class HybridAttentionMetadata:
     block_types: Optional[torch.Tensor] = None      # uint8 [batch, width]: 1 = block read from the K/V workspace
     holder_src: Optional[torch.Tensor] = None       # int64 [num_tot]: resolved source of every holder row
     kv_dest: Optional[torch.Tensor] = None          # int64 [num_tot]: cache slot the row's re-projected K/V go to
+    token_is_hidden: Optional[torch.Tensor] = None  # uint8 [prompt tokens]: 1 = token of a hidden-cached prompt
     _cached_prefill_metadata: Optional["HybridAttentionMetadata"] = None
     _cached_decode_metadata: Optional["HybridAttentionMetadata"] = None
 
@@ -82,7 +83,7 @@ class HybridAttentionMetadata:
                 seq_start_loc=self.seq_start_loc[:self.num_prefills + 1],
                 context_lens_tensor=self.context_lens_tensor[:self.num_prefills],
                 block_tables=self.block_tables[:self.num_prefills], use_cuda_graph=False,
-                input_positions=self.input_positions, block_types=None)
+                input_positions=self.input_positions, block_types=None, token_is_hidden=self.token_is_hidden)
         return self._cached_prefill_metadata
 
     @property
@@ -281,11 +282,13 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
     sizes32 = [B + 1, B + 1, B]
     buf32 = torch.empty(sum(sizes32), **i32)
     seq_start, query_start, ctx = torch.split(buf32, sizes32)
+    token_is_hidden = torch.empty(n_tok, dtype=torch.uint8, device=device)
     with torch.cuda.device(device):
         st = lib.aps_build_prefill_metadata(
             d_lens.data_ptr(), d_ctx_in.data_ptr(), d_hid.data_ptr(), d_bt.data_ptr() if W else None, W, W, B,
             block_size, slot_mapping.data_ptr(), positions.data_ptr(), use_input.data_ptr() if n_ht else None,
-            kv_use.data_ptr() if n_kt else None, n_tok, n_ht, n_kt, seq_start.data_ptr(), query_start.data_ptr(),
+            kv_use.data_ptr() if n_kt else None, token_is_hidden.data_ptr(), n_tok, n_ht, n_kt,
+            seq_start.data_ptr(), query_start.data_ptr(),
             ctx.data_ptr(), totals.data_ptr(), torch.cuda.current_stream(device).cuda_stream)
     _lib.check(st, "build_prefill_metadata")
     if check_totals:
@@ -301,7 +304,8 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
         seq_lens=[int(x) for x in lens], seq_lens_tensor=d_lens, max_query_len=int(qlens.max()),
         max_prefill_seq_len=int(lens.max()), max_decode_seq_len=0, query_start_loc=query_start,
         seq_start_loc=seq_start, context_lens_tensor=ctx,
-        block_tables=torch.empty(B, 0, **i32), use_cuda_graph=False, input_positions=positions, block_types=None)
+        block_tables=torch.empty(B, 0, **i32), use_cuda_graph=False, input_positions=positions, block_types=None,
+        token_is_hidden=token_is_hidden)
 
 
 def build_from_batch(batch, device, **kw) -> HybridAttentionMetadata:

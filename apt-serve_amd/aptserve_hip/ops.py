@@ -228,6 +228,77 @@ def reshape_and_cache_flash(key, value, key_cache, value_cache, slot_mapping, kv
     _lib.check(st, "reshape_and_cache_flash")
 
 
+def mixed_reshape_and_cache(key, value, hidden, kv_cache, slot_mapping, is_hidden, kv_cache_dtype: str = "auto",
+                            k_scale: float = 1.0, v_scale: float = 1.0, hidden_cache=None) -> None:
+    """Cache write of a step whose tokens differ in cache type, one launch.
+
+    Token ``t`` with ``is_hidden[t]`` stores ``hidden[t]`` at slot ``slot_mapping[t]`` of the
+    flattened paged cache (what ``hidden_to_cache`` does for the hidden tokens of a prompt step,
+    additional_designs/model_executor/models/aptserve_opt.py:125-126); every other token stores
+    ``key[t]`` / ``value[t]`` by block (``reshape_and_cache_flash`` over the K/V tokens,
+    additional_designs/attention/backends/aptserve_flash_attn.py:347-355).  ``kv_cache`` is the
+    ``(2, N, BS, H, D)`` cache of the layer.  With ``kv_cache_dtype='fp8'`` the K/V rows are stored
+    as e4m3 codes of ``x / scale`` in the 1-byte ``kv_cache`` and hidden rows go, unquantised, to
+    the separate ``hidden_cache`` (same shape, activation dtype).  ``key``/``value`` or ``hidden``
+    may be ``None`` to store only the other kind."""
+    _need(kv_cache is not None and kv_cache.dim() == 5 and kv_cache.size(0) == 2,
+          "kv_cache must be (2, num_blocks, block_size, heads, head_dim)")
+    dev = kv_cache.device
+    _check_data("kv_cache", kv_cache, dev)
+    _need(kv_cache.is_contiguous(), "kv_cache must be contiguous")
+    _, nblk, bs, heads, head_size = kv_cache.shape
+    width = heads * head_size
+    _need((key is None) == (value is None), "key and value must be given together")
+    _need(key is not None or hidden is not None, "nothing to store")
+    _check_index("slot_mapping", slot_mapping, dev)
+    T = slot_mapping.numel()
+    src_dtype = None
+    if key is not None:
+        for n, t in (("key", key), ("value", value)):
+            _check_data(n, t, dev)
+        key = _as_thd("key", key, heads, head_size)
+        value = _as_thd("value", value, heads, head_size)
+        _need(key.dtype == value.dtype, "K and V dtypes differ")
+        _need(key.size(0) >= T and value.size(0) >= T, "slot_mapping longer than key/value")
+        src_dtype = key.dtype
+    if hidden is not None:
+        _check_data("hidden", hidden, dev)
+        _need(hidden.dim() == 2 and hidden.size(1) == width and hidden.size(0) >= T,
+              "hidden must be [tokens, heads*head_dim]")
+        _need(src_dtype is None or hidden.dtype == src_dtype, "hidden and key dtypes differ")
+        src_dtype = hidden.dtype
+        _need(is_hidden is not None, "hidden rows need the is_hidden mask")
+    _need(src_dtype in (torch.float16, torch.bfloat16, torch.float32), f"unsupported dtype {src_dtype}")
+    if is_hidden is not None:
+        _need(is_hidden.device == dev and is_hidden.dtype in (torch.uint8, torch.bool) and is_hidden.is_contiguous()
+              and is_hidden.numel() == T, "is_hidden must be a contiguous uint8/bool vector, one entry per token")
+    if kv_cache_dtype == "auto":
+        _need(kv_cache.dtype == src_dtype, "kv_cache_dtype='auto' needs cache dtype == activation dtype")
+        hcache = kv_cache if hidden_cache is None else hidden_cache
+    elif kv_cache_dtype in ("fp8", "fp8_e4m3"):
+        _need(kv_cache.element_size() == 1, "fp8 cache must be uint8 / float8_e4m3fn")
+        _need(hidden is None or hidden_cache is not None, "an fp8 K/V cache cannot hold hidden rows: pass hidden_cache")
+        hcache = hidden_cache
+    else:
+        raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
+    hidden_slots = hidden_stride = 0
+    if hidden is not None:
+        _check_data("hidden_cache", hcache, dev)
+        _check_paged(hcache, width)
+        _need(hcache.dtype == src_dtype, "hidden cache dtype differs from the activations")
+        hidden_stride = hcache.stride(2)
+        hidden_slots = hcache.numel() // hidden_stride
+    cache_code = _DTYPE_CODE[kv_cache.dtype] if key is not None else _DTYPE_CODE[src_dtype]
+    with torch.cuda.device(dev):
+        st = _lib.load().aps_mixed_reshape_and_cache(
+            _ptr(key), _ptr(value), _ptr(hidden), kv_cache[0].data_ptr(), kv_cache[1].data_ptr(),
+            None if hidden is None else hcache.data_ptr(), _ptr(slot_mapping), _ptr(is_hidden), T, heads, head_size, bs,
+            0 if key is None else key.stride(0), 0 if key is None else value.stride(0),
+            0 if hidden is None else hidden.stride(0), kv_cache.stride(1), nblk, hidden_stride, hidden_slots,
+            _DTYPE_CODE[src_dtype], cache_code, float(k_scale), float(v_scale), _stream(kv_cache))
+    _lib.check(st, "mixed_reshape_and_cache")
+
+
 def mixed_kv_to_cache(key, value, k_cache, v_cache, shared_k_cache, shared_v_cache, slot_mapping,
                       slot_mapping_shared, kv_cache_use_tot, hidden_cache_use_tot, *,
                       literal_modulo: bool = False, skip_mirror: bool = False) -> None:
@@ -523,3 +594,34 @@ def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_se
             k.stride(0), v.stride(0), out.stride(0), float(softmax_scale), _DTYPE_CODE[q.dtype], _stream(q))
     _lib.check(st, "flash_attn_varlen_func")
     return out
+
+
+# ------------------------------------------------------------------ names of the operator surface
+
+def gather_hidden_blocks(holder, paged_cache, slot_mapping, dst_idx) -> None:
+    """Hidden-block gather into a contiguous ``[T, Hd]`` buffer: ``cache_to_hidden`` under the name
+    the operator surface uses for it."""
+    cache_to_hidden(holder, paged_cache, slot_mapping, dst_idx)
+
+
+def paged_hybrid_attention(q, kv_cache, kv_workspace, block_tables, block_types, seq_lens, scale=None,
+                           kv_scale=None, **kw):
+    """Decode attention over a cache whose blocks hold either K/V (read from the layer's
+    ``kv_cache (2, N, BS, H, D)``) or re-projected hidden states (read from ``kv_workspace
+    (2, M, BS, H, D)``), chosen per block by ``block_types`` (uint8, 1 = workspace).
+    ``kv_scale``: per-tensor scale of an fp8 cache (one float, or a ``(k_scale, v_scale)`` pair)."""
+    if kv_scale is not None:
+        ks, vs = (kv_scale if isinstance(kv_scale, (tuple, list)) else (kv_scale, kv_scale))
+        kw.update(k_scale=float(ks), v_scale=float(vs))
+    ws_k = ws_v = None
+    if kv_workspace is not None:
+        ws_k, ws_v = kv_workspace[0], kv_workspace[1]
+    return paged_decode_attention(q, kv_cache[0], kv_cache[1], block_tables, seq_lens, scale,
+                                  block_types=block_types if kv_workspace is not None else None,
+                                  ws_k_cache=ws_k, ws_v_cache=ws_v, **kw)
+
+
+def build_hybrid_metadata(*args, **kwargs):
+    """``aptserve_hip.metadata.build_metadata`` (GPU-side construction of the ragged-batch metadata)."""
+    from . import metadata
+    return metadata.build_metadata(*args, **kwargs)

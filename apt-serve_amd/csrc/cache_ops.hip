@@ -189,6 +189,38 @@ struct KvScatterOp {
   }
 };
 
+// Write of one step's tokens by cache type: item = 2*t + plane.  A K/V token stores its K row (plane 0)
+// and V row (plane 1) by block; a hidden token stores its hidden row (plane 0 only) at its slot of the
+// flattened cache.  A null source pointer switches that kind of row off.
+struct MixedTokenOp {
+  const char* key; const char* value; const char* hidden;
+  char* k_cache; char* v_cache; char* hidden_cache;
+  const int64_t* slot_mapping; const uint8_t* is_hidden;
+  int64_t key_stride_b, value_stride_b, hidden_stride_b, block_stride_b, row_b, num_blocks;
+  int64_t hidden_slot_stride_b, num_hidden_slots;
+  BlockSplit split;
+  __device__ RowDesc operator()(int64_t item) const {
+    RowDesc r{nullptr, nullptr};
+    const int64_t t = item >> 1;
+    const int64_t slot = slot_mapping[t];
+    if (slot < 0) return r;
+    if (is_hidden && is_hidden[t]) {
+      if ((item & 1) || !hidden || slot >= num_hidden_slots) return r;
+      r.src = hidden + t * hidden_stride_b;
+      r.dst = hidden_cache + slot * hidden_slot_stride_b;
+      return r;
+    }
+    if (!key) return r;
+    int64_t blk, in_blk;
+    split(slot, blk, in_blk);
+    if (blk >= num_blocks) return r;
+    const int64_t off = blk * block_stride_b + in_blk * row_b;
+    if (item & 1) { r.src = value + t * value_stride_b; r.dst = v_cache + off; }
+    else          { r.src = key + t * key_stride_b;     r.dst = k_cache + off; }
+    return r;
+  }
+};
+
 // item = 2*blk + plane over the reference's grid of 2*nkv + nh blocks
 struct MixedKvOp {
   const char* key; const char* value;
@@ -296,13 +328,15 @@ template <class InT, int EPT>
 __global__ __launch_bounds__(kMaxThreads) void kv_scatter_fp8(
     const InT* __restrict__ key, const InT* __restrict__ value, uint8_t* __restrict__ k_cache,
     uint8_t* __restrict__ v_cache, const int64_t* __restrict__ slot_mapping,
-    const int64_t* __restrict__ token_idx, int64_t num_tokens, int64_t key_stride, int64_t value_stride,
-    int64_t block_stride, int64_t num_blocks, int block_size, int row_elems, float k_scale, float v_scale) {
+    const int64_t* __restrict__ token_idx, const uint8_t* __restrict__ skip_mask, int64_t num_tokens,
+    int64_t key_stride, int64_t value_stride, int64_t block_stride, int64_t num_blocks, int block_size,
+    int row_elems, float k_scale, float v_scale) {
   const int64_t item = blockIdx.x;
   const int64_t t = item >> 1;
   const bool is_v = item & 1;
   const int64_t tok = token_idx ? token_idx[t] : t;
   if (tok < 0 || tok >= num_tokens) return;
+  if (skip_mask && skip_mask[tok]) return;
   const int64_t slot = slot_mapping[tok];
   if (slot < 0) return;
   const int64_t blk = slot / block_size;
@@ -337,9 +371,10 @@ __global__ __launch_bounds__(kMaxThreads) void kv_scatter_fp8(
 
 template <class InT>
 int launch_kv_scatter_fp8(const void* key, const void* value, void* k_cache, void* v_cache,
-                          const int64_t* slot_mapping, const int64_t* token_idx, int64_t n, int64_t num_tokens,
-                          int64_t key_stride, int64_t value_stride, int64_t block_stride, int64_t num_blocks,
-                          int block_size, int row_elems, float k_scale, float v_scale, hipStream_t s) {
+                          const int64_t* slot_mapping, const int64_t* token_idx, const uint8_t* skip_mask,
+                          int64_t n, int64_t num_tokens, int64_t key_stride, int64_t value_stride,
+                          int64_t block_stride, int64_t num_blocks, int block_size, int row_elems, float k_scale,
+                          float v_scale, hipStream_t s) {
   const int in_b = (int)sizeof(InT);
   const bool aligned = row_elems % 8 == 0 &&
                        common_vec_bytes({addr(key), addr(value), (uint64_t)key_stride * in_b,
@@ -351,13 +386,37 @@ int launch_kv_scatter_fp8(const void* key, const void* value, void* k_cache, voi
   const dim3 grid((unsigned)(2 * n));
   if (aligned)
     hipLaunchKernelGGL((kv_scatter_fp8<InT, 8>), grid, dim3(threads), 0, s, (const InT*)key, (const InT*)value,
-                       (uint8_t*)k_cache, (uint8_t*)v_cache, slot_mapping, token_idx, num_tokens, key_stride,
-                       value_stride, block_stride, num_blocks, block_size, row_elems, k_scale, v_scale);
+                       (uint8_t*)k_cache, (uint8_t*)v_cache, slot_mapping, token_idx, skip_mask, num_tokens,
+                       key_stride, value_stride, block_stride, num_blocks, block_size, row_elems, k_scale, v_scale);
   else
     hipLaunchKernelGGL((kv_scatter_fp8<InT, 1>), grid, dim3(threads), 0, s, (const InT*)key, (const InT*)value,
-                       (uint8_t*)k_cache, (uint8_t*)v_cache, slot_mapping, token_idx, num_tokens, key_stride,
-                       value_stride, block_stride, num_blocks, block_size, row_elems, k_scale, v_scale);
+                       (uint8_t*)k_cache, (uint8_t*)v_cache, slot_mapping, token_idx, skip_mask, num_tokens,
+                       key_stride, value_stride, block_stride, num_blocks, block_size, row_elems, k_scale, v_scale);
   return launch_status();
+}
+
+int dispatch_kv_scatter_fp8(const void* key, const void* value, void* key_cache, void* value_cache,
+                            const int64_t* slot_mapping, const int64_t* token_idx, const uint8_t* skip_mask,
+                            int64_t n, int64_t num_tokens, int64_t key_stride, int64_t value_stride,
+                            int64_t block_stride, int64_t num_blocks, int block_size, int64_t row, int in_dtype,
+                            float k_scale, float v_scale, hipStream_t s) {
+  if (!(k_scale > 0.f) || !(v_scale > 0.f) || row >= (int64_t)1 << 30) return APS_ERR_INVALID_ARG;
+  switch (in_dtype) {
+    case APS_F16:
+      return launch_kv_scatter_fp8<_Float16>(key, value, key_cache, value_cache, slot_mapping, token_idx, skip_mask,
+                                             n, num_tokens, key_stride, value_stride, block_stride, num_blocks,
+                                             block_size, (int)row, k_scale, v_scale, s);
+    case APS_BF16:
+      return launch_kv_scatter_fp8<bf16_bits>(key, value, key_cache, value_cache, slot_mapping, token_idx,
+                                              skip_mask, n, num_tokens, key_stride, value_stride, block_stride,
+                                              num_blocks, block_size, (int)row, k_scale, v_scale, s);
+    case APS_F32:
+      return launch_kv_scatter_fp8<float>(key, value, key_cache, value_cache, slot_mapping, token_idx, skip_mask, n,
+                                          num_tokens, key_stride, value_stride, block_stride, num_blocks,
+                                          block_size, (int)row, k_scale, v_scale, s);
+    default:
+      return APS_ERR_UNSUPPORTED;
+  }
 }
 
 __global__ __launch_bounds__(kMaxThreads) void copy_bytes_kernel(VecOf<16>::type* __restrict__ dst,
@@ -496,23 +555,54 @@ int aps_reshape_and_cache_flash(const void* key, const void* value, void* key_ca
     return launch_rows(op, 2 * n, row * e, vb, s);
   }
   if (cache_dtype != APS_FP8_E4M3) return APS_ERR_UNSUPPORTED;
-  if (!(k_scale > 0.f) || !(v_scale > 0.f) || row >= (int64_t)1 << 30) return APS_ERR_INVALID_ARG;
-  switch (in_dtype) {
-    case APS_F16:
-      return launch_kv_scatter_fp8<_Float16>(key, value, key_cache, value_cache, slot_mapping, token_idx, n,
-                                             num_tokens, key_stride, value_stride, block_stride, num_blocks,
-                                             block_size, (int)row, k_scale, v_scale, s);
-    case APS_BF16:
-      return launch_kv_scatter_fp8<bf16_bits>(key, value, key_cache, value_cache, slot_mapping, token_idx, n,
-                                              num_tokens, key_stride, value_stride, block_stride, num_blocks,
-                                              block_size, (int)row, k_scale, v_scale, s);
-    case APS_F32:
-      return launch_kv_scatter_fp8<float>(key, value, key_cache, value_cache, slot_mapping, token_idx, n,
-                                          num_tokens, key_stride, value_stride, block_stride, num_blocks,
-                                          block_size, (int)row, k_scale, v_scale, s);
-    default:
-      return APS_ERR_UNSUPPORTED;
+  return dispatch_kv_scatter_fp8(key, value, key_cache, value_cache, slot_mapping, token_idx, nullptr, n,
+                                 num_tokens, key_stride, value_stride, block_stride, num_blocks, block_size, row,
+                                 in_dtype, k_scale, v_scale, s);
+}
+
+int aps_mixed_reshape_and_cache(const void* key, const void* value, const void* hidden, void* key_cache,
+                                void* value_cache, void* hidden_cache, const int64_t* slot_mapping,
+                                const uint8_t* is_hidden, int64_t num_tokens, int num_heads, int head_size,
+                                int block_size, int64_t key_stride, int64_t value_stride, int64_t hidden_stride,
+                                int64_t block_stride, int64_t num_blocks, int64_t hidden_slot_stride,
+                                int64_t num_hidden_slots, int in_dtype, int cache_dtype, float k_scale,
+                                float v_scale, aps_stream_t stream) {
+  if (num_tokens < 0 || num_heads <= 0 || head_size <= 0 || block_size <= 0) return APS_ERR_INVALID_ARG;
+  const int in_b = elem_bytes_of(in_dtype);
+  if (in_b == 0 || in_dtype == APS_FP8_E4M3) return APS_ERR_INVALID_ARG;
+  if (num_tokens == 0) return APS_OK;
+  if (!slot_mapping) return APS_ERR_INVALID_ARG;
+  const bool have_kv = key != nullptr, have_hidden = hidden != nullptr && is_hidden != nullptr;
+  if (have_kv && (!value || !key_cache || !value_cache)) return APS_ERR_INVALID_ARG;
+  if (hidden && !hidden_cache) return APS_ERR_INVALID_ARG;
+  if (!have_kv && !have_hidden) return APS_OK;
+  const int64_t row = (int64_t)num_heads * head_size;
+  if (have_kv && (key_stride < row || value_stride < row || block_stride < row * block_size))
+    return APS_ERR_INVALID_ARG;
+  if (have_hidden && (hidden_stride < row || hidden_slot_stride < row)) return APS_ERR_INVALID_ARG;
+  if (2 * num_tokens >= (int64_t)1 << 31) return APS_ERR_UNSUPPORTED;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t e = in_b;
+  const bool quantise = have_kv && cache_dtype != in_dtype;
+  if (quantise && cache_dtype != APS_FP8_E4M3) return APS_ERR_UNSUPPORTED;
+  // hidden rows (always in the activation dtype) and, unless they are quantised, K/V rows: one launch
+  MixedTokenOp op{quantise ? nullptr : (const char*)key, (const char*)value, have_hidden ? (const char*)hidden : nullptr,
+                  (char*)key_cache, (char*)value_cache, (char*)hidden_cache, slot_mapping, is_hidden,
+                  key_stride * e, value_stride * e, hidden_stride * e, block_stride * e, row * e, num_blocks,
+                  hidden_slot_stride * e, num_hidden_slots, BlockSplit(block_size)};
+  if (op.key || op.hidden) {
+    uint64_t bits = (uint64_t)(row * e);
+    if (op.key)
+      bits |= addr(key) | addr(value) | addr(key_cache) | addr(value_cache) | (uint64_t)(key_stride * e) |
+              (uint64_t)(value_stride * e) | (uint64_t)(block_stride * e);
+    if (op.hidden) bits |= addr(hidden) | addr(hidden_cache) | (uint64_t)(hidden_stride * e) | (uint64_t)(hidden_slot_stride * e);
+    const int st = launch_rows(op, 2 * num_tokens, row * e, common_vec_bytes({bits}), s);
+    if (st != APS_OK) return st;
   }
+  if (!quantise) return APS_OK;
+  return dispatch_kv_scatter_fp8(key, value, key_cache, value_cache, slot_mapping, nullptr, is_hidden, num_tokens,
+                                 num_tokens, key_stride, value_stride, block_stride, num_blocks, block_size, row,
+                                 in_dtype, k_scale, v_scale, s);
 }
 
 int aps_mixed_kv_to_cache(const void* key, const void* value, void* k_cache, void* v_cache, void* shared_k_cache,

@@ -59,6 +59,7 @@ struct MetaArgs {
   int64_t* hidden_cache_use_tot; int64_t* kv_cache_use_tot;
   int64_t* hidden_cache_use_input; int64_t* hidden_cache_store_tot;
   int64_t* hidden_holder_upd; int64_t* hidden_holder_pull; int64_t* holder_src; int64_t* kv_dest;
+  uint8_t* token_is_hidden;
   int32_t* block_tables_out; int64_t out_stride; int out_width;
   int32_t* seq_start_loc; int32_t* query_start_loc; int32_t* context_lens_out; int64_t* input_positions;
   int64_t* totals;
@@ -166,6 +167,7 @@ __global__ __launch_bounds__(kThreads) void prefill_metadata_kernel(const MetaAr
     if (tok < a.cap_rows) {
       a.slot_mapping[tok] = slot_of(bt, a.table_width, ctx + j, a.block_size);
       a.input_positions[tok] = ctx + j;
+      if (a.token_is_hidden) a.token_is_hidden[tok] = hid ? 1 : 0;
     }
     if (hid) {
       if (h0 + j < a.cap_hidden_rows) a.hidden_cache_use_input[h0 + j] = tok;
@@ -242,7 +244,8 @@ int aps_build_decode_metadata(const int32_t* seq_lens, const int32_t* use_hidden
 int aps_build_prefill_metadata(const int32_t* seq_lens, const int32_t* context_lens_in, const int32_t* use_hidden,
                                const int32_t* block_tables, int64_t table_stride, int64_t table_width,
                                int64_t batch, int block_size, int64_t* slot_mapping, int64_t* input_positions,
-                               int64_t* hidden_cache_use_input, int64_t* kv_cache_use_tot, int64_t cap_tokens,
+                               int64_t* hidden_cache_use_input, int64_t* kv_cache_use_tot,
+                               uint8_t* token_is_hidden, int64_t cap_tokens,
                                int64_t cap_hidden_tokens, int64_t cap_kv_tokens, int32_t* seq_start_loc,
                                int32_t* query_start_loc, int32_t* context_lens, int64_t* totals,
                                aps_stream_t stream) {
@@ -259,6 +262,7 @@ int aps_build_prefill_metadata(const int32_t* seq_lens, const int32_t* context_l
   a.table_stride = table_stride; a.table_width = (int)table_width; a.batch = (int)batch; a.block_size = block_size;
   a.slot_mapping = slot_mapping; a.input_positions = input_positions;
   a.hidden_cache_use_input = hidden_cache_use_input; a.kv_cache_use_tot = kv_cache_use_tot;
+  a.token_is_hidden = token_is_hidden;
   a.seq_start_loc = seq_start_loc; a.query_start_loc = query_start_loc; a.context_lens_out = context_lens;
   a.totals = totals;
   a.cap_rows = cap_tokens; a.cap_hidden_rows = cap_hidden_tokens; a.cap_kv = cap_kv_tokens;

@@ -141,6 +141,28 @@ int aps_reshape_and_cache_flash(const void* key, const void* value,
                                 int in_dtype, int cache_dtype, float k_scale,
                                 float v_scale, aps_stream_t stream);
 
+/* One write for a step whose tokens differ in cache type (the "mixed reshape
+ * and cache"): token t with is_hidden[t] != 0 stores hidden[t, :H*D] at slot
+ * slot_mapping[t] of the flattened hidden cache (hidden_cache + slot *
+ * hidden_slot_stride, as aps_hidden_to_cache does), any other token stores
+ * key[t] / value[t] by block as aps_reshape_and_cache_flash does.  Replaces, in
+ * one launch, the pair model_executor/models/aptserve_opt.py:125-126
+ * (hidden_to_cache over the hidden tokens) and
+ * attention/backends/aptserve_flash_attn.py:347-355 (reshape_and_cache_flash
+ * over gathered copies of the K/V tokens) of a prompt step.
+ * is_hidden nullable (all K/V); key/value nullable (only hidden rows are
+ * stored); hidden nullable (only K/V rows).  cache_dtype applies to the K/V
+ * rows only (APS_FP8_E4M3: quantised with k_scale / v_scale, then the K/V and
+ * the hidden cache are separate allocations); hidden rows keep in_dtype. */
+int aps_mixed_reshape_and_cache(
+    const void* key, const void* value, const void* hidden, void* key_cache,
+    void* value_cache, void* hidden_cache, const int64_t* slot_mapping,
+    const uint8_t* is_hidden, int64_t num_tokens, int num_heads, int head_size,
+    int block_size, int64_t key_stride, int64_t value_stride,
+    int64_t hidden_stride, int64_t block_stride, int64_t num_blocks,
+    int64_t hidden_slot_stride, int64_t num_hidden_slots, int in_dtype,
+    int cache_dtype, float k_scale, float v_scale, aps_stream_t stream);
+
 /* ref: mixed_cache.cu:179-230 (mixed_kv_to_cache) and :56-116 (kernel).
  * Range A: K/V rows kv_cache_use_tot[i] -> private caches at
  * slot_mapping[tok]; range B: the same rows -> shared caches; range C: rows
@@ -275,14 +297,17 @@ int aps_build_decode_metadata(
  * sequence (i in [context_len, seq_len)) gets slot table[i/BS]*BS + i%BS, or
  * -1 when table_width is 0.  hidden_cache_use_input = tokens of hidden-cached
  * prompts (it also serves as hidden_cache_use_tot and hidden_cache_store_tot),
- * kv_cache_use_tot = the other tokens.  context_lens_in may be NULL (= 0). */
+ * kv_cache_use_tot = the other tokens.  context_lens_in may be NULL (= 0).
+ * token_is_hidden (nullable, not in the reference): 1 for every token of a
+ * hidden-cached prompt, 0 otherwise: the mask aps_mixed_reshape_and_cache takes. */
 int aps_build_prefill_metadata(
     const int32_t* seq_lens, const int32_t* context_lens_in,
     const int32_t* use_hidden, const int32_t* block_tables,
     int64_t table_stride, int64_t table_width, int64_t batch, int block_size,
     int64_t* slot_mapping, int64_t* input_positions,
     int64_t* hidden_cache_use_input, int64_t* kv_cache_use_tot,
-    int64_t cap_tokens, int64_t cap_hidden_tokens, int64_t cap_kv_tokens,
+    uint8_t* token_is_hidden, int64_t cap_tokens, int64_t cap_hidden_tokens,
+    int64_t cap_kv_tokens,
     int32_t* seq_start_loc, int32_t* query_start_loc, int32_t* context_lens,
     int64_t* totals, aps_stream_t stream);
 

@@ -110,6 +110,22 @@ def reshape_and_cache_flash(key, value, key_cache, value_cache, slot_mapping,
     _store_rows(value_cache, slot_mapping, value[:n])
 
 
+def mixed_reshape_and_cache(key, value, hidden, paged_cache, slot_mapping, is_hidden) -> None:
+    """The two writes of a prompt step with hidden-cached sequences, as the reference issues them:
+    ``hidden_to_cache`` over the tokens of hidden-cached prompts
+    (additional_designs/model_executor/models/aptserve_opt.py:125-126) and
+    ``reshape_and_cache_flash`` over gathered copies of the other tokens
+    (additional_designs/attention/backends/aptserve_flash_attn.py:347-355).  Pinned through the
+    two functions it composes."""
+    mask = torch.as_tensor(is_hidden).bool()
+    hid_idx = torch.nonzero(mask).flatten()
+    kv_idx = torch.nonzero(~mask).flatten()
+    if hidden is not None:
+        hidden_to_cache(hidden, paged_cache, slot_mapping, hid_idx, hid_idx)
+    if key is not None:
+        reshape_and_cache_flash(key[kv_idx], value[kv_idx], paged_cache[0], paged_cache[1], slot_mapping[kv_idx])
+
+
 def mixed_kv_to_cache(key, value, k_cache, v_cache, shared_k_cache, shared_v_cache,
                       slot_mapping, slot_mapping_shared, kv_cache_use_tot,
                       hidden_cache_use_tot, literal_modulo: bool = False) -> None:

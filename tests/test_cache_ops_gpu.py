@@ -56,12 +56,88 @@ def test_config1_mixed_write_opt125m_bit_exact(dev):
     ops.hidden_to_cache(dh, g2, dsm, h_use.to(dev), idx(md, "hidden_cache_store_tot", dev))
     ops.reshape_and_cache_flash(dk, dv, g2[0], g2[1], dsm, "auto", token_idx=dkv)
     assert bits_equal(g2, ref)
+    # HIP, one launch by token type, mask from the GPU metadata builder
+    from aptserve_hip import metadata
+    gmd = metadata.build_from_batch(b, dev)
+    mask = torch.zeros(T, dtype=torch.uint8); mask[h_use] = 1
+    assert torch.equal(gmd.token_is_hidden.cpu(), mask)
+    g3 = cache.to(dev)
+    ops.mixed_reshape_and_cache(dk, dv, dh, g3, gmd.slot_mapping, gmd.token_is_hidden)
+    assert bits_equal(g3, ref)
+    ref2 = cache.clone()
+    O.mixed_reshape_and_cache(key, value, hidden, ref2, sm, mask)
+    assert bits_equal(ref2, ref)
     # untouched slots still hold the sentinel
     touched = torch.zeros(2 * N * BS, dtype=torch.bool)
     touched[sm[h_use]] = True
     touched[sm[kv_use]] = True
     touched[sm[kv_use] + N * BS] = True
     assert bits_equal(g2.cpu().view(-1, H * D)[~touched], cache.view(-1, H * D)[~touched])
+
+
+# ------------------------------------------------------- write by token type
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("H,D", [(2, 4), (12, 64), (1, 5)])
+@pytest.mark.parametrize("seed,frac", [(0, 0.4), (1, 1.0), (2, 0.0)])
+def test_mixed_reshape_and_cache_small(dev, dtype, H, D, seed, frac):
+    b = workloads.small_prefill_batch(seed, 7, 60, frac, 64)
+    md = oracle_metadata(b)
+    T, N, BS = md["num_prefill_tokens"], 64, 16
+    sm = t64(md["slot_mapping"]).clone()
+    sm[::11] = -1                                          # padding tokens of either kind
+    mask = torch.zeros(T, dtype=torch.uint8); mask[t64(md["hidden_cache_use_input"])] = 1
+    wide = randn((T, 3 * H * D), seed, dtype)              # K and V as chunk views of a fused projection
+    key, value = wide[:, :H * D].view(T, H, D), wide[:, H * D:2 * H * D].view(T, H, D)
+    hidden = randn((T, H * D), seed + 9, dtype)
+    cache = sentinel_cache((2, N, BS, H, D), dtype)
+    ref = cache.clone()
+    O.mixed_reshape_and_cache(key, value, hidden, ref, sm, mask)
+    g = cache.to(dev)
+    dw = wide.to(dev)
+    dk, dv = dw[:, :H * D].view(T, H, D), dw[:, H * D:2 * H * D].view(T, H, D)
+    ops.mixed_reshape_and_cache(dk, dv, hidden.to(dev), g, sm.to(dev), mask.to(dev))
+    assert bits_equal(g, ref)
+    # one kind only
+    ref_h, ref_kv = cache.clone(), cache.clone()
+    O.mixed_reshape_and_cache(None, None, hidden, ref_h, sm, mask)
+    O.mixed_reshape_and_cache(key, value, None, ref_kv, sm, mask)
+    g_h, g_kv = cache.to(dev), cache.to(dev)
+    ops.mixed_reshape_and_cache(None, None, hidden.to(dev), g_h, sm.to(dev), mask.to(dev))
+    ops.mixed_reshape_and_cache(dk, dv, None, g_kv, sm.to(dev), mask.to(dev))
+    assert bits_equal(g_h, ref_h) and bits_equal(g_kv, ref_kv)
+    # no mask: every token is a K/V token == reshape_and_cache_flash
+    # (hidden sequences use block ids >= N for their odd blocks: no K/V block there, mark as padding)
+    ref_all, g_all = cache.clone(), cache.to(dev)
+    sm_kv = torch.where(sm < N * BS, sm, torch.full_like(sm, -1))
+    O.reshape_and_cache_flash(key, value, ref_all[0], ref_all[1], sm_kv, "auto")
+    ops.mixed_reshape_and_cache(dk, dv, None, g_all, sm_kv.to(dev), None)
+    assert bits_equal(g_all, ref_all)
+
+
+def test_mixed_reshape_and_cache_fp8_kv_rows(dev):
+    """K/V rows quantised into a 1-byte cache, hidden rows unquantised into their own cache."""
+    H, D, N, BS = 12, 64, 64, 16
+    b = workloads.small_prefill_batch(5, 7, 60, 0.5, N)
+    md = oracle_metadata(b)
+    T = md["num_prefill_tokens"]
+    sm = t64(md["slot_mapping"])
+    mask = torch.zeros(T, dtype=torch.uint8); mask[t64(md["hidden_cache_use_input"])] = 1
+    key, value, hidden = randn((T, H, D), 0) * 3, randn((T, H, D), 1) * 3, randn((T, H * D), 2)
+    kv_idx = torch.nonzero(mask == 0).flatten()
+    q_ref = torch.full((2, N, BS, H, D), 0x55, dtype=torch.uint8)
+    O.reshape_and_cache_flash(key[kv_idx], value[kv_idx], q_ref[0], q_ref[1], sm[kv_idx], "fp8", 0.5, 0.25)
+    h_ref = sentinel_cache((2, N, BS, H, D))
+    h0 = h_ref.clone()
+    O.mixed_reshape_and_cache(None, None, hidden, h_ref, sm, mask)
+    q = torch.full((2, N, BS, H, D), 0x55, dtype=torch.uint8, device=dev)
+    hc = h0.to(dev)
+    ops.mixed_reshape_and_cache(key.to(dev), value.to(dev), hidden.to(dev), q, sm.to(dev), mask.to(dev), "fp8",
+                                0.5, 0.25, hidden_cache=hc)
+    assert torch.equal(q.cpu(), q_ref)
+    assert bits_equal(hc, h_ref)
+    with pytest.raises(ValueError):                        # an fp8 cache cannot hold hidden rows itself
+        ops.mixed_reshape_and_cache(key.to(dev), value.to(dev), hidden.to(dev), q, sm.to(dev), mask.to(dev), "fp8")
 
 
 # ------------------------------------------------------- small random batches
