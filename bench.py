@@ -304,6 +304,19 @@ def reproject_figures(torch, ops, dev, seed):
             "workload": "config3 [T,5120]x[5120,10240] f16, f32 accumulate, T=%d" % T, "ms": ms, "tflops": tf,
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": None}}
+        if T == 16384 and hasattr(ops, "kv_reproject_to_cache"):
+            # same product, rows written straight to random slots of [blocks,16,40,128] K and V caches
+            nblk = 2 * T // 16
+            caches = [torch.empty(nblk, 16, 40, 128, dtype=torch.float16, device=dev) for _ in range(2)]
+            dest = torch.randperm(nblk * 16, generator=g, device=dev)[:T].contiguous()
+            ms2 = median(event_times(
+                torch, lambda: ops.kv_reproject_to_cache(x, w, bias, caches[0], caches[1], None, None, dest), 20))
+            out["kv_reproject_to_cache_T%d" % T] = {
+                "workload": "config3 with the cache write in the epilogue (random slots), T=%d" % T, "ms": ms2,
+                "tflops": flops / ms2 / 1e9,
+                "roofline": {"bound": "mfma", "achieved": flops / ms2 / 1e9, "peak": MFMA_F16_PEAK_TFLOPS,
+                             "unit": "TFLOP/s", "frac": flops / ms2 / 1e9 / MFMA_F16_PEAK_TFLOPS, "traffic": None}}
+            del caches
     return out
 
 
