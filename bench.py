@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip attention / re-projection figures")
+    ap.add_argument("--extras", default="attention,metadata,write,reproject,step_loop",
+                    help="comma-separated subset of the extra figures to run")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="first run the plain copy kernel on 1 GiB three times (known traffic for counter scaling)")
     return ap.parse_args()
@@ -198,23 +200,25 @@ def main():
                      "algorithmic_bytes_per_launch": gather_alg, "avg_launch_ms": gather_ms},
     }
 
-    if not args.no_extras:
+    want = set() if args.no_extras else set(x for x in args.extras.split(",") if x)
+    if want:
         extras = {}
         del holder
-        for fp8 in (False, True):
+        for fp8 in ((False, True) if "attention" in want else ()):
             torch.cuda.empty_cache()
             extras["decode_attention_fp8" if fp8 else "decode_attention_f16"] = attention_figures(
                 torch, ops, workloads, np, dev, args.seed, fp8)
         # metadata build, GPU vs the list-based host algorithm
         t = []
-        for _ in range(10):
+        for _ in range(10 if "metadata" in want else 0):
             torch.cuda.synchronize()
             a = time.perf_counter()
             metadata.build_from_batch(batch, dev)
             torch.cuda.synchronize()
             t.append((time.perf_counter() - a) * 1e6)
-        extras["metadata_build_us"] = median(t)
-        if not args.no_cpu:
+        if t:
+            extras["metadata_build_us"] = median(t)
+        if not args.no_cpu and "metadata" in want:
             # the reference's approach to the same metadata: Python lists per cached token, then tensors
             from oracle.metadata import SeqRecord, build_metadata as list_build
             recs = [SeqRecord(False, h, l, l - 1, bt, bts) for l, h, bt, bts in
@@ -225,11 +229,13 @@ def main():
                 list_build(recs, batch.block_size)
                 t.append((time.perf_counter() - a) * 1e6)
             extras["metadata_build_us_cpu_list_algorithm"] = median(t)
-        extras["kv_write_prefill_16384"] = write_figures(torch, ops, dev, args.seed)
-        if hasattr(ops, "kv_reproject"):
+        if "write" in want:
+            extras["kv_write_prefill_16384"] = write_figures(torch, ops, dev, args.seed)
+        if "reproject" in want:
             extras.update(reproject_figures(torch, ops, dev, args.seed))
         torch.cuda.empty_cache()
-        extras["opt13b_step_loop"] = step_loop_figures(torch, dev, args.seed)
+        if "step_loop" in want:
+            extras["opt13b_step_loop"] = step_loop_figures(torch, dev, args.seed)
         result["extras"] = extras
 
     if not args.no_cpu:
