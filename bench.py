@@ -25,7 +25,8 @@ for p in (ROOT, ROOT / "apt-serve_amd"):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (seed 0 workloads), scaled by what the
 # same counters read for the 1 GiB copy kernel (x2.000 and x1.000); summary in profiles/bench_step_hbm_counters.txt
-PMC_TRAFFIC_BYTES = {"gather": 1804.9e6, "attention_f16": 1800.4e6, "attention_fp8": 905.3e6}
+PMC_TRAFFIC_BYTES = {"gather": 1804.9e6, "attention_f16": 1800.4e6, "attention_fp8": 906.6e6,
+                     "gemm_T4096": 805.0e6, "gemm_T16384": 2884.9e6}
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 
 
@@ -309,7 +310,8 @@ def reproject_figures(torch, ops, dev, seed):
         out["kv_reproject_T%d" % T] = {
             "workload": "config3 [T,5120]x[5120,10240] f16, f32 accumulate, T=%d" % T, "ms": ms, "tflops": tf,
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": None}}
+                         "frac": tf / MFMA_F16_PEAK_TFLOPS,
+                         "traffic": PMC_TRAFFIC_BYTES["gemm_T%d" % T] if seed == 0 else None}}
         if T == 16384 and hasattr(ops, "kv_reproject_to_cache"):
             # same product, rows written straight to random slots of [blocks,16,40,128] K and V caches
             nblk = 2 * T // 16
