@@ -56,6 +56,7 @@ constexpr int kLdsBytes =
     kWaves * kEpiWaveBytes > kStages * kStageBytes ? kWaves * kEpiWaveBytes : kStages * kStageBytes;
 constexpr int kNumXcd = 8;
 constexpr int kGroupM = 8;
+constexpr int kSkinnyMaxRows = 16;  // at most this many rows: the weight-streaming kernel
 
 // Where a result row goes.  Plain: row t of C is row t (or map[t], negative skipped) of base[0], ld elements
 // apart.  Cache mode (n_split > 0): columns below n_split are the K part of the row and columns from n_split
@@ -322,6 +323,254 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
 }
 
+// ---------------------------------------------------------------- few rows (a decode step's projections)
+// out[m, n] for m <= 16: the product is a stream of the weights.  One workgroup owns 16 weight rows;
+// its 8 wavefronts split K, each feeding v_mfma_f32_16x16x32 with the 16 weight rows as the A operand
+// (lane l: row l%16, k-chunk l/16 of 8 elements) and the <=16 activation rows as B (rows beyond m read
+// as zero through the buffer bounds); the 8 partial 16x16 results are added in LDS in a fixed order.
+// No workspace and no second launch; every lane keeps up to 2 x kSkU 16-byte weight loads in flight.
+typedef float float4v __attribute__((ext_vector_type(4)));
+constexpr int kSkWaves = 8, kSkU = 8;
+
+template <bool BF16>
+__device__ __forceinline__ float4v mfma16(const u32x4& a, const u32x4& b, const float4v& c) {
+  if constexpr (BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                   0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0,
+                                                  0);
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(kSkWaves * 64) void skinny_nt_kernel(const GemmArgs g, int steps_per_wave) {
+  __shared__ float4v red[kSkWaves][64];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int64_t n0 = (int64_t)blockIdx.x * 16;
+  const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(g.w + n0 * g.ldw_b, (g.n - n0) * g.ldw_b);
+  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(g.a, g.m * g.lda_b);
+  const int row = lane & 15, kg = lane >> 4;
+  const uint32_t voff_w = (uint32_t)(row * g.ldw_b + kg * 16);
+  const uint32_t voff_x = (uint32_t)(row * g.lda_b + kg * 16);  // rows >= m are out of bounds: zero
+  const int total_steps = (int)(g.k / 32);
+  const int s_begin = wave * steps_per_wave;
+  const int s_end = min(total_steps, s_begin + steps_per_wave);
+  float4v acc = {0.f, 0.f, 0.f, 0.f};
+  u32x4 wa[kSkU], xa[kSkU], wb[kSkU], xb[kSkU];
+  auto load_block = [&](int s0, u32x4(&wq)[kSkU], u32x4(&xq)[kSkU]) {
+#pragma unroll
+    for (int u = 0; u < kSkU; ++u) {
+      if (s0 + u < s_end) {
+        const uint32_t koff = (uint32_t)(s0 + u) * 64;
+        wq[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, voff_w, koff, 2));
+        xq[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff_x, koff, 0));
+      }
+    }
+  };
+  auto mac_block = [&](int s0, const u32x4(&wq)[kSkU], const u32x4(&xq)[kSkU]) {
+#pragma unroll
+    for (int u = 0; u < kSkU; ++u)
+      if (s0 + u < s_end) acc = mfma16<BF16>(wq[u], xq[u], acc);
+  };
+  int s = s_begin;
+  if (s < s_end) load_block(s, wa, xa);
+  while (s < s_end) {
+    load_block(s + kSkU, wb, xb);
+    mac_block(s, wa, xa);
+    s += kSkU;
+    if (s >= s_end) break;
+    load_block(s + kSkU, wa, xa);
+    mac_block(s, wb, xb);
+    s += kSkU;
+  }
+  red[wave][lane] = acc;
+  __syncthreads();
+  if (wave != 0) return;
+  float4v sum = red[0][lane];
+#pragma unroll
+  for (int w = 1; w < kSkWaves; ++w) {
+    const float4v p = red[w][lane];
+    sum[0] += p[0]; sum[1] += p[1]; sum[2] += p[2]; sum[3] += p[3];
+  }
+  // lane l holds out[token l%16][n0 + 4*(l/16) + i], i = 0..3
+  const int64_t token = row;
+  if (token >= g.m) return;
+  const int64_t n = n0 + 4 * kg;
+  const int half = (g.out.n_split && n >= g.out.n_split) ? 1 : 0;
+  uint16_t* dst = out_row(g.out, token, half);
+  if (!dst) return;
+  dst += n - (half ? g.out.n_split : 0);
+  uint16_t h[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float v = sum[i];
+    if (g.bias) {
+      const uint16_t bb = ((const uint16_t*)g.bias)[n + i];
+      v += BF16 ? __uint_as_float((uint32_t)bb << 16) : (float)__builtin_bit_cast(_Float16, bb);
+    }
+    h[i] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+  }
+  if (g.out.aligned16) {  // 8-byte store
+    uint2 v2 = {(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+    *(uint2*)dst = v2;
+  } else {
+    dst[0] = h[0]; dst[1] = h[1]; dst[2] = h[2]; dst[3] = h[3];
+  }
+}
+
+// ---------------------------------------------------------------- at most 8 rows: weights as a pure stream
+// Every wavefront owns 2 whole weight rows and reads them as contiguous 1 KiB wave-wide loads (lane l:
+// 8 elements at k = 512*j + 8*l), straight into registers: on this part a wave-wide load that covers
+// 16 rows x 64 B streams at 4.4 TB/s, one that covers 1 KiB of a row at 7 TB/s.  The activations are tiny
+// and shared: the workgroup stages them in LDS, 2048 elements of K at a time ([MT][2048], copied
+// global -> LDS without a register round trip), from where a lane reads the 8 elements that match its
+// weight chunk (consecutive lanes, consecutive 16 bytes).  v_dot2 with fp32 accumulation does the
+// arithmetic (4*MT per weight load); the 64 partial sums of a row are added once, at the end.
+// Chunk c+1 (weights into a second register set, activations into the other LDS buffer) is in flight
+// while chunk c is multiplied; one barrier per chunk.
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+constexpr int kRsWaves = 8, kRsRows = 2, kRsKc = 2048, kRsJ = kRsKc / 512;
+
+template <bool BF16>
+__device__ __forceinline__ float dot8(const u32x4& a, const u32x4& b, float c) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t ai = a[i], bi = b[i];
+    if constexpr (BF16)
+      c = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, ai), __builtin_bit_cast(bf16x2, bi), c, false);
+    else
+      c = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, ai), __builtin_bit_cast(half2v, bi), c, false);
+  }
+  return c;
+}
+
+__device__ __forceinline__ float wave_total(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true));
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  return v;
+}
+
+template <bool BF16, int MT>
+__global__ __launch_bounds__(kRsWaves * 64) void rowstream_nt_kernel(const GemmArgs g) {
+  __shared__ __attribute__((aligned(1024))) char xs[2][MT][kRsKc * 2];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int64_t n_first = ((int64_t)blockIdx.x * kRsWaves + wave) * kRsRows;
+  const char* wrow = g.w + n_first * g.ldw_b + lane * 16;
+  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(g.a, g.m * g.lda_b);
+  float acc[kRsRows][MT];
+#pragma unroll
+  for (int i = 0; i < kRsRows; ++i)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[i][m] = 0.f;
+  const int nchunks = (int)((g.k + kRsKc - 1) / kRsKc);
+
+  // 1 KiB pieces of the activation chunk (MT rows x kRsJ pieces) are spread over the wavefronts
+  auto stage_x = [&](int c) {
+    const int64_t k0 = (int64_t)c * kRsKc;
+    const int kcur = (int)min((int64_t)kRsKc, g.k - k0);
+#pragma unroll
+    for (int p = 0; p < (MT * kRsJ + kRsWaves - 1) / kRsWaves; ++p) {
+      const int piece = p * kRsWaves + wave;
+      const int m = piece / kRsJ, q = piece % kRsJ;
+      if (piece < MT * kRsJ && q * 512 < kcur)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (__attribute__((address_space(3))) void*)(&xs[c & 1][m][q * 1024]),
+                                                 16, (uint32_t)(lane * 16), (uint32_t)(m * g.lda_b + (k0 + q * 512) * 2),
+                                                 0, 0);
+    }
+  };
+  auto load_w = [&](int c, u32x4(&wq)[kRsRows][kRsJ]) {
+    const int64_t k0 = (int64_t)c * kRsKc;
+    const int kcur = (int)min((int64_t)kRsKc, g.k - k0);
+#pragma unroll
+    for (int i = 0; i < kRsRows; ++i)
+#pragma unroll
+      for (int j = 0; j < kRsJ; ++j) {
+        wq[i][j] = u32x4{0u, 0u, 0u, 0u};
+        if (j * 512 + lane * 8 < kcur)
+          wq[i][j] = __builtin_nontemporal_load((const u32x4*)(wrow + i * g.ldw_b + (k0 + j * 512) * 2));
+      }
+  };
+  auto multiply = [&](int c, const u32x4(&wq)[kRsRows][kRsJ]) {
+    const int kcur = (int)min((int64_t)kRsKc, g.k - (int64_t)c * kRsKc);
+#pragma unroll
+    for (int j = 0; j < kRsJ; ++j) {
+      if (j * 512 + lane * 8 < kcur) {  // lanes past the end of K hold no weights and stale activations
+        u32x4 xv[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) xv[m] = *(const u32x4*)(&xs[c & 1][m][j * 1024 + lane * 16]);
+#pragma unroll
+        for (int i = 0; i < kRsRows; ++i)
+#pragma unroll
+          for (int m = 0; m < MT; ++m) acc[i][m] = dot8<BF16>(wq[i][j], xv[m], acc[i][m]);
+      }
+    }
+  };
+
+  u32x4 wa[kRsRows][kRsJ], wb[kRsRows][kRsJ];
+  stage_x(0);
+  load_w(0, wa);
+  for (int c = 0; c < nchunks; c += 2) {
+    APS_WAIT_VM(0);  // chunk c has landed (activations in LDS, weights in registers)
+    APS_BARRIER();   // ... for every wavefront, and the other LDS buffer is free
+    if (c + 1 < nchunks) { stage_x(c + 1); load_w(c + 1, wb); }
+    multiply(c, wa);
+    if (c + 1 >= nchunks) break;
+    APS_WAIT_VM(0);
+    APS_BARRIER();
+    if (c + 2 < nchunks) { stage_x(c + 2); load_w(c + 2, wa); }
+    multiply(c + 1, wb);
+  }
+#pragma unroll
+  for (int i = 0; i < kRsRows; ++i)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[i][m] = wave_total(acc[i][m]);
+  // lane i*MT + m stores out[m][n_first + i]
+#pragma unroll
+  for (int i = 0; i < kRsRows; ++i)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      if (lane != i * MT + m) continue;
+      const int64_t n = n_first + i;
+      const int half = (g.out.n_split && n >= g.out.n_split) ? 1 : 0;
+      uint16_t* dst = out_row(g.out, m, half);
+      if (!dst) continue;
+      float v = acc[i][m];
+      if (g.bias) {
+        const uint16_t bb = ((const uint16_t*)g.bias)[n];
+        v += BF16 ? __uint_as_float((uint32_t)bb << 16) : (float)__builtin_bit_cast(_Float16, bb);
+      }
+      dst[n - (half ? g.out.n_split : 0)] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+    }
+}
+
+template <bool BF16, int MT>
+int launch_rowstream(const GemmArgs& g, hipStream_t s) {
+  hipLaunchKernelGGL((rowstream_nt_kernel<BF16, MT>), dim3((unsigned)(g.n / (kRsWaves * kRsRows))),
+                     dim3(kRsWaves * 64), 0, s, g);
+  return launch_status();
+}
+
+template <bool BF16>
+int launch_rowstream_m(const GemmArgs& g, hipStream_t s) {
+  switch (g.m) {
+    case 1: return launch_rowstream<BF16, 1>(g, s);
+    case 2: return launch_rowstream<BF16, 2>(g, s);
+    case 3: return launch_rowstream<BF16, 3>(g, s);
+    case 4: return launch_rowstream<BF16, 4>(g, s);
+    case 5: return launch_rowstream<BF16, 5>(g, s);
+    case 6: return launch_rowstream<BF16, 6>(g, s);
+    case 7: return launch_rowstream<BF16, 7>(g, s);
+    default: return launch_rowstream<BF16, 8>(g, s);
+  }
+}
+
 // out[m][n] = sum_z partial[z][m][n] + bias[n], rounded once; 4 columns per thread
 template <bool BF16>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, const void* bias,
@@ -358,6 +607,7 @@ int aps_linear_nt_splits(int64_t m, int64_t n, int64_t k) {
   // Few tiles (a decode step's handful of tokens) cannot pull the weights at HBM speed with one workgroup
   // per tile: split K until about two waves of workgroups exist, keeping at least 4 k-tiles per split.
   if (m <= 0 || n <= 0 || k <= 0 || n % BN != 0 || k % BK != 0) return 1;
+  if (m <= kSkinnyMaxRows) return 1;  // streamed in one launch
   if (m > 2 * BM) return 1;  // beyond two row tiles the fp32 partials cost more than the extra workgroups gain
   const int64_t tiles = ((m + BM - 1) / BM) * (n / BN);
   const int64_t nk = k / BK;
@@ -388,6 +638,19 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   g.m = m; g.n = n; g.k = k;
   g.tiles_m = (int)((m + BM - 1) / BM); g.tiles_n = (int)(n / BN);
   g.out = om;
+  hipStream_t s = (hipStream_t)stream;
+  if (m <= 8) return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
+  if (m <= kSkinnyMaxRows && n / 16 < ((int64_t)1 << 31) && x_stride * 2 * 16 < ((int64_t)1 << 31) &&
+      w_stride * 2 * 16 < ((int64_t)1 << 31)) {
+    const int steps = (int)(k / 32);
+    const int per_wave = (steps + kSkWaves - 1) / kSkWaves;
+    const dim3 grid((unsigned)(n / 16));
+    if (dtype == APS_BF16)
+      hipLaunchKernelGGL(skinny_nt_kernel<true>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
+    else
+      hipLaunchKernelGGL(skinny_nt_kernel<false>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
+    return launch_status();
+  }
   const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
   if (total >= ((int64_t)1 << 30)) return APS_ERR_UNSUPPORTED;
   const int64_t per_xcd = (total + kNumXcd - 1) / kNumXcd;
@@ -401,7 +664,6 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   g.kt_per_split = (int)((nk_all + splits - 1) / splits);
   if (splits > 1) splits = (int)((nk_all + g.kt_per_split - 1) / g.kt_per_split);  // no empty split
   const dim3 grid((unsigned)(per_xcd * kNumXcd), (unsigned)splits);
-  hipStream_t s = (hipStream_t)stream;
   // more than 64 KiB of dynamic LDS has to be allowed per function (and per device)
   const void* fn = dtype == APS_BF16 ? (const void*)gemm_nt_kernel<true> : (const void*)gemm_nt_kernel<false>;
   const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
