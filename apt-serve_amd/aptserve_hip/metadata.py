@@ -59,6 +59,9 @@ class HybridAttentionMetadata:
     holder_src: Optional[torch.Tensor] = None       # int64 [num_tot]: resolved source of every holder row
     kv_dest: Optional[torch.Tensor] = None          # int64 [num_tot]: cache slot the row's re-projected K/V go to
     token_is_hidden: Optional[torch.Tensor] = None  # uint8 [prompt tokens]: 1 = token of a hidden-cached prompt
+    hidden_slots: Optional[torch.Tensor] = None     # int64 [hidden rows]: private slot of every cached hidden row
+    hidden_seq_start: Optional[torch.Tensor] = None  # int64 [hidden seqs + 1]: first hidden row of each hidden sequence
+    max_hidden_seq_len: int = 0
     _cached_prefill_metadata: Optional["HybridAttentionMetadata"] = None
     _cached_decode_metadata: Optional["HybridAttentionMetadata"] = None
 
@@ -105,7 +108,8 @@ class HybridAttentionMetadata:
                 seq_start_loc=None, context_lens_tensor=None, block_tables=self.block_tables[self.num_prefills:],
                 use_cuda_graph=self.use_cuda_graph, input_positions=self.input_positions,
                 block_types=None if self.block_types is None else self.block_types[self.num_prefills:],
-                holder_src=self.holder_src, kv_dest=self.kv_dest)
+                holder_src=self.holder_src, kv_dest=self.kv_dest, hidden_slots=self.hidden_slots,
+                hidden_seq_start=self.hidden_seq_start, max_hidden_seq_len=self.max_hidden_seq_len)
         return self._cached_decode_metadata
 
 
@@ -222,10 +226,10 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
         d_bt = packed[2 * B:2 * B + B * W].view(B, W)
         d_bts = packed[2 * B + B * W:].view(B, Ws)
         # one allocation per output dtype
-        sizes64 = [num_tot, n_hr, n_hr, n_kv, n_hs, n_hs, B, num_tot - B, B, 4, num_tot, num_tot]
+        sizes64 = [num_tot, n_hr, n_hr, n_kv, n_hs, n_hs, B, num_tot - B, B, 4, num_tot, num_tot, n_hr, n_hs + 1]
         buf64 = torch.empty(sum(sizes64), **i64)
         (slot_mapping, slot_mapping_shared, use_tot, kv_use, use_input, store_tot, upd, pull, positions,
-         totals, holder_src, kv_dest) = torch.split(buf64, sizes64)
+         totals, holder_src, kv_dest, hidden_slots, hidden_seq_start) = torch.split(buf64, sizes64)
         sizes32 = [B * Wo, B + 1, B + 1, B]
         buf32 = torch.empty(sum(sizes32), **i32)
         bt_out, seq_start, query_start, ctx = torch.split(buf32, sizes32)
@@ -237,7 +241,8 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
                 slot_mapping_shared.data_ptr() if n_hr else None, use_tot.data_ptr() if n_hr else None,
                 kv_use.data_ptr() if n_kv else None, use_input.data_ptr() if n_hs else None,
                 store_tot.data_ptr() if n_hs else None, upd.data_ptr(), pull.data_ptr() if num_tot > B else None,
-                holder_src.data_ptr(), kv_dest.data_ptr(), num_tot, n_hr, n_hs, n_kv,
+                holder_src.data_ptr(), kv_dest.data_ptr(), hidden_slots.data_ptr() if n_hr else None,
+                hidden_seq_start.data_ptr() if n_hs else None, num_tot, n_hr, n_hs, n_kv,
                 bt_out.data_ptr() if Wo else None, Wo, Wo, seq_start.data_ptr(),
                 query_start.data_ptr(), ctx.data_ptr(), positions.data_ptr(), totals.data_ptr(),
                 torch.cuda.current_stream(device).cuda_stream)
@@ -256,7 +261,8 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
             seq_lens=[int(x) for x in lens], seq_lens_tensor=d_lens, max_query_len=1, max_prefill_seq_len=0,
             max_decode_seq_len=int(lens.max()), query_start_loc=query_start, seq_start_loc=seq_start,
             context_lens_tensor=ctx, block_tables=bt_out, use_cuda_graph=False, input_positions=positions,
-            block_types=block_types, holder_src=holder_src, kv_dest=kv_dest)
+            block_types=block_types, holder_src=holder_src, kv_dest=kv_dest, hidden_slots=hidden_slots,
+            hidden_seq_start=hidden_seq_start, max_hidden_seq_len=int(lens[hid].max()) if n_hs else 0)
 
     # ------------------------------------------------------------------ prompts
     ctxs = np.zeros(B, dtype=np.int64) if context_lens is None else np.asarray(context_lens, dtype=np.int64)

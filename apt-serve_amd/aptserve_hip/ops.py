@@ -596,6 +596,61 @@ def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_se
     return out
 
 
+# ------------------------------------------------------------------ attention on cached hidden rows
+
+def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, seq_rows, max_len, w_k, w_v, b_v,
+                              softmax_scale, out, workspace=None):
+    """Decode attention of the hidden-cached sequences of a batch, computed on their cached hidden
+    rows with the K/V projection weights absorbed into the query and the output:
+    ``s[h,t] = scale <W_k[h]^T q[h], hidden_t>``, ``out[h] = W_v[h] (sum_t p[h,t] hidden_t) + b_v[h]``.
+    Equal (up to rounding) to re-projecting every row and attending over the result — the sequence
+    of additional_designs/model_executor/models/aptserve_opt.py:112-124 and
+    additional_designs/attention/backends/aptserve_flash_attn.py:359-373, :464-473 — without the
+    gather, the re-projection GEMM and the K/V workspace.
+
+    ``q [B, H*D]`` query rows of the batch; ``seq_rows`` (= ``hidden_cache_use_input``) batch
+    positions of the hidden-cached sequences; ``hidden_slots`` / ``hidden_seq_start`` from the
+    metadata builder; ``w_k``, ``w_v [H*D, H*D]`` row slices of the fused QKV weight; the result of
+    sequence ``i`` is written to ``out[seq_rows[i]]`` (``out [B, H*D]``).  The newest hidden row of
+    every sequence must already be in the cache."""
+    dev = q.device
+    for n, t in (("q", q), ("paged_cache", paged_cache), ("w_k", w_k), ("w_v", w_v), ("out", out)):
+        _check_data(n, t, dev)
+    _need(paged_cache.dim() == 5 and paged_cache.is_contiguous(), "paged_cache must be contiguous (2, N, BS, H, D)")
+    heads, head_size = paged_cache.size(3), paged_cache.size(4)
+    hidden = heads * head_size
+    _need(q.dim() == 2 and q.size(1) == hidden and out.dim() == 2 and out.size(1) == hidden,
+          "q and out must be [rows, heads*head_dim]")
+    _need(w_k.dim() == 2 and w_k.shape == (hidden, hidden) and w_v.shape == (hidden, hidden),
+          "w_k and w_v must be [H*D, H*D]")
+    _need(w_k.stride(0) == w_v.stride(0), "w_k and w_v must have the same row stride")
+    _need(q.dtype in (torch.float16, torch.bfloat16), "f16 or bf16 expected")
+    _need(all(t.dtype == q.dtype for t in (paged_cache, w_k, w_v, out)), "dtypes differ")
+    if b_v is not None:
+        _check_data("b_v", b_v, dev)
+        _need(b_v.dim() == 1 and b_v.numel() == hidden and b_v.dtype == q.dtype and b_v.is_contiguous(),
+              "b_v must be a contiguous [H*D] vector of the operand dtype")
+    for n, t in (("hidden_slots", hidden_slots), ("hidden_seq_start", hidden_seq_start), ("seq_rows", seq_rows)):
+        _check_index(n, t, dev)
+    n_seqs = seq_rows.numel()
+    _need(hidden_seq_start.numel() == n_seqs + 1, "hidden_seq_start needs one entry per sequence plus one")
+    if n_seqs == 0:
+        return out
+    lib = _lib.load()
+    need = lib.aps_absorbed_attention_workspace_bytes(n_seqs, int(max_len), heads, head_size)
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)      # scratch is host-side plumbing
+    with torch.cuda.device(dev):
+        st = lib.aps_absorbed_attention(
+            q.data_ptr(), q.stride(0), seq_rows.data_ptr(), q.size(0), paged_cache.data_ptr(), paged_cache.stride(2),
+            paged_cache.numel() // paged_cache.stride(2), hidden_slots.data_ptr(), hidden_seq_start.data_ptr(),
+            n_seqs, int(max_len), w_k.data_ptr(), w_v.data_ptr(), None if b_v is None else b_v.data_ptr(),
+            w_k.stride(0), heads, head_size, float(softmax_scale), out.data_ptr(), out.stride(0), out.size(0),
+            _DTYPE_CODE[q.dtype], workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream(q))
+    _lib.check(st, "absorbed_hidden_attention")
+    return out
+
+
 # ------------------------------------------------------------------ names of the operator surface
 
 def gather_hidden_blocks(holder, paged_cache, slot_mapping, dst_idx) -> None:

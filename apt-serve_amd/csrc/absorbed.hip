@@ -1,0 +1,506 @@
+// Decode attention of hidden-cached sequences computed on the cached hidden rows themselves
+// ("absorbed" projection weights), for gfx950.
+//
+// For a hidden-cached sequence the K and V of a context token are W_k h_t + b_k and W_v h_t + b_v.
+// Instead of re-projecting every cached row in every layer,
+//     s[h][t] = scale * <W_k[h]^T q[h], h_t>      (the b_k term is the same for all t: softmax drops it)
+//     out[h]  = W_v[h] (sum_t p[h][t] h_t) + b_v[h]
+// so the hidden rows are read twice (scores, then the weighted sum) and the projections shrink to
+// products with one row per sequence and head:
+//   1. qt[s][h][:]  = scale*log2(e) * W_k[h]^T q[s][h]            nn_few_rows_kernel (B = rows of W_k)
+//   2. S[s][h][t]   = <qt[s][h], h_t>                               hidden_scores_kernel (paged rows)
+//   3. P[s][h][:]   = softmax_t, 16-bit, zero padded                softmax_rows_kernel
+//   4. ctx[s][h][:] = sum_t P[s][h][t] h_t                          nn_few_rows_kernel (B = paged rows)
+//   5. out[s][h*D+d] = <W_v[h*D+d], ctx[s][h]> + b_v                the weight-streaming kernels of the
+//                                                                   projection file, x chosen per head
+// Per cached token and layer that is 2 x Hd x 2 bytes of HBM reads and ~4*H*Hd flops, against a
+// gather, a 4*Hd*Hd-flop GEMM, a cache write and an attention read for the re-projection flow.
+#include "aps_common.h"
+#include "mfma_common.h"
+
+namespace aps {
+namespace {
+
+// ------------------------------------------------------------------ NN product with few rows
+// out[z][m][n] = alpha * sum_k A[z][m][k] * B[row(z,k)][n],  m < m_rows (tiles of 16*MT rows), k < K(z).
+// B rows are n-contiguous; row(z,k) = row_ids[row_start[z] + k] (paged rows) or z*k_fixed + k.
+// A is K-contiguous and readable (finite, normally zero) up to the next multiple of 32 in k.
+//
+// The matrix core wants, per lane, 8 consecutive k of one column.  A lane therefore loads an 8x8
+// block (8 rows k, 16 bytes = 8 columns each; the 16 lanes of a quarter-wave read 256 contiguous
+// bytes of a row), transposes it in registers with v_perm_b32 and feeds 8 MFMAs, MFMA j taking
+// column 8c+j from lane (g, c).  No LDS; a workgroup of 8 wavefronts covers 1024 columns.
+struct NnArgs {
+  const char* a; int64_t a_batch_stride_b, lda_b; int m_rows;
+  const int64_t* a_row_ids; int64_t num_a_rows;  // nullable: row m of A is row a_row_ids[m] (rows of lda_b bytes)
+  const char* b; int64_t b_row_stride_b, num_b_rows;
+  const int64_t* row_ids; const int64_t* row_start; int k_fixed;
+  int64_t n;
+  char* out; int64_t out_batch_stride, out_row_stride;  // elements
+  float* partial;  // non-null: fp32 partial sums [k part][batch][m_rows][n] instead of out
+  int batches, k_per_part, m_tiles;
+  float alpha;
+};
+
+constexpr int kNnWaves = 8;
+
+template <bool BF16, int MT>
+__global__ __launch_bounds__(kNnWaves * 64) void nn_few_rows_kernel(const NnArgs g) {
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int g4 = lane >> 4, c = lane & 15;
+  const int z = blockIdx.y / g.m_tiles;
+  const int m0 = (blockIdx.y % g.m_tiles) * (16 * MT);
+  int64_t rs = 0;
+  int K = g.k_fixed;
+  if (g.row_ids) {
+    rs = g.row_start[z];
+    K = (int)(g.row_start[z + 1] - rs);
+  }
+  const int kbeg = blockIdx.z * g.k_per_part;
+  const int kend = min(K, kbeg + g.k_per_part);
+  const int64_t col0 = (int64_t)blockIdx.x * (kNnWaves * 128) + wave * 128 + 8 * c;
+  const bool col_ok = col0 < g.n;
+  const char* a_ptr[MT];
+  bool a_ok[MT];
+#pragma unroll
+  for (int ht = 0; ht < MT; ++ht) {
+    const int m = m0 + 16 * ht + c;
+    a_ok[ht] = m < g.m_rows;
+    int64_t arow = m;
+    if (a_ok[ht] && g.a_row_ids) {
+      arow = g.a_row_ids[m];
+      a_ok[ht] = arow >= 0 && arow < g.num_a_rows;
+    }
+    a_ptr[ht] = g.a + (int64_t)z * g.a_batch_stride_b + arow * g.lda_b + g4 * 16;
+  }
+  float4v acc[MT][8];
+#pragma unroll
+  for (int ht = 0; ht < MT; ++ht)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[ht][j] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  auto load_step = [&](int t0, u32x4(&r)[8], u32x4(&pf)[MT]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      r[i] = u32x4{0u, 0u, 0u, 0u};
+      const int t = t0 + 8 * g4 + i;
+      if (col_ok && t < kend) {
+        const int64_t row = g.row_ids ? g.row_ids[rs + t] : (int64_t)z * g.k_fixed + t;
+        if (row >= 0 && row < g.num_b_rows)
+          r[i] = __builtin_nontemporal_load((const u32x4*)(g.b + row * g.b_row_stride_b + col0 * 2));
+      }
+    }
+#pragma unroll
+    for (int ht = 0; ht < MT; ++ht) {
+      pf[ht] = u32x4{0u, 0u, 0u, 0u};
+      if (a_ok[ht] && t0 < kend) pf[ht] = *(const u32x4*)(a_ptr[ht] + (int64_t)t0 * 2);
+    }
+  };
+  auto mac_step = [&](const u32x4(&r)[8], const u32x4(&pf)[MT]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      // column j of the 8x8 block: dword p = (row 2p, row 2p+1)
+      u32x4 tcol;
+      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const uint32_t lo = r[2 * p][j >> 1], hi = r[2 * p + 1][j >> 1];
+        tcol[p] = __builtin_amdgcn_perm(hi, lo, sel);
+      }
+#pragma unroll
+      for (int ht = 0; ht < MT; ++ht) acc[ht][j] = mfma16<BF16>(pf[ht], tcol, acc[ht][j]);
+    }
+  };
+
+  u32x4 ra[8], rb[8], pa[MT], pb[MT];
+  int t0 = kbeg;
+  if (t0 < kend) load_step(t0, ra, pa);
+  while (t0 < kend) {
+    load_step(t0 + 32, rb, pb);
+    mac_step(ra, pa);
+    t0 += 32;
+    if (t0 >= kend) break;
+    load_step(t0 + 32, ra, pa);
+    mac_step(rb, pb);
+    t0 += 32;
+  }
+
+  // lane (g4, c) holds rows 16*ht + 4*g4 + i and columns col0 .. col0+7 (MFMA j = column j)
+  if (!col_ok) return;
+#pragma unroll
+  for (int ht = 0; ht < MT; ++ht)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + 16 * ht + 4 * g4 + i;
+      if (m >= g.m_rows) continue;
+      if (g.partial) {
+        float* dst = g.partial + (((int64_t)blockIdx.z * g.batches + z) * g.m_rows + m) * g.n + col0;
+        *(float4v*)dst = float4v{acc[ht][0][i], acc[ht][1][i], acc[ht][2][i], acc[ht][3][i]};
+        *(float4v*)(dst + 4) = float4v{acc[ht][4][i], acc[ht][5][i], acc[ht][6][i], acc[ht][7][i]};
+      } else {
+        uint16_t h[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float v = acc[ht][j][i] * g.alpha;
+          h[j] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+        }
+        u32x4 o;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) o[p] = (uint32_t)h[2 * p] | ((uint32_t)h[2 * p + 1] << 16);
+        *(u32x4*)(g.out + ((int64_t)z * g.out_batch_stride + (int64_t)m * g.out_row_stride + col0) * 2) = o;
+      }
+    }
+}
+
+// out[z][m][n] = alpha * sum_p partial[p][z][m][n], 4 columns per thread
+template <bool BF16>
+__global__ __launch_bounds__(256) void nn_reduce_kernel(const float* __restrict__ partial, char* out, int parts,
+                                                        int batches, int m_rows, int64_t n, int64_t out_batch_stride,
+                                                        int64_t out_row_stride, float alpha) {
+  const int64_t per_part = (int64_t)batches * m_rows * n;
+  const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (idx >= per_part) return;
+  float4v s = *(const float4v*)(partial + idx);
+  for (int p = 1; p < parts; ++p) {
+    const float4v v = *(const float4v*)(partial + p * per_part + idx);
+    s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
+  }
+  const int64_t col = idx % n, zm = idx / n;
+  const int64_t m = zm % m_rows, z = zm / m_rows;
+  uint16_t* o = (uint16_t*)out + z * out_batch_stride + m * out_row_stride + col;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = BF16 ? f32_to_bf16_bits(s[i] * alpha) : f32_to_f16_bits(s[i] * alpha);
+}
+
+// ------------------------------------------------------------------ scores over paged hidden rows
+// S[z][h][t] = sum_k hidden[row_ids[row_start[z] + t]][k] * qt[z][h][k]  (fp32), t < L(z).
+// One workgroup = 256 tokens of one sequence x all heads (padded to 32*NHT); K in tiles of 64 through a
+// two-stage LDS ring.  Rows are copied global -> LDS by global_load_lds_dwordx4 from per-lane row pointers
+// (8 rows x 128 B per wave-wide instruction), chunk c of row r stored at c ^ ((r >> 1) % 8) so that the
+// fragment reads are conflict-free.  8 wavefronts, 32 tokens each, MFMA 32x32x16.
+struct ScoreArgs {
+  const char* cache; int64_t slot_stride_b, num_slots;
+  const int64_t* row_ids; const int64_t* row_start;
+  const char* qt; int64_t qt_batch_stride_b, qt_row_stride_b; int heads;
+  float* s; int64_t s_batch_stride, s_row_stride;  // elements
+  int64_t k;
+};
+
+constexpr int kScTokens = 256, kScBK = 64, kScThreads = 512;
+
+template <bool BF16, int NHT>
+__global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreArgs g) {
+  constexpr int kATile = kScTokens * kScBK * 2;  // 32 KiB
+  constexpr int kBGroups = NHT * 4;              // groups of 8 head rows (1 KiB each)
+  constexpr int kBPerWave = (kBGroups + 7) / 8;
+  constexpr int kBTile = kBPerWave * 8 * 1024;   // every wavefront copies kBPerWave groups, real or dummy
+  constexpr int kStage = kATile + kBTile;
+  __shared__ __attribute__((aligned(1024))) char lds[2 * kStage];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int z = blockIdx.y;
+  const int64_t rs = g.row_start[z];
+  const int L = (int)(g.row_start[z + 1] - rs);
+  const int tile0 = blockIdx.x * kScTokens;
+  if (tile0 >= L) return;
+
+  // DMA sources: 4 groups of 8 token rows per wavefront; lane -> row lane/8, chunk (lane%8) ^ swizzle(row)
+  // Every wavefront issues the same number of copies per tile (the wait counts below rely on it): rows past
+  // the sequence, padding slots and head rows past the last head read slot 0 / head 0 instead; what they
+  // produce is never stored.
+  const char* a_src[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = (wave * 4 + j) * 8 + (lane >> 3);
+    const int t = tile0 + row;
+    int64_t slot = 0;
+    if (t < L) {
+      slot = g.row_ids[rs + t];
+      if (slot < 0 || slot >= g.num_slots) slot = 0;
+    }
+    a_src[j] = g.cache + slot * g.slot_stride_b + (((lane & 7) ^ ((row >> 1) & 7)) * 16);
+  }
+  const char* b_src[kBPerWave];
+  int b_group[kBPerWave];
+#pragma unroll
+  for (int j = 0; j < kBPerWave; ++j) {
+    b_group[j] = wave + 8 * j;
+    const int row = b_group[j] * 8 + (lane >> 3);
+    const int src_row = row < g.heads ? row : 0;
+    b_src[j] = g.qt + (int64_t)z * g.qt_batch_stride_b + (int64_t)src_row * g.qt_row_stride_b +
+               (((lane & 7) ^ ((row >> 1) & 7)) * 16);
+  }
+  auto issue = [&](int kt) {
+    char* sa = lds + (kt & 1) * kStage;
+    char* sb = sa + kATile;
+    const int64_t koff = (int64_t)kt * (kScBK * 2);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[j] + koff),
+                                       (__attribute__((address_space(3))) void*)(sa + (wave * 4 + j) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < kBPerWave; ++j)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[j] + koff),
+                                       (__attribute__((address_space(3))) void*)(sb + b_group[j] * 1024), 16, 0, 0);
+  };
+
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const uint32_t a_row_off = (uint32_t)((wave * 32 + frow) * (kScBK * 2));
+  const uint32_t b_row_off = (uint32_t)(frow * (kScBK * 2));
+  uint32_t chunk_off[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) chunk_off[ks] = (uint32_t)(((2 * ks + fhalf) ^ ((frow >> 1) & 7)) * 16);
+  float16v acc[NHT];
+#pragma unroll
+  for (int nt = 0; nt < NHT; ++nt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[nt][e] = 0.f;
+
+  const int nk = (int)(g.k / kScBK);
+  issue(0);
+  if (nk > 1) issue(1);
+  for (int kt = 0; kt < nk; ++kt) {
+    // tile kt has landed when every load issued so far except tile kt+1's has: wait for all of them on the
+    // last tile, otherwise the loads of tile kt+1 (issued after those of tile kt) may stay in flight
+    if (kt + 1 < nk) {
+      if (kBPerWave == 1) APS_WAIT_VM(5); else APS_WAIT_VM(6);
+    } else {
+      APS_WAIT_VM(0);
+    }
+    APS_BARRIER();
+    const char* sa = lds + (kt & 1) * kStage;
+    const char* sb = sa + kATile;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const u32x4 af = *(const u32x4*)(sa + a_row_off + chunk_off[ks]);
+#pragma unroll
+      for (int nt = 0; nt < NHT; ++nt) {
+        const u32x4 bf = *(const u32x4*)(sb + b_row_off + nt * (32 * kScBK * 2) + chunk_off[ks]);
+        acc[nt] = mfma32<BF16>(af, bf, acc[nt]);
+      }
+    }
+    APS_WAIT_LGKM0();
+    APS_BARRIER();  // every wavefront has its fragments of tile kt: the stage can be refilled
+    if (kt + 2 < nk) issue(kt + 2);
+  }
+
+  // lane holds head nt*32 + frow and tokens 8*(e/4) + 4*fhalf + e%4 of its wavefront's 32
+#pragma unroll
+  for (int nt = 0; nt < NHT; ++nt) {
+    const int head = nt * 32 + frow;
+    if (head >= g.heads) continue;
+    float* row = g.s + (int64_t)z * g.s_batch_stride + (int64_t)head * g.s_row_stride;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int t = tile0 + wave * 32 + 8 * q + 4 * fhalf;
+      if (t < g.s_row_stride)
+        *(float4v*)(row + t) = float4v{acc[nt][4 * q], acc[nt][4 * q + 1], acc[nt][4 * q + 2], acc[nt][4 * q + 3]};
+    }
+  }
+}
+
+// ------------------------------------------------------------------ softmax over the tokens of a row
+// P[z][h][t] = exp2(S - max) / sum for t < L(z), 0 for L <= t < lp; S already carries scale*log2(e).
+template <bool BF16>
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restrict__ s, uint16_t* __restrict__ p,
+                                                           const int64_t* __restrict__ row_start, int heads,
+                                                           int64_t lp) {
+  __shared__ float red[4];
+  const int z = blockIdx.y, h = blockIdx.x;
+  const int L = (int)(row_start[z + 1] - row_start[z]);
+  const float* row = s + ((int64_t)z * heads + h) * lp;
+  uint16_t* out = p + ((int64_t)z * heads + h) * lp;
+  float mx = -INFINITY;
+  for (int t = threadIdx.x; t < L; t += 256) mx = fmaxf(mx, row[t]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  float sum = 0.f;
+  for (int t = threadIdx.x; t < L; t += 256) sum += exp2f(row[t] - mx);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = sum;
+  __syncthreads();
+  sum = (red[0] + red[1]) + (red[2] + red[3]);
+  const float inv = 1.f / sum;
+  for (int64_t t = threadIdx.x; t < lp; t += 256) {
+    const float v = t < L ? exp2f(row[t] - mx) * inv : 0.f;
+    out[t] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+  }
+}
+
+template <bool BF16>
+int launch_nn(const NnArgs& g, int kparts, hipStream_t s) {
+  const int mt = g.m_tiles > 1 ? 3 : (g.m_rows <= 16 ? 1 : (g.m_rows <= 32 ? 2 : 3));  // row tiles are 16*mt rows
+  const dim3 grid((unsigned)((g.n + kNnWaves * 128 - 1) / (kNnWaves * 128)), (unsigned)(g.batches * g.m_tiles),
+                  (unsigned)kparts);
+  if (mt == 1)
+    hipLaunchKernelGGL((nn_few_rows_kernel<BF16, 1>), grid, dim3(kNnWaves * 64), 0, s, g);
+  else if (mt == 2)
+    hipLaunchKernelGGL((nn_few_rows_kernel<BF16, 2>), grid, dim3(kNnWaves * 64), 0, s, g);
+  else
+    hipLaunchKernelGGL((nn_few_rows_kernel<BF16, 3>), grid, dim3(kNnWaves * 64), 0, s, g);
+  return launch_status();
+}
+
+inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+struct Plan {
+  int64_t lp;        // padded row length of S and P
+  int kparts;        // token partitions of the weighted sum
+  int k_per_part;
+  int64_t off_qt, off_s, off_p, off_ctx, off_partial, total;
+};
+
+Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
+  Plan p{};
+  p.lp = align_up(max_len > 0 ? max_len : 1, 32);
+  const int64_t col_tiles = (hidden + kNnWaves * 128 - 1) / (kNnWaves * 128);
+  int64_t parts = 1;
+  // few sequences: split the tokens so that about two workgroups per CU exist
+  while (n_seqs * col_tiles * parts < 512 && p.lp / (parts * 2) >= 64) parts *= 2;
+  p.k_per_part = (int)align_up((p.lp + parts - 1) / parts, 32);
+  p.kparts = (int)((p.lp + p.k_per_part - 1) / p.k_per_part);
+  int64_t o = 0;
+  p.off_qt = o; o += align_up(n_seqs * heads * hidden * 2, 256);
+  p.off_s = o; o += align_up(n_seqs * heads * p.lp * 4, 256);
+  p.off_p = o; o += align_up(n_seqs * heads * p.lp * 2, 256);
+  p.off_ctx = o; o += align_up(n_seqs * heads * hidden * 2, 256);
+  p.off_partial = o;
+  if (p.kparts > 1) o += align_up((int64_t)p.kparts * n_seqs * heads * hidden * 4, 256);
+  p.total = o;
+  return p;
+}
+
+}  // namespace
+}  // namespace aps
+
+using namespace aps;
+
+// the per-head value projection lives with the other weight-streaming kernels
+int aps_internal_headwise_linear(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n,
+                                 int64_t k, int64_t x_stride, int64_t x_head_stride, int head_rows, int64_t w_stride,
+                                 int64_t out_stride, const int64_t* out_row_map, int64_t out_rows, int dtype,
+                                 hipStream_t stream);
+
+extern "C" {
+
+int64_t aps_absorbed_attention_workspace_bytes(int64_t n_seqs, int64_t max_len, int num_heads, int head_size) {
+  if (n_seqs <= 0 || max_len <= 0 || num_heads <= 0 || head_size <= 0) return 0;
+  return make_plan(n_seqs, max_len, num_heads, (int64_t)num_heads * head_size).total;
+}
+
+int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_rows, int64_t num_q_rows,
+                           const void* paged_cache, int64_t slot_stride, int64_t num_slots,
+                           const int64_t* hidden_slots, const int64_t* seq_start, int64_t n_seqs, int64_t max_len,
+                           const void* w_k, const void* w_v, const void* b_v, int64_t w_stride, int num_heads,
+                           int head_size, float softmax_scale, void* out, int64_t out_stride, int64_t out_rows,
+                           int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream) {
+  if (n_seqs < 0 || max_len < 0 || num_heads <= 0 || head_size <= 0) return APS_ERR_INVALID_ARG;
+  if (n_seqs == 0) return APS_OK;
+  if (!q || !seq_rows || !paged_cache || !hidden_slots || !seq_start || !w_k || !w_v || !out || !workspace)
+    return APS_ERR_INVALID_ARG;
+  if (dtype != APS_F16 && dtype != APS_BF16) return APS_ERR_UNSUPPORTED;
+  const int64_t hidden = (int64_t)num_heads * head_size;
+  if (head_size % 32 != 0 || hidden % 64 != 0 || num_heads > 96) return APS_ERR_UNSUPPORTED;
+  if (q_stride < hidden || slot_stride < hidden || w_stride < hidden || out_stride < hidden) return APS_ERR_INVALID_ARG;
+  if (common_vec_bytes({addr(q), addr(paged_cache), addr(w_k), addr(w_v), addr(out), addr(workspace),
+                        (uint64_t)q_stride * 2, (uint64_t)slot_stride * 2, (uint64_t)w_stride * 2,
+                        (uint64_t)out_stride * 2}) != 16)
+    return APS_ERR_UNSUPPORTED;
+  if (n_seqs > 65535 || max_len > ((int64_t)1 << 24)) return APS_ERR_UNSUPPORTED;
+  const Plan p = make_plan(n_seqs, max_len, num_heads, hidden);
+  if (workspace_bytes < p.total) return APS_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  const bool bf16 = dtype == APS_BF16;
+  char* ws = (char*)workspace;
+  char* qt = ws + p.off_qt;
+  float* sc = (float*)(ws + p.off_s);
+  char* pr = ws + p.off_p;
+  char* ctx = ws + p.off_ctx;
+  float* partial = (float*)(ws + p.off_partial);
+
+  // 1. qt[s][h][:] = scale*log2(e) * W_k[h]^T q[seq_rows[s]][h]: batch = head, K = head_size, B = rows of W_k
+  {
+    NnArgs g{};
+    g.a = (const char*)q; g.a_batch_stride_b = (int64_t)head_size * 2; g.lda_b = q_stride * 2;
+    g.m_rows = (int)n_seqs; g.a_row_ids = seq_rows; g.num_a_rows = num_q_rows;
+    g.b = (const char*)w_k; g.b_row_stride_b = w_stride * 2; g.num_b_rows = hidden;
+    g.row_ids = nullptr; g.row_start = nullptr; g.k_fixed = head_size;
+    g.n = hidden;
+    g.out = qt; g.out_batch_stride = hidden; g.out_row_stride = (int64_t)num_heads * hidden;
+    g.partial = nullptr; g.batches = num_heads; g.k_per_part = head_size;
+    g.m_tiles = (int)((n_seqs + 47) / 48);
+    g.alpha = softmax_scale * 1.4426950408889634f;
+    const int st = bf16 ? launch_nn<true>(g, 1, s) : launch_nn<false>(g, 1, s);
+    if (st != APS_OK) return st;
+  }
+  // 2. S[s][h][t] = <qt[s][h], hidden row t of sequence s>
+  {
+    ScoreArgs g{};
+    g.cache = (const char*)paged_cache; g.slot_stride_b = slot_stride * 2; g.num_slots = num_slots;
+    g.row_ids = hidden_slots; g.row_start = seq_start;
+    g.qt = qt; g.qt_batch_stride_b = (int64_t)num_heads * hidden * 2; g.qt_row_stride_b = hidden * 2;
+    g.heads = num_heads;
+    g.s = sc; g.s_batch_stride = (int64_t)num_heads * p.lp; g.s_row_stride = p.lp;
+    g.k = hidden;
+    const dim3 grid((unsigned)((max_len + kScTokens - 1) / kScTokens), (unsigned)n_seqs);
+    const int nht = (num_heads + 31) / 32;
+#define APS_LAUNCH_SCORES(B, N) hipLaunchKernelGGL((hidden_scores_kernel<B, N>), grid, dim3(kScThreads), 0, s, g)
+    if (bf16) {
+      if (nht == 1) APS_LAUNCH_SCORES(true, 1); else if (nht == 2) APS_LAUNCH_SCORES(true, 2); else APS_LAUNCH_SCORES(true, 3);
+    } else {
+      if (nht == 1) APS_LAUNCH_SCORES(false, 1); else if (nht == 2) APS_LAUNCH_SCORES(false, 2); else APS_LAUNCH_SCORES(false, 3);
+    }
+#undef APS_LAUNCH_SCORES
+    const int st = launch_status();
+    if (st != APS_OK) return st;
+  }
+  // 3. P = softmax over the tokens, zero padded to lp
+  {
+    const dim3 grid((unsigned)num_heads, (unsigned)n_seqs);
+    if (bf16)
+      hipLaunchKernelGGL(softmax_rows_kernel<true>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp);
+    else
+      hipLaunchKernelGGL(softmax_rows_kernel<false>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp);
+    const int st = launch_status();
+    if (st != APS_OK) return st;
+  }
+  // 4. ctx[s][h][:] = sum_t P[s][h][t] * hidden row t: batch = sequence, K = its length, B = paged rows
+  {
+    NnArgs g{};
+    g.a = pr; g.a_batch_stride_b = (int64_t)num_heads * p.lp * 2; g.lda_b = p.lp * 2;
+    g.m_rows = num_heads; g.a_row_ids = nullptr; g.num_a_rows = num_heads;
+    g.b = (const char*)paged_cache; g.b_row_stride_b = slot_stride * 2; g.num_b_rows = num_slots;
+    g.row_ids = hidden_slots; g.row_start = seq_start; g.k_fixed = 0;
+    g.n = hidden;
+    g.out = ctx; g.out_batch_stride = (int64_t)num_heads * hidden; g.out_row_stride = hidden;
+    g.partial = p.kparts > 1 ? partial : nullptr;
+    g.batches = (int)n_seqs; g.k_per_part = p.k_per_part;
+    g.m_tiles = (num_heads + 47) / 48;
+    g.alpha = 1.f;
+    int st = bf16 ? launch_nn<true>(g, p.kparts, s) : launch_nn<false>(g, p.kparts, s);
+    if (st != APS_OK) return st;
+    if (p.kparts > 1) {
+      const int64_t quads = n_seqs * num_heads * hidden / 4;
+      const dim3 rgrid((unsigned)((quads + 255) / 256));
+      if (bf16)
+        hipLaunchKernelGGL(nn_reduce_kernel<true>, rgrid, dim3(256), 0, s, partial, ctx, p.kparts, (int)n_seqs,
+                           num_heads, hidden, g.out_batch_stride, g.out_row_stride, 1.f);
+      else
+        hipLaunchKernelGGL(nn_reduce_kernel<false>, rgrid, dim3(256), 0, s, partial, ctx, p.kparts, (int)n_seqs,
+                           num_heads, hidden, g.out_batch_stride, g.out_row_stride, 1.f);
+      st = launch_status();
+      if (st != APS_OK) return st;
+    }
+  }
+  // 5. out[seq_rows[s]][h*D + d] = <W_v[h*D + d], ctx[s][h]> + b_v
+  return aps_internal_headwise_linear(ctx, w_v, b_v, out, n_seqs, hidden, hidden, (int64_t)num_heads * hidden, hidden,
+                                      head_size, w_stride, out_stride, seq_rows, out_rows, dtype, s);
+}
+
+}  // extern "C"

@@ -60,6 +60,7 @@ struct MetaArgs {
   int64_t* hidden_cache_use_input; int64_t* hidden_cache_store_tot;
   int64_t* hidden_holder_upd; int64_t* hidden_holder_pull; int64_t* holder_src; int64_t* kv_dest;
   uint8_t* token_is_hidden;
+  int64_t* hidden_slots; int64_t* hidden_seq_start;
   int32_t* block_tables_out; int64_t out_stride; int out_width;
   int32_t* seq_start_loc; int32_t* query_start_loc; int32_t* context_lens_out; int64_t* input_positions;
   int64_t* totals;
@@ -101,6 +102,7 @@ __global__ __launch_bounds__(kThreads) void decode_metadata_kernel(const MetaArg
       if (h0 + j < a.cap_hidden_rows) {
         a.slot_mapping_shared[h0 + j] = shared_slot;
         a.hidden_cache_use_tot[h0 + j] = row0 + j;
+        if (a.hidden_slots) a.hidden_slots[h0 + j] = slot_of(bt, a.table_width, j, a.block_size);
       }
       if (j < L - 1 && pull0 + j < a.cap_rows - a.batch) a.hidden_holder_pull[pull0 + j] = row0 + j;
     }
@@ -109,6 +111,10 @@ __global__ __launch_bounds__(kThreads) void decode_metadata_kernel(const MetaArg
       if (pre.hidden_seqs < a.cap_hidden_seqs) {
         a.hidden_cache_use_input[pre.hidden_seqs] = b;
         a.hidden_cache_store_tot[pre.hidden_seqs] = row0 + L - 1;
+        if (a.hidden_seq_start) {
+          a.hidden_seq_start[pre.hidden_seqs] = h0;
+          a.hidden_seq_start[pre.hidden_seqs + 1] = h0 + L;  // the next hidden sequence writes the same value
+        }
       }
     }
   } else if (threadIdx.x == 0) {
@@ -203,7 +209,8 @@ int aps_build_decode_metadata(const int32_t* seq_lens, const int32_t* use_hidden
                               int64_t* kv_cache_use_tot, int64_t* hidden_cache_use_input,
                               int64_t* hidden_cache_store_tot, int64_t* hidden_holder_upd,
                               int64_t* hidden_holder_pull, int64_t* holder_src, int64_t* kv_dest,
-                              int64_t cap_rows, int64_t cap_hidden_rows,
+                              int64_t* hidden_slots, int64_t* hidden_seq_start, int64_t cap_rows,
+                              int64_t cap_hidden_rows,
                               int64_t cap_hidden_seqs, int64_t cap_kv_seqs, int32_t* block_tables_out,
                               int64_t out_stride, int64_t out_width, int32_t* seq_start_loc,
                               int32_t* query_start_loc, int32_t* context_lens, int64_t* input_positions,
@@ -232,6 +239,7 @@ int aps_build_decode_metadata(const int32_t* seq_lens, const int32_t* use_hidden
   a.hidden_cache_use_tot = hidden_cache_use_tot; a.kv_cache_use_tot = kv_cache_use_tot;
   a.hidden_cache_use_input = hidden_cache_use_input; a.hidden_cache_store_tot = hidden_cache_store_tot;
   a.hidden_holder_upd = hidden_holder_upd; a.hidden_holder_pull = hidden_holder_pull; a.holder_src = holder_src; a.kv_dest = kv_dest;
+  a.hidden_slots = hidden_slots; a.hidden_seq_start = hidden_seq_start;
   a.block_tables_out = block_tables_out; a.out_stride = out_stride; a.out_width = (int)out_width;
   a.seq_start_loc = seq_start_loc; a.query_start_loc = query_start_loc; a.context_lens_out = context_lens;
   a.input_positions = input_positions; a.totals = totals;

@@ -1,0 +1,61 @@
+// Shared pieces of the matrix-core kernels (gfx950): operand vector types, MFMA wrappers,
+// buffer descriptors, rounding to the 16-bit output types, hand-placed wait points.
+#pragma once
+#include "aps_common.h"
+
+namespace aps {
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
+  const uint32_t n = bytes > 0xffffffffll ? 0xffffffffu : (uint32_t)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, n, 0x00020000);
+}
+
+template <bool BF16>
+__device__ __forceinline__ float16v mfma32(const u32x4& a, const u32x4& b, const float16v& c) {
+  if constexpr (BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                   0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0,
+                                                  0);
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
+  uint32_t u = __float_as_uint(x);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+// Hand-placed wait points: a __syncthreads() would add fences that wait for every outstanding DMA load.
+#define APS_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
+#define APS_WAIT_LGKM0() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
+#define APS_BARRIER() asm volatile("s_barrier" ::: "memory")
+
+template <bool BF16>
+__device__ __forceinline__ float4v mfma16(const u32x4& a, const u32x4& b, const float4v& c) {
+  if constexpr (BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                   0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0,
+                                                  0);
+}
+
+template <bool BF16>
+__device__ __forceinline__ float load_16bit_as_f32(const void* p, int64_t i) {
+  const uint16_t v = ((const uint16_t*)p)[i];
+  return BF16 ? __uint_as_float((uint32_t)v << 16) : (float)__builtin_bit_cast(_Float16, v);
+}
+
+}  // namespace
+}  // namespace aps

@@ -34,14 +34,10 @@
 // Workgroups are renumbered so that the 32 workgroups an XCD runs together
 // form an 8 x 4 block of tiles and share their A and W panels in that XCD's L2.
 #include "aps_common.h"
+#include "mfma_common.h"
 
 namespace aps {
 namespace {
-
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float float16v __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int kThreads = 512;
@@ -94,39 +90,15 @@ struct GemmArgs {
   int64_t m, n, k;
   int tiles_m, tiles_n;
   OutMap out;
+  // weight-streaming kernels only: weight rows come in groups of head_rows (a head); the rows of group h are
+  // multiplied with x[m] + h * x_head_stride_b instead of x[m] (0: one x for all rows)
+  int64_t x_head_stride_b;
+  int head_rows;
   // split-K (small M): workgroup (tile, z) handles k-tiles [z*kt_per_split, ...) and stores its fp32
   // partial tile to partial[z][m][n]; a second kernel adds the splits and the bias
   float* partial;
   int kt_per_split;
 };
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
-  const uint32_t n = bytes > 0xffffffffll ? 0xffffffffu : (uint32_t)bytes;
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, n, 0x00020000);
-}
-
-template <bool BF16>
-__device__ __forceinline__ float16v mfma32(const u32x4& a, const u32x4& b, const float16v& c) {
-  if constexpr (BF16)
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
-                                                   0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0,
-                                                  0);
-}
-
-__device__ __forceinline__ uint16_t f32_to_f16_bits(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }
-__device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
-  uint32_t u = __float_as_uint(x);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
-}
-
-// Hand-placed wait points: a __syncthreads() would add fences that wait for every outstanding DMA load.
-#define APS_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
-#define APS_WAIT_LGKM0() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
-#define APS_BARRIER() asm volatile("s_barrier" ::: "memory")
 
 template <bool BF16>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_nt_kernel(
@@ -329,18 +301,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 // (lane l: row l%16, k-chunk l/16 of 8 elements) and the <=16 activation rows as B (rows beyond m read
 // as zero through the buffer bounds); the 8 partial 16x16 results are added in LDS in a fixed order.
 // No workspace and no second launch; every lane keeps up to 2 x kSkU 16-byte weight loads in flight.
-typedef float float4v __attribute__((ext_vector_type(4)));
 constexpr int kSkWaves = 8, kSkU = 8;
-
-template <bool BF16>
-__device__ __forceinline__ float4v mfma16(const u32x4& a, const u32x4& b, const float4v& c) {
-  if constexpr (BF16)
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
-                                                   0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0,
-                                                  0);
-}
 
 template <bool BF16>
 __global__ __launch_bounds__(kSkWaves * 64) void skinny_nt_kernel(const GemmArgs g, int steps_per_wave) {
@@ -348,8 +309,10 @@ __global__ __launch_bounds__(kSkWaves * 64) void skinny_nt_kernel(const GemmArgs
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int64_t n0 = (int64_t)blockIdx.x * 16;
+  const int64_t m0 = (int64_t)blockIdx.y * 16;  // 16 activation rows per workgroup row
   const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(g.w + n0 * g.ldw_b, (g.n - n0) * g.ldw_b);
-  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(g.a, g.m * g.lda_b);
+  const int64_t x_head_b = g.head_rows ? (n0 / g.head_rows) * g.x_head_stride_b : 0;
+  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(g.a + m0 * g.lda_b + x_head_b, (g.m - m0) * g.lda_b - x_head_b);
   const int row = lane & 15, kg = lane >> 4;
   const uint32_t voff_w = (uint32_t)(row * g.ldw_b + kg * 16);
   const uint32_t voff_x = (uint32_t)(row * g.lda_b + kg * 16);  // rows >= m are out of bounds: zero
@@ -394,7 +357,7 @@ __global__ __launch_bounds__(kSkWaves * 64) void skinny_nt_kernel(const GemmArgs
     sum[0] += p[0]; sum[1] += p[1]; sum[2] += p[2]; sum[3] += p[3];
   }
   // lane l holds out[token l%16][n0 + 4*(l/16) + i], i = 0..3
-  const int64_t token = row;
+  const int64_t token = m0 + row;
   if (token >= g.m) return;
   const int64_t n = n0 + 4 * kg;
   const int half = (g.out.n_split && n >= g.out.n_split) ? 1 : 0;
@@ -463,7 +426,9 @@ __global__ __launch_bounds__(kRsWaves * 64) void rowstream_nt_kernel(const GemmA
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int64_t n_first = ((int64_t)blockIdx.x * kRsWaves + wave) * kRsRows;
   const char* wrow = g.w + n_first * g.ldw_b + lane * 16;
-  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(g.a, g.m * g.lda_b);
+  const int64_t x_head_b =
+      g.head_rows ? (((int64_t)blockIdx.x * kRsWaves * kRsRows) / g.head_rows) * g.x_head_stride_b : 0;
+  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(g.a + x_head_b, g.m * g.lda_b - x_head_b);
   float acc[kRsRows][MT];
 #pragma unroll
   for (int i = 0; i < kRsRows; ++i)
@@ -684,6 +649,40 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
                        splits);
   return launch_status();
 }
+
+}  // extern "C"
+
+// out[map[m]][n] = <weight[n], x[m] + (n / head_rows) * x_head_stride> + bias[n]: the value projection of the
+// absorbed attention, where the rows of head h multiply that head's context vector.  Any m: at most 8 rows
+// stream the weights through the dot kernel, more go through the MFMA kernel in tiles of 16 rows.
+int aps_internal_headwise_linear(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n,
+                                 int64_t k, int64_t x_stride, int64_t x_head_stride, int head_rows, int64_t w_stride,
+                                 int64_t out_stride, const int64_t* out_row_map, int64_t out_rows, int dtype,
+                                 hipStream_t s) {
+  if (m <= 0) return APS_OK;
+  if (n % 16 != 0 || k % 64 != 0 || head_rows % 16 != 0) return APS_ERR_UNSUPPORTED;
+  if (x_stride * 2 * 16 >= ((int64_t)1 << 31) || w_stride * 2 * 16 >= ((int64_t)1 << 31)) return APS_ERR_UNSUPPORTED;
+  GemmArgs g{};
+  g.a = (const char*)x; g.w = (const char*)weight; g.bias = bias;
+  g.lda_b = x_stride * 2; g.ldw_b = w_stride * 2;
+  g.m = m; g.n = n; g.k = k;
+  g.out.base[0] = (char*)out; g.out.ld = out_stride; g.out.n_split = 0;
+  g.out.map = out_row_map; g.out.limit0 = out_rows;
+  g.out.aligned16 = common_vec_bytes({addr(out), (uint64_t)out_stride * 2}) == 16;
+  g.x_head_stride_b = x_head_stride * 2; g.head_rows = head_rows;
+  if (m <= 8 && n % (kRsWaves * kRsRows) == 0)
+    return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
+  const int steps = (int)(k / 32);
+  const int per_wave = (steps + kSkWaves - 1) / kSkWaves;
+  const dim3 grid((unsigned)(n / 16), (unsigned)((m + 15) / 16));
+  if (dtype == APS_BF16)
+    hipLaunchKernelGGL(skinny_nt_kernel<true>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
+  else
+    hipLaunchKernelGGL(skinny_nt_kernel<false>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
+  return launch_status();
+}
+
+extern "C" {
 
 int aps_linear_nt(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n, int64_t k,
                   int64_t x_stride, int64_t w_stride, int64_t out_stride, const int64_t* out_row_map,

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define APS_ABI_VERSION 2
+#define APS_ABI_VERSION 3
 
 typedef void* aps_stream_t; /* a hipStream_t; NULL = the null stream */
 
@@ -272,6 +272,9 @@ int aps_varlen_prefill_attention(void* out, const void* q, const void* k,
  *   hidden_cache_store_tot   their newest rows
  *   holder_src[row]          (nullable, not in the reference) resolved source of the row for
  *                            aps_gather_hidden_rows: slot, -(b+1) for the newest row, INT64_MIN for padding
+ *   hidden_slots[i]          (nullable, not in the reference) private slot of hidden row i, in the order of
+ *                            hidden_cache_use_tot; hidden_seq_start[j] (nullable, n hidden sequences + 1
+ *                            entries) first hidden row of the j-th hidden sequence: aps_absorbed_attention
  *   kv_dest[row]             (nullable, not in the reference) where the row's re-projected K/V go, for
  *                            aps_kv_reproject_to_cache: shared slot (hidden rows), -(private slot + 2)
  *                            (the new token of a K/V sequence), -1 for padding
@@ -287,7 +290,8 @@ int aps_build_decode_metadata(
     int64_t* kv_cache_use_tot, int64_t* hidden_cache_use_input,
     int64_t* hidden_cache_store_tot, int64_t* hidden_holder_upd,
     int64_t* hidden_holder_pull, int64_t* holder_src, int64_t* kv_dest,
-    int64_t cap_rows, int64_t cap_hidden_rows,
+    int64_t* hidden_slots, int64_t* hidden_seq_start, int64_t cap_rows,
+    int64_t cap_hidden_rows,
     int64_t cap_hidden_seqs, int64_t cap_kv_seqs, int32_t* block_tables_out,
     int64_t out_stride, int64_t out_width, int32_t* seq_start_loc,
     int32_t* query_start_loc, int32_t* context_lens, int64_t* input_positions,
@@ -360,6 +364,39 @@ int aps_kv_reproject_to_cache(
     int64_t w_stride, int64_t slot_stride, int64_t ws_slots,
     int64_t cache_slots, int dtype, void* workspace, int64_t workspace_bytes,
     aps_stream_t stream);
+
+/* Decode attention of hidden-cached sequences on their cached hidden rows, the
+ * projections absorbed into the query and the output ("next" item 2 of the
+ * hybrid path; replaces, for those sequences, the holder gather
+ * model_executor/models/aptserve_opt.py:112-121, the kv_only re-projection
+ * :123-124, mixed_kv_to_cache and the attention over the shared cache
+ * attention/backends/aptserve_flash_attn.py:359-373, :464-473):
+ *   s[h][t] = scale * <W_k[h]^T q[h], hidden_t>;  p = softmax_t(s)
+ *   out[h]  = W_v[h] (sum_t p[h][t] hidden_t) + b_v[h]
+ * (the key bias adds the same amount to every score of a head and drops out).
+ *   q [num_q_rows, H*D] (row stride q_stride): query rows of the batch; sequence
+ *     i of the n_seqs hidden-cached ones uses row seq_rows[i] and its result is
+ *     stored at out[seq_rows[i]] (rows of out_stride elements, < out_rows).
+ *   hidden_slots[seq_start[i] .. seq_start[i+1]) : slot of every cached row of
+ *     sequence i in the flattened paged cache (row = paged_cache + slot *
+ *     slot_stride), oldest first, the newest row included (it must have been
+ *     stored already); both written by aps_build_decode_metadata.
+ *   w_k, w_v [H*D, H*D] row-major [out, in] with row stride w_stride (row
+ *     slices of the fused QKV weight); b_v nullable.
+ *   max_len >= the longest sequence.  f16 / bf16; head_size % 32 == 0.
+ * workspace: aps_absorbed_attention_workspace_bytes(...) bytes, 16-byte
+ * aligned, owned by the caller (query images, fp32 scores, probabilities,
+ * per-head context vectors). */
+int64_t aps_absorbed_attention_workspace_bytes(int64_t n_seqs, int64_t max_len,
+                                               int num_heads, int head_size);
+int aps_absorbed_attention(
+    const void* q, int64_t q_stride, const int64_t* seq_rows,
+    int64_t num_q_rows, const void* paged_cache, int64_t slot_stride,
+    int64_t num_slots, const int64_t* hidden_slots, const int64_t* seq_start,
+    int64_t n_seqs, int64_t max_len, const void* w_k, const void* w_v,
+    const void* b_v, int64_t w_stride, int num_heads, int head_size,
+    float softmax_scale, void* out, int64_t out_stride, int64_t out_rows,
+    int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream);
 
 /* Plain device copy of nbytes (16-byte aligned pointers): the known-size
  * kernel that hardware counters of the kernels above are scaled against. */

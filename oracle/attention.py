@@ -105,3 +105,38 @@ def varlen_causal_attention(q, k, v, cu_seqlens, softmax_scale):
         p = torch.softmax(s, dim=-1)
         out[a:e] = torch.einsum("hqk,khd->qhd", p, vf)
     return out
+
+
+def absorbed_hidden_attention(q, hidden_rows, w_k, w_v, b_v, softmax_scale):
+    """Decode attention of ONE hidden-cached sequence computed on its cached hidden rows,
+    without materialising K and V ("absorbed" projection weights).
+
+    The reference re-projects the whole context every layer
+    (additional_designs/model_executor/models/aptserve_opt.py:118-124:
+    ``k_t = W_k h_t + b_k``, ``v_t = W_v h_t + b_v``) and then attends
+    (aptserve_flash_attn.py:464-473).  Per head ``h`` with ``W_k[h], W_v[h]`` the ``[D, Hd]``
+    row blocks of the projection weights:
+
+        s[h, t]  = scale * <q[h], W_k[h] h_t + b_k[h]>
+                 = scale * <W_k[h]^T q[h], h_t>  +  (a term that does not depend on t)
+        p[h, :]  = softmax_t(s[h, :])            (shift invariant: the b_k term drops out)
+        out[h]   = sum_t p[h, t] (W_v[h] h_t + b_v[h]) = W_v[h] (sum_t p[h, t] h_t) + b_v[h]
+
+    ``q [H, D]``, ``hidden_rows [L, Hd]``, ``w_k``/``w_v [H*D, Hd]``, ``b_v [H*D]`` or None;
+    float64 result ``[H, D]``.  Pinned in tests against ``paged_decode_attention`` applied to
+    the re-projected K/V of the same rows.
+    """
+    h_cnt, d = q.shape
+    hd = hidden_rows.shape[1]
+    q64 = q.to(torch.float64)
+    x = hidden_rows.to(torch.float64)
+    wk = w_k.to(torch.float64).view(h_cnt, d, hd)
+    wv = w_v.to(torch.float64).view(h_cnt, d, hd)
+    qt = torch.einsum("hd,hdn->hn", q64, wk) * softmax_scale          # [H, Hd]
+    s = qt @ x.t()                                                     # [H, L]
+    p = torch.softmax(s, dim=-1)
+    ctx = p @ x                                                        # [H, Hd]
+    out = torch.einsum("hdn,hn->hd", wv, ctx)
+    if b_v is not None:
+        out = out + b_v.to(torch.float64).view(h_cnt, d)
+    return out

@@ -200,3 +200,29 @@ def test_fp8_quantize_agrees_with_torch_cast_after_clamp():
         assert torch.equal(ours, y)
         back = O8.dequantize_e4m3(ours, scale)
         assert torch.equal(back, y.view(torch.float8_e4m3fn).float() * scale)
+
+
+@pytest.mark.parametrize("L", [1, 5, 33])
+def test_absorbed_attention_equals_attention_over_reprojected_kv(L):
+    """The absorbed form is an algebraic rearrangement: it must agree with the textbook softmax
+    attention over k_t = W_k h_t + b_k, v_t = W_v h_t + b_v to float64 rounding, for any b_k."""
+    H, D = 3, 8
+    Hd = H * D
+    g = torch.Generator().manual_seed(L)
+    q = torch.randn(H, D, generator=g, dtype=torch.float64)
+    x = torch.randn(L, Hd, generator=g, dtype=torch.float64)
+    wk, wv = (torch.randn(Hd, Hd, generator=g, dtype=torch.float64) * 0.3 for _ in range(2))
+    bk, bv = (torch.randn(Hd, generator=g, dtype=torch.float64) for _ in range(2))
+    scale = 0.37
+    k = (x @ wk.t() + bk).view(L, H, D)
+    v = (x @ wv.t() + bv).view(L, H, D)
+    ref = torch.empty(H, D, dtype=torch.float64)
+    for h in range(H):
+        p = torch.softmax(scale * (k[:, h] @ q[h]), dim=0)
+        ref[h] = p @ v[:, h]
+    got = OA.absorbed_hidden_attention(q, x, wk, wv, bv, scale)
+    assert torch.allclose(got, ref, atol=1e-11, rtol=1e-11)
+    # a dropped bias term or a transposed weight block would show here
+    assert not torch.allclose(OA.absorbed_hidden_attention(q, x, wk, wv, None, scale), ref, atol=1e-3)
+    if L > 1:
+        assert not torch.allclose(OA.absorbed_hidden_attention(q, x, wk.t().contiguous(), wv, bv, scale), ref, atol=1e-3)
