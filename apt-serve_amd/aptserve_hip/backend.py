@@ -183,7 +183,7 @@ class HybridOPTAttention:
 
     def __init__(self, embed_dim: int, num_heads: int, qkv_weight, qkv_bias, out_weight, out_bias, *,
                  fused: bool = True, literal: bool = False, prefill_attention: Optional[Callable] = None,
-                 fuse_kv_write: bool = True) -> None:
+                 fuse_kv_write: bool = True, absorbed: bool = False) -> None:
         self.embed_dim, self.num_heads = embed_dim, num_heads
         self.head_dim = embed_dim // num_heads
         self.scaling = self.head_dim ** -0.5
@@ -191,12 +191,42 @@ class HybridOPTAttention:
         self.out_weight, self.out_bias = out_weight, out_bias
         self.fused = fused
         self.fuse_kv_write = fuse_kv_write and fused and not literal
+        self.absorbed = absorbed and not literal
         self.attn = HybridAttentionImpl(num_heads, self.head_dim, self.scaling, literal=literal,
                                         prefill_attention=prefill_attention)
+
+    def _forward_absorbed(self, hidden_states, kv_cache, md: HybridAttentionMetadata):
+        """Decode step without re-projection: hidden-cached sequences attend on their cached hidden rows
+        (projection weights absorbed), K/V-cached sequences on their private cache."""
+        w, b = self.qkv_proj.weight, self.qkv_proj.bias
+        s = w.shape[0] // 3
+        H, D = self.num_heads, self.head_dim
+        # the newest hidden row of every hidden-cached sequence joins its cache first
+        ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
+                            md.hidden_cache_store_tot)
+        n_kv = md.num_decode_tokens - md.num_hidden_cache_tokens
+        attn_output = torch.empty_like(hidden_states)
+        if n_kv:
+            qkv, _ = self.qkv_proj(hidden_states)
+            q, k, v = qkv.chunk(chunks=3, dim=-1)
+            ops.reshape_and_cache_flash(k, v, kv_cache[0], kv_cache[1], md.new_token_slot, "auto",
+                                        token_idx=md.kv_cache_use_input)
+            ops.paged_decode_attention(q.view(-1, H, D), kv_cache[0], kv_cache[1], md.private_block_tables,
+                                       md.kv_seq_lens, self.scaling, max_seq_len=md.max_kv_seq_len or None,
+                                       out=attn_output.view(-1, H, D))
+        else:
+            q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
+        ops.absorbed_hidden_attention(q, kv_cache, md.hidden_slots, md.hidden_seq_start, md.hidden_cache_use_input,
+                                      md.max_hidden_seq_len, w[s:2 * s], w[2 * s:], None if b is None else b[2 * s:],
+                                      self.scaling, attn_output)
+        return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
 
     def forward(self, hidden_states, kv_cache, shared_cache, attn_metadata: HybridAttentionMetadata):
         md = attn_metadata
         if md.num_hidden_cache_tokens != 0:
+            if (self.absorbed and md.num_decode_tokens != 0 and md.hidden_slots is not None and kv_cache is not None
+                    and kv_cache.dtype == hidden_states.dtype):
+                return self._forward_absorbed(hidden_states, kv_cache, md)
             if md.num_decode_tokens != 0:
                 if self.fused and md.holder_src is not None:
                     holder = torch.empty(md.num_tot_tokens, hidden_states.shape[1], device=hidden_states.device,

@@ -62,6 +62,11 @@ class HybridAttentionMetadata:
     hidden_slots: Optional[torch.Tensor] = None     # int64 [hidden rows]: private slot of every cached hidden row
     hidden_seq_start: Optional[torch.Tensor] = None  # int64 [hidden seqs + 1]: first hidden row of each hidden sequence
     max_hidden_seq_len: int = 0
+    kv_cache_use_input: Optional[torch.Tensor] = None   # int64 [kv seqs]: batch positions of K/V-cached sequences
+    new_token_slot: Optional[torch.Tensor] = None       # int64 [batch]: private slot of every sequence's newest token
+    kv_seq_lens: Optional[torch.Tensor] = None          # int32 [batch]: seq_len, 0 for hidden-cached sequences
+    max_kv_seq_len: int = 0
+    private_block_tables: Optional[torch.Tensor] = None  # int32 [batch, W]: every sequence's private table
     _cached_prefill_metadata: Optional["HybridAttentionMetadata"] = None
     _cached_decode_metadata: Optional["HybridAttentionMetadata"] = None
 
@@ -109,7 +114,10 @@ class HybridAttentionMetadata:
                 use_cuda_graph=self.use_cuda_graph, input_positions=self.input_positions,
                 block_types=None if self.block_types is None else self.block_types[self.num_prefills:],
                 holder_src=self.holder_src, kv_dest=self.kv_dest, hidden_slots=self.hidden_slots,
-                hidden_seq_start=self.hidden_seq_start, max_hidden_seq_len=self.max_hidden_seq_len)
+                hidden_seq_start=self.hidden_seq_start, max_hidden_seq_len=self.max_hidden_seq_len,
+                kv_cache_use_input=self.kv_cache_use_input, new_token_slot=self.new_token_slot,
+                kv_seq_lens=self.kv_seq_lens, max_kv_seq_len=self.max_kv_seq_len,
+                private_block_tables=self.private_block_tables)
         return self._cached_decode_metadata
 
 
@@ -226,13 +234,15 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
         d_bt = packed[2 * B:2 * B + B * W].view(B, W)
         d_bts = packed[2 * B + B * W:].view(B, Ws)
         # one allocation per output dtype
-        sizes64 = [num_tot, n_hr, n_hr, n_kv, n_hs, n_hs, B, num_tot - B, B, 4, num_tot, num_tot, n_hr, n_hs + 1]
+        sizes64 = [num_tot, n_hr, n_hr, n_kv, n_hs, n_hs, B, num_tot - B, B, 4, num_tot, num_tot, n_hr, n_hs + 1,
+                   n_kv, B]
         buf64 = torch.empty(sum(sizes64), **i64)
         (slot_mapping, slot_mapping_shared, use_tot, kv_use, use_input, store_tot, upd, pull, positions,
-         totals, holder_src, kv_dest, hidden_slots, hidden_seq_start) = torch.split(buf64, sizes64)
-        sizes32 = [B * Wo, B + 1, B + 1, B]
+         totals, holder_src, kv_dest, hidden_slots, hidden_seq_start, kv_use_input,
+         new_token_slot) = torch.split(buf64, sizes64)
+        sizes32 = [B * Wo, B + 1, B + 1, B, B]
         buf32 = torch.empty(sum(sizes32), **i32)
-        bt_out, seq_start, query_start, ctx = torch.split(buf32, sizes32)
+        bt_out, seq_start, query_start, ctx, kv_seq_lens = torch.split(buf32, sizes32)
         bt_out = bt_out.view(B, Wo)
         with torch.cuda.device(device):
             st = lib.aps_build_decode_metadata(
@@ -242,7 +252,8 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
                 kv_use.data_ptr() if n_kv else None, use_input.data_ptr() if n_hs else None,
                 store_tot.data_ptr() if n_hs else None, upd.data_ptr(), pull.data_ptr() if num_tot > B else None,
                 holder_src.data_ptr(), kv_dest.data_ptr(), hidden_slots.data_ptr() if n_hr else None,
-                hidden_seq_start.data_ptr() if n_hs else None, num_tot, n_hr, n_hs, n_kv,
+                hidden_seq_start.data_ptr() if n_hs else None, kv_use_input.data_ptr() if n_kv else None,
+                new_token_slot.data_ptr(), kv_seq_lens.data_ptr(), num_tot, n_hr, n_hs, n_kv,
                 bt_out.data_ptr() if Wo else None, Wo, Wo, seq_start.data_ptr(),
                 query_start.data_ptr(), ctx.data_ptr(), positions.data_ptr(), totals.data_ptr(),
                 torch.cuda.current_stream(device).cuda_stream)
@@ -262,7 +273,9 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
             max_decode_seq_len=int(lens.max()), query_start_loc=query_start, seq_start_loc=seq_start,
             context_lens_tensor=ctx, block_tables=bt_out, use_cuda_graph=False, input_positions=positions,
             block_types=block_types, holder_src=holder_src, kv_dest=kv_dest, hidden_slots=hidden_slots,
-            hidden_seq_start=hidden_seq_start, max_hidden_seq_len=int(lens[hid].max()) if n_hs else 0)
+            hidden_seq_start=hidden_seq_start, max_hidden_seq_len=int(lens[hid].max()) if n_hs else 0,
+            kv_cache_use_input=kv_use_input, new_token_slot=new_token_slot, kv_seq_lens=kv_seq_lens,
+            max_kv_seq_len=int(lens[~hid].max()) if n_kv else 0, private_block_tables=d_bt)
 
     # ------------------------------------------------------------------ prompts
     ctxs = np.zeros(B, dtype=np.int64) if context_lens is None else np.asarray(context_lens, dtype=np.int64)

@@ -29,7 +29,7 @@ namespace {
 // The matrix core wants, per lane, 8 consecutive k of one column.  A lane therefore loads an 8x8
 // block (8 rows k, 16 bytes = 8 columns each; the 16 lanes of a quarter-wave read 256 contiguous
 // bytes of a row), transposes it in registers with v_perm_b32 and feeds 8 MFMAs, MFMA j taking
-// column 8c+j from lane (g, c).  No LDS; a workgroup of 8 wavefronts covers 1024 columns.
+// column 8c+j from lane (g, c).  No LDS for the data; a workgroup of 4 wavefronts covers 512 columns.
 struct NnArgs {
   const char* a; int64_t a_batch_stride_b, lda_b; int m_rows;
   const int64_t* a_row_ids; int64_t num_a_rows;  // nullable: row m of A is row a_row_ids[m] (rows of lda_b bytes)
@@ -42,10 +42,13 @@ struct NnArgs {
   float alpha;
 };
 
-constexpr int kNnWaves = 8;
+constexpr int kNnWaves = 4;   // one wavefront per SIMD: the register file holds a 4-deep ring of row blocks
+constexpr int kNnRing = 4;
+constexpr int kNnMaxPart = 4096;  // rows of B per k-partition when they are addressed through row_ids
 
 template <bool BF16, int MT>
-__global__ __launch_bounds__(kNnWaves * 64) void nn_few_rows_kernel(const NnArgs g) {
+__global__ __launch_bounds__(kNnWaves * 64) __attribute__((amdgpu_waves_per_eu(1, 1))) void nn_few_rows_kernel(
+    const NnArgs g) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int g4 = lane >> 4, c = lane & 15;
@@ -59,9 +62,18 @@ __global__ __launch_bounds__(kNnWaves * 64) void nn_few_rows_kernel(const NnArgs
   }
   const int kbeg = blockIdx.z * g.k_per_part;
   const int kend = min(K, kbeg + g.k_per_part);
+  // Row ids of this partition go to LDS first: read from there they cost an LDS access instead of a global
+  // load whose result every row load would have to wait for, one after the other.
+  __shared__ __attribute__((aligned(16))) int64_t ids[kNnMaxPart];
+  if (g.row_ids) {
+    const int staged = (kend - kbeg + 31) / 32 * 32;
+    for (int i = tid; i < staged; i += kNnWaves * 64) ids[i] = kbeg + i < kend ? g.row_ids[rs + kbeg + i] : -1;
+    __syncthreads();
+  }
   const int64_t col0 = (int64_t)blockIdx.x * (kNnWaves * 128) + wave * 128 + 8 * c;
   const bool col_ok = col0 < g.n;
-  const char* a_ptr[MT];
+  const char* a_base = g.a + (int64_t)z * g.a_batch_stride_b;  // uniform; rows of a batch lie within 4 GiB of it
+  uint32_t a_off[MT];
   bool a_ok[MT];
 #pragma unroll
   for (int ht = 0; ht < MT; ++ht) {
@@ -72,7 +84,8 @@ __global__ __launch_bounds__(kNnWaves * 64) void nn_few_rows_kernel(const NnArgs
       arow = g.a_row_ids[m];
       a_ok[ht] = arow >= 0 && arow < g.num_a_rows;
     }
-    a_ptr[ht] = g.a + (int64_t)z * g.a_batch_stride_b + arow * g.lda_b + g4 * 16;
+    if (!a_ok[ht]) arow = g.a_row_ids ? 0 : m0;  // a row that exists; its product is discarded
+    a_off[ht] = (uint32_t)(arow * g.lda_b + g4 * 16);
   }
   float4v acc[MT][8];
 #pragma unroll
@@ -80,24 +93,43 @@ __global__ __launch_bounds__(kNnWaves * 64) void nn_few_rows_kernel(const NnArgs
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[ht][j] = float4v{0.f, 0.f, 0.f, 0.f};
 
-  auto load_step = [&](int t0, u32x4(&r)[8], u32x4(&pf)[MT]) {
+  // Loads are unconditional (a row or column that does not exist reads row 0 / column 0 and is replaced by
+  // zeros afterwards): with per-lane branches around them the wait counts before the MFMAs degrade to
+  // "everything outstanding", which serialises the two register sets.
+  const char* b_col = g.b + (col_ok ? col0 : 0) * 2;
+  auto load_step = [&](int t0, u32x4(&r)[8], u32x4(&pf)[MT], uint32_t& bad) {
+    int64_t row[8];
+    if (g.row_ids) {
+      const u32x4* src = (const u32x4*)(ids + (t0 - kbeg + 8 * g4));  // 8 ids = 64 bytes, 64-byte aligned
+      const u32x4 q0 = src[0], q1 = src[1], q2 = src[2], q3 = src[3];
+      row[0] = (int64_t)q0[0] | ((int64_t)q0[1] << 32); row[1] = (int64_t)q0[2] | ((int64_t)q0[3] << 32);
+      row[2] = (int64_t)q1[0] | ((int64_t)q1[1] << 32); row[3] = (int64_t)q1[2] | ((int64_t)q1[3] << 32);
+      row[4] = (int64_t)q2[0] | ((int64_t)q2[1] << 32); row[5] = (int64_t)q2[2] | ((int64_t)q2[3] << 32);
+      row[6] = (int64_t)q3[0] | ((int64_t)q3[1] << 32); row[7] = (int64_t)q3[2] | ((int64_t)q3[3] << 32);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) row[i] = (int64_t)z * g.k_fixed + t0 + 8 * g4 + i;
+    }
+    bad = 0;  // bit i: row i of this lane does not exist; applied when the block is consumed
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      r[i] = u32x4{0u, 0u, 0u, 0u};
-      const int t = t0 + 8 * g4 + i;
-      if (col_ok && t < kend) {
-        const int64_t row = g.row_ids ? g.row_ids[rs + t] : (int64_t)z * g.k_fixed + t;
-        if (row >= 0 && row < g.num_b_rows)
-          r[i] = __builtin_nontemporal_load((const u32x4*)(g.b + row * g.b_row_stride_b + col0 * 2));
-      }
+      const bool ok = col_ok && (t0 + 8 * g4 + i < kend) && row[i] >= 0 && row[i] < g.num_b_rows;
+      if (!ok) bad |= 1u << i;
+      const int64_t rr = ok ? row[i] : 0;
+      r[i] = __builtin_nontemporal_load((const u32x4*)(b_col + rr * g.b_row_stride_b));
     }
 #pragma unroll
-    for (int ht = 0; ht < MT; ++ht) {
-      pf[ht] = u32x4{0u, 0u, 0u, 0u};
-      if (a_ok[ht] && t0 < kend) pf[ht] = *(const u32x4*)(a_ptr[ht] + (int64_t)t0 * 2);
-    }
+    for (int ht = 0; ht < MT; ++ht) pf[ht] = *(const u32x4*)(a_base + (a_off[ht] + (uint32_t)t0 * 2));
   };
-  auto mac_step = [&](const u32x4(&r)[8], const u32x4(&pf)[MT]) {
+  auto mac_step = [&](u32x4(&r)[8], u32x4(&pf)[MT], uint32_t bad) {
+    if (__builtin_amdgcn_ballot_w64(bad != 0) != 0) {  // rare: the last step of a sequence
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (bad & (1u << i)) r[i] = u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int ht = 0; ht < MT; ++ht)
+      if (!a_ok[ht]) pf[ht] = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       // column j of the 8x8 block: dword p = (row 2p, row 2p+1)
@@ -113,17 +145,24 @@ __global__ __launch_bounds__(kNnWaves * 64) void nn_few_rows_kernel(const NnArgs
     }
   };
 
-  u32x4 ra[8], rb[8], pa[MT], pb[MT];
+  // ring of kNnRing row blocks: three steps (24 KiB per wavefront) are in flight while one is multiplied
+  u32x4 r[kNnRing][8], pf[kNnRing][MT];
+  uint32_t bad[kNnRing];
   int t0 = kbeg;
-  if (t0 < kend) load_step(t0, ra, pa);
+#pragma unroll
+  for (int d = 0; d < kNnRing - 1; ++d)
+    if (t0 + 32 * d < kend) load_step(t0 + 32 * d, r[d], pf[d], bad[d]);
   while (t0 < kend) {
-    load_step(t0 + 32, rb, pb);
-    mac_step(ra, pa);
-    t0 += 32;
-    if (t0 >= kend) break;
-    load_step(t0 + 32, ra, pa);
-    mac_step(rb, pb);
-    t0 += 32;
+#pragma unroll
+    for (int u = 0; u < kNnRing; ++u) {
+      if (t0 < kend) {
+        const int ahead = t0 + 32 * (kNnRing - 1);
+        if (ahead < kend) load_step(ahead, r[(u + kNnRing - 1) % kNnRing], pf[(u + kNnRing - 1) % kNnRing],
+                                    bad[(u + kNnRing - 1) % kNnRing]);
+        mac_step(r[u], pf[u], bad[u]);
+        t0 += 32;
+      }
+    }
   }
 
   // lane (g4, c) holds rows 16*ht + 4*g4 + i and columns col0 .. col0+7 (MFMA j = column j)
@@ -363,6 +402,7 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   int64_t parts = 1;
   // few sequences: split the tokens so that about two workgroups per CU exist
   while (n_seqs * col_tiles * parts < 512 && p.lp / (parts * 2) >= 64) parts *= 2;
+  while (p.lp / parts > kNnMaxPart) parts *= 2;
   p.k_per_part = (int)align_up((p.lp + parts - 1) / parts, 32);
   p.kparts = (int)((p.lp + p.k_per_part - 1) / p.k_per_part);
   int64_t o = 0;

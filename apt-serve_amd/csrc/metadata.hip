@@ -61,6 +61,7 @@ struct MetaArgs {
   int64_t* hidden_holder_upd; int64_t* hidden_holder_pull; int64_t* holder_src; int64_t* kv_dest;
   uint8_t* token_is_hidden;
   int64_t* hidden_slots; int64_t* hidden_seq_start;
+  int64_t* kv_cache_use_input; int64_t* new_token_slot; int32_t* kv_seq_lens;
   int32_t* block_tables_out; int64_t out_stride; int out_width;
   int32_t* seq_start_loc; int32_t* query_start_loc; int32_t* context_lens_out; int64_t* input_positions;
   int64_t* totals;
@@ -125,7 +126,10 @@ __global__ __launch_bounds__(kThreads) void decode_metadata_kernel(const MetaArg
       if (a.kv_dest) a.kv_dest[row0] = slot >= 0 ? -(slot + 2) : -1;
     }
     const int64_t kv_rank = b - pre.hidden_seqs;
-    if (kv_rank < a.cap_kv) a.kv_cache_use_tot[kv_rank] = row0;
+    if (kv_rank < a.cap_kv) {
+      a.kv_cache_use_tot[kv_rank] = row0;
+      if (a.kv_cache_use_input) a.kv_cache_use_input[kv_rank] = b;
+    }
     a.hidden_holder_upd[b] = row0;
   }
 
@@ -141,6 +145,8 @@ __global__ __launch_bounds__(kThreads) void decode_metadata_kernel(const MetaArg
     a.query_start_loc[b + 1] = b + 1;
     a.context_lens_out[b] = L - 1;
     a.input_positions[b] = L - 1;
+    if (a.new_token_slot) a.new_token_slot[b] = L > 0 ? slot_of(bt, a.table_width, L - 1, a.block_size) : -1;
+    if (a.kv_seq_lens) a.kv_seq_lens[b] = hid ? 0 : L;
     if (b == a.batch - 1 && a.totals) {
       a.totals[0] = pre.rows + (hid ? L : 1);
       a.totals[1] = pre.hidden_rows + (hid ? L : 0);
@@ -209,7 +215,8 @@ int aps_build_decode_metadata(const int32_t* seq_lens, const int32_t* use_hidden
                               int64_t* kv_cache_use_tot, int64_t* hidden_cache_use_input,
                               int64_t* hidden_cache_store_tot, int64_t* hidden_holder_upd,
                               int64_t* hidden_holder_pull, int64_t* holder_src, int64_t* kv_dest,
-                              int64_t* hidden_slots, int64_t* hidden_seq_start, int64_t cap_rows,
+                              int64_t* hidden_slots, int64_t* hidden_seq_start, int64_t* kv_cache_use_input,
+                              int64_t* new_token_slot, int32_t* kv_seq_lens, int64_t cap_rows,
                               int64_t cap_hidden_rows,
                               int64_t cap_hidden_seqs, int64_t cap_kv_seqs, int32_t* block_tables_out,
                               int64_t out_stride, int64_t out_width, int32_t* seq_start_loc,
@@ -240,6 +247,7 @@ int aps_build_decode_metadata(const int32_t* seq_lens, const int32_t* use_hidden
   a.hidden_cache_use_input = hidden_cache_use_input; a.hidden_cache_store_tot = hidden_cache_store_tot;
   a.hidden_holder_upd = hidden_holder_upd; a.hidden_holder_pull = hidden_holder_pull; a.holder_src = holder_src; a.kv_dest = kv_dest;
   a.hidden_slots = hidden_slots; a.hidden_seq_start = hidden_seq_start;
+  a.kv_cache_use_input = kv_cache_use_input; a.new_token_slot = new_token_slot; a.kv_seq_lens = kv_seq_lens;
   a.block_tables_out = block_tables_out; a.out_stride = out_stride; a.out_width = (int)out_width;
   a.seq_start_loc = seq_start_loc; a.query_start_loc = query_start_loc; a.context_lens_out = context_lens;
   a.input_positions = input_positions; a.totals = totals;

@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip attention / re-projection figures")
-    ap.add_argument("--extras", default="attention,metadata,write,reproject,step_loop",
+    ap.add_argument("--extras", default="attention,metadata,write,reproject,layer,step_loop",
                     help="comma-separated subset of the extra figures to run")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="first run the plain copy kernel on 1 GiB three times (known traffic for counter scaling)")
@@ -235,8 +235,16 @@ def main():
         if "reproject" in want:
             extras.update(reproject_figures(torch, ops, dev, args.seed))
         torch.cuda.empty_cache()
+        if "layer" in want:
+            extras["decode_layer_config2"] = decode_layer_figures(torch, ops, workloads, metadata, dev, args.seed)
+            torch.cuda.empty_cache()
         if "step_loop" in want:
-            extras["opt13b_step_loop"] = step_loop_figures(torch, dev, args.seed)
+            from aptserve_hip import opt_model
+            w13 = opt_model.random_weights(opt_model.OPTConfig.opt_13b(), args.seed, dev)
+            extras["opt13b_step_loop"] = step_loop_figures(torch, dev, args.seed, weights=w13)
+            torch.cuda.empty_cache()
+            extras["opt13b_step_loop_absorbed"] = step_loop_figures(torch, dev, args.seed, absorbed=True, weights=w13)
+            del w13
         result["extras"] = extras
 
     if not args.no_cpu:
@@ -265,14 +273,14 @@ def write_figures(torch, ops, dev, seed):
                          "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
 
 
-def step_loop_figures(torch, dev, seed, max_steps=48):
+def step_loop_figures(torch, dev, seed, max_steps=48, absorbed=False, weights=None):
     """BASELINE configs[4]: OPT-13B (random-init fp16, 40 layers) serving steps on the hybrid cache with
     synthetic arrivals (3 req/s, CV 1) and lognormal prompt/output lengths; half of the requests hidden-cached."""
     from aptserve_hip import backend, opt_model, step_loop
     cfg = opt_model.OPTConfig.opt_13b()
     N, BS = 6144, 16
-    w = opt_model.random_weights(cfg, seed, dev)
-    model = opt_model.HybridOPTModel(cfg, w)
+    w = weights if weights is not None else opt_model.random_weights(cfg, seed, dev)
+    model = opt_model.HybridOPTModel(cfg, w, absorbed=absorbed)
     kv, shared = backend.allocate_caches(cfg.num_hidden_layers, N, BS, cfg.num_attention_heads,
                                          cfg.hidden_size // cfg.num_attention_heads, torch.float16, dev)
     reqs = step_loop.synth_requests(seed, 64, rate=3.0, cv=1.0, hidden_fraction=0.5)
@@ -283,7 +291,9 @@ def step_loop_figures(torch, dev, seed, max_steps=48):
     pre = [e for e in log if e["kind"] == "prefill"]
     mean = lambda xs: sum(xs) / len(xs) if xs else None
     return {"workload": "OPT-13B 40 layers fp16 random-init, eager; gamma arrivals 3 req/s cv 1; prompts "
-                        "lognormal(5.5,1.0) in [4,2048]; outputs lognormal(5.0,0.9) in [4,1024]; 50% hidden-cached",
+                        "lognormal(5.5,1.0) in [4,2048]; outputs lognormal(5.0,0.9) in [4,1024]; 50% hidden-cached; "
+                        + ("hidden-cached sequences attend on their hidden rows (absorbed projections)" if absorbed
+                           else "hidden-cached sequences are re-projected every layer (the reference's data flow)"),
             "steps": len(log), "decode_steps": len(dec), "prefill_steps": len(pre),
             "decode_ms_per_step": mean([e["model_ms"] for e in dec]),
             "decode_seqs_per_step": mean([e["seqs"] for e in dec]),
@@ -293,6 +303,38 @@ def step_loop_figures(torch, dev, seed, max_steps=48):
             "metadata_ms_per_step": mean([e["metadata_ms"] for e in log]),
             "decode_tokens_per_s": (sum(e["seqs"] for e in dec) / (sum(e["model_ms"] + e["metadata_ms"] for e in dec) * 1e-3)
                                     if dec else None)}
+
+
+def decode_layer_figures(torch, ops, workloads, metadata, dev, seed):
+    """One decoder self-attention layer of the configs[1] decode batch (256 sequences, half of them
+    hidden-cached, ~87.6 k cached hidden rows) in the two data flows: re-projection of every cached row
+    (gather, K/V GEMM into the workspace, attention) and attention on the hidden rows themselves."""
+    from aptserve_hip import backend
+    H, D, BS = 40, 128, 16
+    Hd = H * D
+    batch = workloads.decode_batch_opt13b(seed)
+    N = batch.num_blocks
+    md = metadata.build_from_batch(batch, dev)
+    g = torch.Generator(device=dev).manual_seed(seed)
+    kv = torch.empty(2, N, BS, H, D, dtype=torch.float16, device=dev)
+    for i in range(0, N, 4096):
+        kv[:, i:i + 4096] = torch.randn(2, min(4096, N - i), BS, H, D, generator=g, device=dev).half()
+    shared = torch.zeros(2, 2 * N, BS, H, D, dtype=torch.float16, device=dev)
+    qkv_w = (torch.randn(3 * Hd, Hd, generator=g, device=dev) * 0.02).half()
+    qkv_b = (torch.randn(3 * Hd, generator=g, device=dev) * 0.02).half()
+    out_w = (torch.randn(Hd, Hd, generator=g, device=dev) * 0.02).half()
+    out_b = (torch.randn(Hd, generator=g, device=dev) * 0.02).half()
+    hs = torch.randn(len(batch.seq_lens), Hd, generator=g, device=dev).half()
+    res = {"workload": "decoder self-attention layer, OPT-13B 40x128, decode batch 256 (128 K/V + 128 hidden), "
+                       "%d cached hidden rows" % int(md.hidden_slots.numel())}
+    outs = {}
+    for name, kw in (("reprojection_ms", dict()), ("absorbed_ms", dict(absorbed=True))):
+        layer = backend.HybridOPTAttention(Hd, H, qkv_w, qkv_b, out_w, out_b, **kw)
+        outs[name] = layer(hs, kv, shared, md)
+        res[name] = median(event_times(torch, lambda: layer(hs, kv, shared, md), 10))
+    res["max_abs_difference"] = (outs["reprojection_ms"].float() - outs["absorbed_ms"].float()).abs().max().item()
+    res["speedup"] = res["reprojection_ms"] / res["absorbed_ms"]
+    return res
 
 
 def reproject_figures(torch, ops, dev, seed):

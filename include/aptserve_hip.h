@@ -275,6 +275,10 @@ int aps_varlen_prefill_attention(void* out, const void* q, const void* k,
  *   hidden_slots[i]          (nullable, not in the reference) private slot of hidden row i, in the order of
  *                            hidden_cache_use_tot; hidden_seq_start[j] (nullable, n hidden sequences + 1
  *                            entries) first hidden row of the j-th hidden sequence: aps_absorbed_attention
+ *   kv_cache_use_input[i]    (nullable, not in the reference) batch position of the i-th K/V-cached sequence;
+ *                            new_token_slot[b] private slot of sequence b's newest token; kv_seq_lens[b]
+ *                            (int32) seq_len of a K/V-cached sequence, 0 for a hidden-cached one — what a
+ *                            step needs to write and attend the K/V-cached sequences only
  *   kv_dest[row]             (nullable, not in the reference) where the row's re-projected K/V go, for
  *                            aps_kv_reproject_to_cache: shared slot (hidden rows), -(private slot + 2)
  *                            (the new token of a K/V sequence), -1 for padding
@@ -290,8 +294,9 @@ int aps_build_decode_metadata(
     int64_t* kv_cache_use_tot, int64_t* hidden_cache_use_input,
     int64_t* hidden_cache_store_tot, int64_t* hidden_holder_upd,
     int64_t* hidden_holder_pull, int64_t* holder_src, int64_t* kv_dest,
-    int64_t* hidden_slots, int64_t* hidden_seq_start, int64_t cap_rows,
-    int64_t cap_hidden_rows,
+    int64_t* hidden_slots, int64_t* hidden_seq_start,
+    int64_t* kv_cache_use_input, int64_t* new_token_slot, int32_t* kv_seq_lens,
+    int64_t cap_rows, int64_t cap_hidden_rows,
     int64_t cap_hidden_seqs, int64_t cap_kv_seqs, int32_t* block_tables_out,
     int64_t out_stride, int64_t out_width, int32_t* seq_start_loc,
     int32_t* query_start_loc, int32_t* context_lens, int64_t* input_positions,

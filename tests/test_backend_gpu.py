@@ -37,7 +37,7 @@ def close(a, b, tol=6e-3):
 
 
 @pytest.mark.parametrize("frac", [0.0, 0.4, 1.0])
-@pytest.mark.parametrize("fused", [True, "gather-only", False])
+@pytest.mark.parametrize("fused", [True, "gather-only", False, "absorbed"])
 def test_decode_layer_matches_oracle(dev, frac, fused):
     W = weights(0)
     batch = workloads.small_decode_batch(3, 10, 150, frac, N)
@@ -49,7 +49,7 @@ def test_decode_layer_matches_oracle(dev, frac, fused):
     ref_kv, ref_sh = kv.clone(), sh.clone()
     ref = OL.opt_attention(hs, ref_kv, ref_sh, ref_md, *W, H)
     layer = backend.HybridOPTAttention(Hd, H, *(w.to(dev) for w in W), fused=bool(fused),
-                                       fuse_kv_write=fused is True)
+                                       fuse_kv_write=fused is True, absorbed=fused == "absorbed")
     md = metadata.build_from_batch(batch, dev)
     d_kv, d_sh = kv.to(dev), sh.to(dev)
     out = layer(hs.to(dev), d_kv, d_sh, md)
@@ -58,6 +58,9 @@ def test_decode_layer_matches_oracle(dev, frac, fused):
     close(d_kv, ref_kv)
     assert torch.equal(d_kv.cpu().view(-1, Hd)[torch.from_numpy(ref_md["slot_mapping"][ref_md["hidden_cache_store_tot"]])],
                        ref_kv.view(-1, Hd)[torch.from_numpy(ref_md["slot_mapping"][ref_md["hidden_cache_store_tot"]])])
+    if fused == "absorbed":          # no re-projection: the shared cache is not touched at all
+        assert torch.equal(d_sh.cpu(), sh)
+        return
     # workspace blocks N..2N-1 hold the re-projected K/V of the hidden sequences
     close(d_sh[:, N:], ref_sh[:, N:])
     # the mirror blocks 0..N-1 are not written by the default data flow

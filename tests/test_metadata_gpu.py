@@ -35,6 +35,15 @@ def assert_same(md, ref):
         private = ref["slot_mapping"][ref["kv_cache_use_tot"]]
         dest[ref["kv_cache_use_tot"]] = np.where(private >= 0, -(private + 2), -1)
         assert np.array_equal(md.kv_dest.cpu().numpy(), dest)
+        hid = np.zeros(md.num_decode_tokens, dtype=bool)
+        hid[ref["hidden_cache_use_input"]] = True
+        assert np.array_equal(md.kv_cache_use_input.cpu().numpy(), np.nonzero(~hid)[0])
+        assert np.array_equal(md.new_token_slot.cpu().numpy(), ref["slot_mapping"][ref["hidden_holder_upd"]])
+        assert np.array_equal(md.kv_seq_lens.cpu().numpy(), np.where(hid, 0, ref["seq_lens_tensor"]).astype(np.int32))
+        assert np.array_equal(md.hidden_slots.cpu().numpy(), ref["slot_mapping"][ref["hidden_cache_use_tot"]])
+        starts = np.concatenate([[0], np.cumsum(ref["seq_lens_tensor"][hid])])
+        if hid.any():
+            assert np.array_equal(md.hidden_seq_start.cpu().numpy(), starts)
 
 
 @pytest.mark.parametrize("seed", range(5))

@@ -16,12 +16,13 @@ META = ["slot_mapping", "slot_mapping_shared", "hidden_cache_use_tot", "kv_cache
         "query_start_loc", "context_lens_tensor", "block_tables", "input_positions"]
 
 
-def test_step_loop_matches_oracle_replay(dev):
+@pytest.mark.parametrize("absorbed", [False, True])
+def test_step_loop_matches_oracle_replay(dev, absorbed):
     cfg = opt_model.OPTConfig(hidden_size=768, num_attention_heads=12, num_hidden_layers=2, ffn_dim=1024,
                               vocab_size=1000, max_position_embeddings=2048)
     N, BS = 96, 16
     w = opt_model.random_weights(cfg, 0, dev)
-    model = opt_model.HybridOPTModel(cfg, w)
+    model = opt_model.HybridOPTModel(cfg, w, absorbed=absorbed)
     kv, shared = backend.allocate_caches(cfg.num_hidden_layers, N, BS, 12, 64, torch.float16, dev)
     reqs = step_loop.synth_requests(3, 7, rate=2000.0, hidden_fraction=0.5, vocab=1000, prompt_mu=3.3,
                                     prompt_sigma=0.6, out_mu=1.6, out_sigma=0.3)
