@@ -334,6 +334,21 @@ def decode_layer_figures(torch, ops, workloads, metadata, dev, seed):
         res[name] = median(event_times(torch, lambda: layer(hs, kv, shared, md), 10))
     res["max_abs_difference"] = (outs["reprojection_ms"].float() - outs["absorbed_ms"].float()).abs().max().item()
     res["speedup"] = res["reprojection_ms"] / res["absorbed_ms"]
+    # the attention on hidden rows alone (query image, scores, softmax, weighted sum, value projection)
+    q = torch.randn(len(batch.seq_lens), Hd, generator=g, device=dev).half()
+    out = torch.empty_like(q)
+    w_k, w_v, b_v = qkv_w[Hd:2 * Hd], qkv_w[2 * Hd:], qkv_b[2 * Hd:]
+    ws = torch.empty(ops._lib.load().aps_absorbed_attention_workspace_bytes(
+        int(md.hidden_cache_use_input.numel()), md.max_hidden_seq_len, H, D), dtype=torch.uint8, device=dev)
+    ms = median(event_times(torch, lambda: ops.absorbed_hidden_attention(
+        q, kv, md.hidden_slots, md.hidden_seq_start, md.hidden_cache_use_input, md.max_hidden_seq_len, w_k, w_v, b_v,
+        D ** -0.5, out, workspace=ws), 10))
+    rows = int(md.hidden_slots.numel())
+    alg = 2 * rows * Hd * 2          # every cached hidden row is read twice (scores, weighted sum)
+    res["absorbed_attention"] = {
+        "ms": ms, "hidden_rows": rows, "algorithmic_bytes": alg,
+        "roofline": {"bound": "hbm", "achieved": alg / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": alg / ms / 1e6 / HBM_PEAK_GBS, "traffic": None}}
     return res
 
 
