@@ -651,6 +651,67 @@ def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, se
     return out
 
 
+# ------------------------------------------------------------------ block maintenance
+
+def copy_blocks(kv_caches, src_to_dsts, kinds=None) -> None:
+    """``FlashAttentionBackend.copy_blocks`` (additional_designs/attention/backends/aptserve_flash_attn.py:58-65)
+    for the caches of all layers in one launch; ``src_to_dsts`` int64 ``[n, 2]`` on the device.
+    ``kinds`` (uint8 ``[n]``, optional): 1 marks a hidden block, whose ids run over the ``2N`` plane
+    slabs of a cache; 0 (default) a K/V block, both planes of block id ``< N``."""
+    if not kv_caches:
+        return
+    c0 = kv_caches[0]
+    dev = c0.device
+    for c in kv_caches:
+        _check_data("kv_cache", c, dev)
+        _need(c.dim() == 5 and c.size(0) == 2 and c.is_contiguous() and c.shape == c0.shape and c.dtype == c0.dtype,
+              "every layer cache must be a contiguous (2, N, BS, H, D) tensor of the same shape and dtype")
+    _need(src_to_dsts.device == dev and src_to_dsts.dtype == torch.int64 and src_to_dsts.dim() == 2
+          and src_to_dsts.size(1) == 2 and src_to_dsts.is_contiguous(), "src_to_dsts must be a contiguous int64 [n, 2] tensor")
+    n = src_to_dsts.size(0)
+    if kinds is not None:
+        _need(kinds.device == dev and kinds.dtype in (torch.uint8, torch.bool) and kinds.is_contiguous()
+              and kinds.numel() == n, "kinds must be a contiguous uint8/bool vector, one entry per pair")
+    if n == 0:
+        return
+    bases = torch.tensor([c.data_ptr() for c in kv_caches], dtype=torch.int64).to(dev)
+    _, N, BS, H, D = c0.shape
+    with torch.cuda.device(dev):
+        st = _lib.load().aps_copy_cache_blocks(bases.data_ptr(), len(kv_caches), src_to_dsts.data_ptr(), _ptr(kinds), n,
+                                               N, BS, H * D, c0.element_size(), _stream(c0))
+    _lib.check(st, "copy_blocks")
+
+
+def swap_blocks(src_kv_cache, dst_kv_cache, src_to_dst, kinds=None) -> None:
+    """``FlashAttentionBackend.swap_blocks`` (aptserve_flash_attn.py:44-56): copies blocks of one layer between
+    two caches (GPU and pinned host memory in the reference's swap-in / swap-out,
+    additional_designs/worker/aptserve_cache_engine.py:88-96).  ``src_to_dst`` is a HOST int64 ``[n, 2]``
+    tensor as in the reference; ``kinds`` a host uint8 ``[n]`` vector (1 = hidden block, ids over the ``2N``
+    plane slabs)."""
+    for c in (src_kv_cache, dst_kv_cache):
+        _need(c.dim() == 5 and c.size(0) == 2 and c.is_contiguous(), "caches must be contiguous (2, N, BS, H, D)")
+    _need(src_kv_cache.shape[2:] == dst_kv_cache.shape[2:] and src_kv_cache.dtype == dst_kv_cache.dtype,
+          "source and destination blocks differ in shape or dtype")
+    _need(src_kv_cache.is_cuda or dst_kv_cache.is_cuda, "one of the caches must live on the GPU")
+    for c in (src_kv_cache, dst_kv_cache):
+        _need(c.is_cuda or c.is_pinned(), "a host cache must be pinned memory")
+    _need(src_to_dst.device.type == "cpu" and src_to_dst.dtype == torch.int64 and src_to_dst.dim() == 2
+          and src_to_dst.size(1) == 2 and src_to_dst.is_contiguous(), "src_to_dst must be a host int64 [n, 2] tensor")
+    n = src_to_dst.size(0)
+    if kinds is not None:
+        _need(kinds.device.type == "cpu" and kinds.dtype in (torch.uint8, torch.bool) and kinds.numel() == n
+              and kinds.is_contiguous(), "kinds must be a host uint8/bool vector, one entry per pair")
+    if n == 0:
+        return
+    gpu = src_kv_cache if src_kv_cache.is_cuda else dst_kv_cache
+    block_bytes = src_kv_cache[0, 0].numel() * src_kv_cache.element_size()
+    with torch.cuda.device(gpu.device):
+        st = _lib.load().aps_swap_cache_blocks(src_kv_cache.data_ptr(), dst_kv_cache.data_ptr(), src_to_dst.data_ptr(),
+                                               None if kinds is None else kinds.data_ptr(), n, src_kv_cache.size(1),
+                                               dst_kv_cache.size(1), block_bytes, _stream(gpu))
+    _lib.check(st, "swap_blocks")
+
+
 # ------------------------------------------------------------------ names of the operator surface
 
 def gather_hidden_blocks(holder, paged_cache, slot_mapping, dst_idx) -> None:

@@ -221,6 +221,42 @@ struct MixedTokenOp {
   }
 };
 
+// Copy of whole cache blocks inside the caches of all layers: item = (layer, pair, plane, token row).
+// A K/V block (kind 0) is both planes of block id b < N; a hidden block (kind 1) is one plane slab, its id
+// runs over the flattened 2N plane slabs (b < N: K plane of block b, b >= N: V plane of block b - N).
+struct BlockCopyOp {
+  const int64_t* layer_base;   // device array: base address of every layer's (2, N, BS, H, D) cache
+  const int64_t* pairs;        // [n][2] (source, destination)
+  const uint8_t* kinds;        // nullable: all K/V blocks
+  int64_t n_pairs, num_blocks, plane_stride_b, block_stride_b, row_b;
+  int rows_per_block;
+  __device__ RowDesc operator()(int64_t item) const {
+    RowDesc r{nullptr, nullptr};
+    const int64_t row = item % rows_per_block;
+    int64_t rest = item / rows_per_block;
+    const int plane = (int)(rest & 1);
+    rest >>= 1;
+    const int64_t pair = rest % n_pairs, layer = rest / n_pairs;
+    const int64_t src = pairs[2 * pair], dst = pairs[2 * pair + 1];
+    const bool hidden = kinds && kinds[pair];
+    char* base = (char*)layer_base[layer];
+    int64_t so, dof;
+    if (hidden) {
+      if (plane) return r;  // a hidden block is a single slab
+      if (src < 0 || dst < 0 || src >= 2 * num_blocks || dst >= 2 * num_blocks) return r;
+      so = (src / num_blocks) * plane_stride_b + (src % num_blocks) * block_stride_b;
+      dof = (dst / num_blocks) * plane_stride_b + (dst % num_blocks) * block_stride_b;
+    } else {
+      if (src < 0 || dst < 0 || src >= num_blocks || dst >= num_blocks) return r;
+      so = plane * plane_stride_b + src * block_stride_b;
+      dof = plane * plane_stride_b + dst * block_stride_b;
+    }
+    r.src = base + so + row * row_b;
+    r.dst = base + dof + row * row_b;
+    return r;
+  }
+};
+
 // item = 2*blk + plane over the reference's grid of 2*nkv + nh blocks
 struct MixedKvOp {
   const char* key; const char* value;
@@ -633,6 +669,52 @@ int aps_mixed_kv_to_cache(const void* key, const void* value, void* k_cache, voi
                                    (uint64_t)(block_stride * e), (uint64_t)(shared_block_stride * e),
                                    (uint64_t)(row * e)});
   return launch_rows(op, 2 * blocks, row * e, vb, (hipStream_t)stream);
+}
+
+int aps_copy_cache_blocks(const int64_t* layer_caches, int64_t num_layers, const int64_t* pairs,
+                          const uint8_t* kinds, int64_t n_pairs, int64_t num_blocks, int block_size,
+                          int64_t row_elems, int elem_size, aps_stream_t stream) {
+  if (num_layers < 0 || n_pairs < 0 || num_blocks <= 0 || block_size <= 0 || row_elems <= 0 || !valid_elem(elem_size))
+    return APS_ERR_INVALID_ARG;
+  if (num_layers == 0 || n_pairs == 0) return APS_OK;
+  if (!layer_caches || !pairs) return APS_ERR_INVALID_ARG;
+  const int64_t row_b = row_elems * elem_size;
+  BlockCopyOp op{layer_caches, pairs, kinds, n_pairs, num_blocks, num_blocks * block_size * row_b,
+                 block_size * row_b, row_b, block_size};
+  const int64_t items = num_layers * n_pairs * 2 * block_size;
+  // layer bases come from the device array: only the row size can be checked here
+  return launch_rows(op, items, row_b, common_vec_bytes({(uint64_t)row_b}), (hipStream_t)stream);
+}
+
+int aps_swap_cache_blocks(const void* src_cache, void* dst_cache, const int64_t* pairs_host,
+                          const uint8_t* kinds_host, int64_t n_pairs, int64_t src_num_blocks,
+                          int64_t dst_num_blocks, int64_t block_bytes, aps_stream_t stream) {
+  if (n_pairs < 0 || src_num_blocks <= 0 || dst_num_blocks <= 0 || block_bytes <= 0) return APS_ERR_INVALID_ARG;
+  if (n_pairs == 0) return APS_OK;
+  if (!src_cache || !dst_cache || !pairs_host) return APS_ERR_INVALID_ARG;
+  const char* s = (const char*)src_cache;
+  char* d = (char*)dst_cache;
+  for (int64_t i = 0; i < n_pairs; ++i) {
+    const int64_t a = pairs_host[2 * i], b = pairs_host[2 * i + 1];
+    const bool hidden = kinds_host && kinds_host[i];
+    if (a < 0 || b < 0) continue;
+    if (hidden) {
+      if (a >= 2 * src_num_blocks || b >= 2 * dst_num_blocks) return APS_ERR_INVALID_ARG;
+      const hipError_t e = hipMemcpyAsync(d + ((b / dst_num_blocks) * dst_num_blocks + b % dst_num_blocks) * block_bytes,
+                                          s + ((a / src_num_blocks) * src_num_blocks + a % src_num_blocks) * block_bytes,
+                                          block_bytes, hipMemcpyDefault, (hipStream_t)stream);
+      if (e != hipSuccess) return (int)e;
+    } else {
+      if (a >= src_num_blocks || b >= dst_num_blocks) return APS_ERR_INVALID_ARG;
+      for (int plane = 0; plane < 2; ++plane) {
+        const hipError_t e = hipMemcpyAsync(d + (plane * dst_num_blocks + b) * block_bytes,
+                                            s + (plane * src_num_blocks + a) * block_bytes, block_bytes,
+                                            hipMemcpyDefault, (hipStream_t)stream);
+        if (e != hipSuccess) return (int)e;
+      }
+    }
+  }
+  return APS_OK;
 }
 
 int aps_copy_bytes(void* dst, const void* src, int64_t nbytes, aps_stream_t stream) {

@@ -403,6 +403,36 @@ int aps_absorbed_attention(
     float softmax_scale, void* out, int64_t out_stride, int64_t out_rows,
     int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * Block maintenance, aware of hidden blocks.
+ * ref: attention/backends/aptserve_flash_attn.py:44-65 (swap_blocks /
+ * copy_blocks over the third-party vllm._custom_ops of the same names, called
+ * from worker/aptserve_cache_engine.py:88-99).  The reference copies the K and
+ * the V plane of block ids < N; a hidden block is ONE plane slab whose id runs
+ * over the 2N slabs (id < N: K plane of block id, id >= N: V plane of block
+ * id - N; core/aptserve_block_manager.py:176-192), which those calls cannot
+ * address.  kinds[i] = 0: K/V block (both planes), 1: hidden block (one slab).
+ * ------------------------------------------------------------------------ */
+
+/* copy_blocks: pairs [n][2] (source, destination) on the device, applied to
+ * every layer; layer_caches is a device array of the layers' cache base
+ * addresses ((2, N, BS, H, D) contiguous, row_elems = H*D). */
+int aps_copy_cache_blocks(const int64_t* layer_caches, int64_t num_layers,
+                          const int64_t* pairs, const uint8_t* kinds,
+                          int64_t n_pairs, int64_t num_blocks, int block_size,
+                          int64_t row_elems, int elem_size,
+                          aps_stream_t stream);
+
+/* swap_blocks: pairs and kinds in HOST memory (as the reference passes them);
+ * one asynchronous copy per plane slab between two caches (device <-> pinned
+ * host, or device <-> device) of src_num_blocks / dst_num_blocks blocks;
+ * block_bytes = BS*H*D*elem_size. */
+int aps_swap_cache_blocks(const void* src_cache, void* dst_cache,
+                          const int64_t* pairs_host, const uint8_t* kinds_host,
+                          int64_t n_pairs, int64_t src_num_blocks,
+                          int64_t dst_num_blocks, int64_t block_bytes,
+                          aps_stream_t stream);
+
 /* Plain device copy of nbytes (16-byte aligned pointers): the known-size
  * kernel that hardware counters of the kernels above are scaled against. */
 int aps_copy_bytes(void* dst, const void* src, int64_t nbytes,

@@ -1,0 +1,71 @@
+"""Block maintenance (copy / swap) aware of hidden blocks, and the scheduler's cost coefficient."""
+import numpy as np
+import pytest
+import torch
+
+from aptserve_hip import cost_model, ops
+from util import sentinel_cache
+
+pytestmark = pytest.mark.gpu
+
+H, D, BS, N = 3, 8, 16, 20
+
+
+def expected_copy(cache, pairs, kinds):
+    ref = cache.clone()
+    flat = ref.view(2 * N, BS, H, D)            # plane slabs: id < N is the K plane of a block, id >= N its V plane
+    src_flat = cache.view(2 * N, BS, H, D)
+    for (a, b), k in zip(pairs, kinds):
+        if k:
+            flat[b] = src_flat[a]
+        else:
+            ref[0, b], ref[1, b] = cache[0, a], cache[1, a]
+    return ref
+
+
+def test_copy_blocks_all_layers_kv_and_hidden(dev):
+    layers = [sentinel_cache((2, N, BS, H, D), seed=i) for i in range(3)]
+    pairs = [(1, 7), (2, 9), (3 + N, 11 + N), (4, 15 + N), (18 + N, 0)]      # distinct destinations
+    kinds = [0, 0, 1, 1, 1]
+    d_layers = [c.to(dev) for c in layers]
+    ops.copy_blocks(d_layers, torch.tensor(pairs, dtype=torch.int64, device=dev),
+                    torch.tensor(kinds, dtype=torch.uint8, device=dev))
+    for c, d in zip(layers, d_layers):
+        assert torch.equal(d.cpu().view(torch.int16), expected_copy(c, pairs, kinds).view(torch.int16))
+    # reference call shape (no kinds): K/V blocks only; out-of-range ids are skipped
+    d2 = [c.to(dev) for c in layers]
+    ops.copy_blocks(d2, torch.tensor([(1, 7), (N + 2, 3), (5, N)], dtype=torch.int64, device=dev))
+    for c, d in zip(layers, d2):
+        assert torch.equal(d.cpu().view(torch.int16), expected_copy(c, [(1, 7)], [0]).view(torch.int16))
+    ops.copy_blocks(d2, torch.empty(0, 2, dtype=torch.int64, device=dev))
+
+
+def test_swap_blocks_out_and_back_in(dev):
+    gpu = sentinel_cache((2, N, BS, H, D)).to(dev)
+    orig = gpu.clone()
+    NC = 12
+    cpu = torch.zeros(2, NC, BS, H, D, dtype=torch.float16).pin_memory()
+    out_pairs = torch.tensor([(3, 0), (5, 1), (7 + N, 2 + NC), (9, 4 + NC)], dtype=torch.int64)
+    kinds = torch.tensor([0, 0, 1, 1], dtype=torch.uint8)
+    ops.swap_blocks(gpu, cpu, out_pairs, kinds)
+    torch.cuda.synchronize()
+    assert torch.equal(cpu[:, 0], orig[:, 3].cpu()) and torch.equal(cpu[:, 1], orig[:, 5].cpu())
+    assert torch.equal(cpu[1, 2], orig[1, 7].cpu()) and torch.equal(cpu[1, 4], orig[0, 9].cpu())
+    assert (cpu[0, 2] == 0).all() and (cpu[0, 4] == 0).all()               # a hidden block is one slab
+    gpu.zero_()
+    back = torch.tensor([(0, 3), (1, 5), (2 + NC, 7 + N), (4 + NC, 9)], dtype=torch.int64)
+    ops.swap_blocks(cpu, gpu, back, kinds)
+    torch.cuda.synchronize()
+    g = gpu.cpu()
+    assert torch.equal(g[:, 3], orig[:, 3].cpu()) and torch.equal(g[:, 5], orig[:, 5].cpu())
+    assert torch.equal(g[1, 7], orig[1, 7].cpu()) and torch.equal(g[0, 9], orig[0, 9].cpu())
+    with pytest.raises(RuntimeError):
+        ops.swap_blocks(cpu, gpu, torch.tensor([(NC, 0)], dtype=torch.int64))   # source block out of range
+
+
+def test_cost_coefficient_is_measured_on_both_flows(dev):
+    counts = (1, 101, 401, 801)
+    c1, st1 = cost_model.get_coef(768, 12, 2, 16, dev, token_counts=counts)
+    c2, st2 = cost_model.get_coef(768, 12, 2, 16, dev, mode="absorbed", token_counts=counts)
+    assert len(st1) == len(st2) == 4 and all(t > 0 for _, t in st1 + st2)
+    assert np.isfinite(c1) and np.isfinite(c2)

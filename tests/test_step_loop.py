@@ -17,3 +17,16 @@ def test_request_stream_and_block_pool():
     assert pool.blocks_needed(r, 65, 16) == (1, 2)
     pool.release(r)
     assert len(pool.free_private) == 8 and len(pool.free_shared) == 8
+
+
+def test_cost_coefficient_regression_follows_the_reference_recipe():
+    """Times linear in the block count with slope s give s/5; the (0, 0) point and the floor at one block
+    are part of the recipe (aptserve_llm_engine.py:336-347)."""
+    from aptserve_hip.cost_model import fit_coef
+    tokens = list(range(1, 4101, 100))
+    blocks = [max(1, t // 16) for t in tokens]
+    slope = 3.5e-4
+    secs = [slope * b for b in blocks]
+    assert abs(fit_coef(tokens, secs, 16) - slope / 5) < 1e-4 * slope
+    # an intercept does not change the slope much (ordinary least squares with intercept)
+    assert abs(fit_coef(tokens, [s + 1e-3 for s in secs], 16) - slope / 5) < 0.05 * slope / 5
