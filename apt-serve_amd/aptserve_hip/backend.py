@@ -272,3 +272,23 @@ class HybridOPTAttention:
         return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
 
     __call__ = forward
+
+
+def promote_hidden_to_kv(qkv_weight, qkv_bias, kv_cache, hidden_slots, kv_slots) -> None:
+    """Turn hidden-cached rows of one layer into K/V-cached rows without a re-prefill: the rows at
+    ``hidden_slots`` (slots of the flattened cache) are re-projected once and written to the K/V slots
+    ``kv_slots`` of the same layer cache.  The reference has no such transition: it changes a sequence's
+    cache type by preempting it in recompute mode
+    (additional_designs/core/aptserve_scheduler.py:748-755).  The opposite direction does not exist
+    (hidden states cannot be recovered from K/V).  Source and destination blocks must not overlap."""
+    n = hidden_slots.numel()
+    if n == 0:
+        return
+    hd = kv_cache.size(3) * kv_cache.size(4)
+    rows = torch.empty(n, hd, dtype=kv_cache.dtype, device=kv_cache.device)
+    idx = torch.arange(n, dtype=torch.int64, device=kv_cache.device)
+    ops.cache_to_hidden(rows, kv_cache, hidden_slots, idx)
+    s = qkv_weight.shape[0] // 3
+    ops.kv_reproject_to_cache(rows, qkv_weight[s:], None if qkv_bias is None else qkv_bias[s:], None, None,
+                              kv_cache[0], kv_cache[1], -(kv_slots + 2))
+

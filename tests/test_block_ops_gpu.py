@@ -69,3 +69,27 @@ def test_cost_coefficient_is_measured_on_both_flows(dev):
     c2, st2 = cost_model.get_coef(768, 12, 2, 16, dev, mode="absorbed", token_counts=counts)
     assert len(st1) == len(st2) == 4 and all(t > 0 for _, t in st1 + st2)
     assert np.isfinite(c1) and np.isfinite(c2)
+
+
+def test_promote_hidden_rows_to_kv(dev):
+    from aptserve_hip import backend
+    from oracle import reproject as OR
+    from util import randn
+    Hh, Dd, Nn = 4, 64, 12
+    Hd = Hh * Dd
+    cache = randn((2, Nn, BS, Hh, Dd), 0)
+    w = (randn((3 * Hd, Hd), 1) * 0.05).half()
+    b = (randn((3 * Hd,), 2) * 0.1).half()
+    hidden_slots = torch.tensor([5, 6, 7, 2 * 16 + 3, Nn * 16 + 9], dtype=torch.int64)     # K- and V-plane slabs
+    kv_slots = torch.tensor([8 * 16 + i for i in range(5)], dtype=torch.int64)
+    rows = cache.view(-1, Hd)[hidden_slots]
+    k_ref, v_ref = OR.kv_reproject(rows, w[Hd:], b[Hd:], keep_fp32=True)
+    d = cache.to(dev)
+    backend.promote_hidden_to_kv(w.to(dev), b.to(dev), d, hidden_slots.to(dev), kv_slots.to(dev))
+    got = d.cpu()
+    assert (got[0].view(-1, Hd)[kv_slots].float() - k_ref.view(5, Hd)).abs().max() < 2e-2
+    assert (got[1].view(-1, Hd)[kv_slots].float() - v_ref.view(5, Hd)).abs().max() < 2e-2
+    untouched = torch.ones(Nn * 16, dtype=torch.bool); untouched[kv_slots] = False
+    assert torch.equal(got[0].view(-1, Hd)[untouched], cache[0].view(-1, Hd)[untouched])
+    assert torch.equal(got[1].view(-1, Hd)[untouched], cache[1].view(-1, Hd)[untouched])
+
