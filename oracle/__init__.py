@@ -26,6 +26,11 @@ kv_reproject / q_only   float64 numpy matmul; identity / one-hot weights
 paged decode attention  float64 textbook softmax on dense K/V; L=1; equal
                         keys -> mean of V; block permutation invariance;
                         all-K/V vs all-hidden equivalence
+absorbed hidden attn.   float64 textbook attention over K = W_k h + b_k, V = W_v h
+                        + b_v of the same rows (any b_k); dropping b_v or
+                        transposing W_k must break the agreement
+mixed_reshape_and_cache composition of hidden_to_cache and
+                        reshape_and_cache_flash (both pinned above)
 layer.opt_attention     composition of the functions above; all-hidden vs
                         all-K/V caches built from the same hidden states agree;
                         decode after prefill equals the last row of a longer
