@@ -214,129 +214,192 @@ __global__ __launch_bounds__(256) void nn_reduce_kernel(const float* __restrict_
 
 // ------------------------------------------------------------------ scores over paged hidden rows
 // S[z][h][t] = sum_k hidden[row_ids[row_start[z] + t]][k] * qt[z][h][k]  (fp32), t < L(z).
-// One workgroup = 256 tokens of one sequence x all heads (padded to 32*NHT); K in tiles of 64 through a
-// two-stage LDS ring.  Rows are copied global -> LDS by global_load_lds_dwordx4 from per-lane row pointers
-// (8 rows x 128 B per wave-wide instruction), chunk c of row r stored at c ^ ((r >> 1) % 8) so that the
-// fragment reads are conflict-free.  8 wavefronts, 32 tokens each, MFMA 32x32x16.
+// One workgroup = kScWaves x 16 tokens of one sequence x all heads x all of K.  What hides the memory latency
+// on this part is bytes in flight per CU (loaded latency ~7 us), so hidden rows go straight from HBM into a
+// 16-step register ring per wavefront (16 KiB in flight each) and never through LDS.  Loads use the
+// coalescing layout (lane l: row l/4, 16-byte piece l%4: four adjacent lanes read 64 contiguous bytes; in
+// MFMA operand order neighbouring lanes would each fetch 16 bytes of a different row, which the memory
+// pipeline serves at a third of the rate) and a ds_bpermute per dword moves a block into operand order
+// (lane 16*g + c: token c, k = 32*step + 8*g) when it is consumed by v_mfma_f32_16x16x32.
+// The query image is the small, reused operand: 512 elements of K at a time, [heads][512], double buffered in
+// LDS (chunk c+1 is fetched into registers at the start of chunk c and written to LDS at its end); the
+// 16-byte chunk ch of head row r sits at position ch ^ (r % 16) of its 16-chunk group (conflict-free fragment
+// reads).  Nothing in the loop is conditional per lane or per step: a guard around a load makes the compiler
+// wait for every outstanding load, which empties the ring.
 struct ScoreArgs {
   const char* cache; int64_t slot_stride_b, num_slots;
-  const int64_t* row_ids; const int64_t* row_start;
+  const int64_t* row_ids; const int64_t* row_start; const int32_t* order;
   const char* qt; int64_t qt_batch_stride_b, qt_row_stride_b; int heads;
   float* s; int64_t s_batch_stride, s_row_stride;  // elements
   int64_t k;
+  const int32_t* tile_start; int n_seqs;  // tile_start[z] = tiles of the sequences before z (n_seqs + 1 entries)
 };
 
-constexpr int kScTokens = 256, kScBK = 64, kScThreads = 512;
+constexpr int kScWaves = 8, kScTokens = kScWaves * 16, kScThreads = kScWaves * 64, kScChunk = 512, kScRing = 16;
+
+// tile_start[z] = sum over y < z of ceil(L(order ? order[y] : y) / tile_tokens); one workgroup.
+__global__ __launch_bounds__(256) void tile_prefix_kernel(const int64_t* __restrict__ row_start,
+                                                          const int32_t* __restrict__ order, int n_seqs,
+                                                          int tile_tokens, int32_t* __restrict__ tile_start) {
+  __shared__ int32_t part[256];
+  __shared__ int32_t carry;
+  if (threadIdx.x == 0) { carry = 0; tile_start[0] = 0; }
+  __syncthreads();
+  for (int base = 0; base < n_seqs; base += 256) {
+    const int y = base + threadIdx.x;
+    int v = 0;
+    if (y < n_seqs) {
+      const int z = order ? order[y] : y;
+      v = (int)((row_start[z + 1] - row_start[z] + tile_tokens - 1) / tile_tokens);
+    }
+    part[threadIdx.x] = v;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {  // inclusive scan
+      const int add = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+      __syncthreads();
+      part[threadIdx.x] += add;
+      __syncthreads();
+    }
+    if (y < n_seqs) tile_start[y + 1] = carry + part[threadIdx.x];
+    __syncthreads();
+    if (threadIdx.x == 0) carry += part[255];
+    __syncthreads();
+  }
+}
+
+template <int NHT>
+constexpr int scores_lds_bytes() { return 2 * NHT * 16 * kScChunk * 2; }
 
 template <bool BF16, int NHT>
 __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreArgs g) {
-  constexpr int kATile = kScTokens * kScBK * 2;  // 32 KiB
-  constexpr int kBGroups = NHT * 4;              // groups of 8 head rows (1 KiB each)
-  constexpr int kBPerWave = (kBGroups + 7) / 8;
-  constexpr int kBTile = kBPerWave * 8 * 1024;   // every wavefront copies kBPerWave groups, real or dummy
-  constexpr int kStage = kATile + kBTile;
-  __shared__ __attribute__((aligned(1024))) char lds[2 * kStage];
+  extern __shared__ __attribute__((aligned(1024))) char lds[];  // [2][NHT*16 heads][1 KiB]
+  constexpr int kBuf = NHT * 16 * kScChunk * 2;
+  constexpr int kPieces = NHT * 16 * 64;                          // 16-byte pieces of a chunk
+  static_assert(kPieces % kScThreads == 0, "pieces are spread evenly over the threads");
+  constexpr int kPerThread = kPieces / kScThreads;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  const int z = blockIdx.y;
+  const int g4 = lane >> 4, c = lane & 15;
+  // Work item blockIdx.x = tile number in the list of all sequences' tiles; workgroups past the end of the list
+  // leave.  (A (tile, sequence) grid would hold mostly absent tiles of short sequences, and since workgroups
+  // are dealt to the 8 XCDs round-robin by linear index, the tiles that exist would crowd onto a few XCDs.)
+  if ((int)blockIdx.x >= g.tile_start[g.n_seqs]) return;
+  int zlo = 0, zhi = g.n_seqs - 1;
+  while (zlo < zhi) {  // last z with tile_start[z] <= blockIdx.x
+    const int mid = (zlo + zhi + 1) >> 1;
+    if (g.tile_start[mid] <= (int)blockIdx.x) zlo = mid; else zhi = mid - 1;
+  }
+  const int z = g.order ? g.order[zlo] : zlo;
   const int64_t rs = g.row_start[z];
   const int L = (int)(g.row_start[z + 1] - rs);
-  const int tile0 = blockIdx.x * kScTokens;
-  if (tile0 >= L) return;
+  const int tile0 = ((int)blockIdx.x - g.tile_start[zlo]) * kScTokens;
+  const int nsteps = (int)(g.k / 32), last_step = nsteps - 1;
+  const int nchunks = (int)((g.k + kScChunk - 1) / kScChunk);
 
-  // DMA sources: 4 groups of 8 token rows per wavefront; lane -> row lane/8, chunk (lane%8) ^ swizzle(row)
-  // Every wavefront issues the same number of copies per tile (the wait counts below rely on it): rows past
-  // the sequence, padding slots and head rows past the last head read slot 0 / head 0 instead; what they
-  // produce is never stored.
-  const char* a_src[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int row = (wave * 4 + j) * 8 + (lane >> 3);
-    const int t = tile0 + row;
+  // row of this lane's token in the loading layout (rows past the sequence / padding slots: slot 0, never stored)
+  const char* rowp;
+  {
+    const int t = tile0 + wave * 16 + (lane >> 2);
     int64_t slot = 0;
     if (t < L) {
       slot = g.row_ids[rs + t];
       if (slot < 0 || slot >= g.num_slots) slot = 0;
     }
-    a_src[j] = g.cache + slot * g.slot_stride_b + (((lane & 7) ^ ((row >> 1) & 7)) * 16);
+    rowp = g.cache + slot * g.slot_stride_b + (lane & 3) * 16;
   }
-  const char* b_src[kBPerWave];
-  int b_group[kBPerWave];
+  const int from_lane = (4 * c + g4) * 4;  // byte address of the lane that loaded (row c, piece g4)
+
+  // query image: piece p = (head p / 64, chunk p % 64); thread tid moves pieces tid + j*threads.  Heads past
+  // the last one and k past the end of K re-read a valid address and are replaced by zeros.
+  const char* qsrc[kPerThread];
+  bool qok[kPerThread];
+  uint32_t qdst[kPerThread];
 #pragma unroll
-  for (int j = 0; j < kBPerWave; ++j) {
-    b_group[j] = wave + 8 * j;
-    const int row = b_group[j] * 8 + (lane >> 3);
-    const int src_row = row < g.heads ? row : 0;
-    b_src[j] = g.qt + (int64_t)z * g.qt_batch_stride_b + (int64_t)src_row * g.qt_row_stride_b +
-               (((lane & 7) ^ ((row >> 1) & 7)) * 16);
+  for (int j = 0; j < kPerThread; ++j) {
+    const int p = tid + j * kScThreads;
+    const int head = p >> 6, ch = p & 63;
+    qok[j] = head < g.heads;
+    qsrc[j] = g.qt + (int64_t)z * g.qt_batch_stride_b + (int64_t)(qok[j] ? head : 0) * g.qt_row_stride_b + ch * 16;
+    qdst[j] = (uint32_t)(head * (kScChunk * 2) + ((ch & ~15) | ((ch ^ head) & 15)) * 16);
   }
-  auto issue = [&](int kt) {
-    char* sa = lds + (kt & 1) * kStage;
-    char* sb = sa + kATile;
-    const int64_t koff = (int64_t)kt * (kScBK * 2);
+  const int64_t k_bytes = g.k * 2;
+  auto fetch_q = [&](int chunk, u32x4(&q)[kPerThread]) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[j] + koff),
-                                       (__attribute__((address_space(3))) void*)(sa + (wave * 4 + j) * 1024), 16, 0, 0);
+    for (int j = 0; j < kPerThread; ++j) {
+      int64_t off = (int64_t)chunk * (kScChunk * 2);
+      if (off + ((tid + j * kScThreads) & 63) * 16 >= k_bytes) off = 0;   // short last chunk: any valid address
+      q[j] = *(const u32x4*)(qsrc[j] + off);
+    }
+  };
+  auto store_q = [&](int buf, int chunk, const u32x4(&q)[kPerThread]) {
+    char* dst = lds + (buf & 1) * kBuf;
 #pragma unroll
-    for (int j = 0; j < kBPerWave; ++j)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[j] + koff),
-                                       (__attribute__((address_space(3))) void*)(sb + b_group[j] * 1024), 16, 0, 0);
+    for (int j = 0; j < kPerThread; ++j) {
+      const bool in_k = (int64_t)chunk * (kScChunk * 2) + ((tid + j * kScThreads) & 63) * 16 < k_bytes;
+      *(u32x4*)(dst + qdst[j]) = (qok[j] && in_k) ? q[j] : u32x4{0u, 0u, 0u, 0u};
+    }
   };
 
-  const int frow = lane & 31, fhalf = lane >> 5;
-  const uint32_t a_row_off = (uint32_t)((wave * 32 + frow) * (kScBK * 2));
-  const uint32_t b_row_off = (uint32_t)(frow * (kScBK * 2));
-  uint32_t chunk_off[4];
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) chunk_off[ks] = (uint32_t)(((2 * ks + fhalf) ^ ((frow >> 1) & 7)) * 16);
-  float16v acc[NHT];
-#pragma unroll
-  for (int nt = 0; nt < NHT; ++nt)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) acc[nt][e] = 0.f;
+  // Workgroups walk K in chunk order rotated by their index.  Slots are a whole number of 256-byte memory
+  // channels apart (10 KiB rows: 40 channels), so workgroups that all started at k = 0 would at every moment
+  // send the whole chip's loads to the few channels that hold that part of a row.
+  const int rot = (int)(blockIdx.x % (unsigned)nchunks);
+  auto chunk_at = [&](int i) { const int ch = i + rot; return ch >= nchunks ? ch - nchunks : ch; };  // i < nchunks
+  auto step_at = [&](int i) {  // the i-th step this workgroup takes (i clamped to the last one)
+    const int ii = min(i, nchunks * (kScChunk / 32) - 1);
+    return min(chunk_at(ii >> 4) * (kScChunk / 32) + (ii & 15), last_step);
+  };
 
-  const int nk = (int)(g.k / kScBK);
-  issue(0);
-  if (nk > 1) issue(1);
-  for (int kt = 0; kt < nk; ++kt) {
-    // tile kt has landed when every load issued so far except tile kt+1's has: wait for all of them on the
-    // last tile, otherwise the loads of tile kt+1 (issued after those of tile kt) may stay in flight
-    if (kt + 1 < nk) {
-      if (kBPerWave == 1) APS_WAIT_VM(5); else APS_WAIT_VM(6);
-    } else {
-      APS_WAIT_VM(0);
-    }
-    APS_BARRIER();
-    const char* sa = lds + (kt & 1) * kStage;
-    const char* sb = sa + kATile;
+  float4v acc[NHT];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const u32x4 af = *(const u32x4*)(sa + a_row_off + chunk_off[ks]);
+  for (int ht = 0; ht < NHT; ++ht) acc[ht] = float4v{0.f, 0.f, 0.f, 0.f};
+  u32x4 qreg[kPerThread];
+  fetch_q(chunk_at(0), qreg);
+  store_q(0, chunk_at(0), qreg);
+  u32x4 ring[kScRing];
 #pragma unroll
-      for (int nt = 0; nt < NHT; ++nt) {
-        const u32x4 bf = *(const u32x4*)(sb + b_row_off + nt * (32 * kScBK * 2) + chunk_off[ks]);
-        acc[nt] = mfma32<BF16>(af, bf, acc[nt]);
+  for (int d = 0; d < kScRing - 1; ++d)
+    ring[d] = __builtin_nontemporal_load((const u32x4*)(rowp + (int64_t)step_at(d) * 64));
+  APS_WAIT_LGKM0();  // own LDS writes done; no fence: it would also wait for the row loads in flight
+  APS_BARRIER();     // chunk 0 of the query image is in LDS
+
+  for (int it = 0; it < nchunks; ++it) {
+    const int next_chunk = chunk_at(min(it + 1, nchunks - 1));
+    fetch_q(next_chunk, qreg);
+    const char* qrow = lds + (it & 1) * kBuf + c * (kScChunk * 2);
+    const int i0 = it * (kScChunk / 32);
+#pragma unroll
+    for (int u = 0; u < kScChunk / 32; ++u) {   // 16 steps = ring size: ring positions are static
+      const int ahead = step_at(i0 + u + kScRing - 1);
+      ring[(u + kScRing - 1) % kScRing] = __builtin_nontemporal_load((const u32x4*)(rowp + (int64_t)ahead * 64));
+      __builtin_amdgcn_sched_barrier(0);  // keep the load here: the scheduler would sink it to its use
+      u32x4 bf;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) bf[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane, (int)ring[u][d]);
+      const int ch = 4 * u + g4;  // chunk of the head row within the 512-element image
+#pragma unroll
+      for (int ht = 0; ht < NHT; ++ht) {
+        const u32x4 af = *(const u32x4*)(qrow + ht * 16 * (kScChunk * 2) + ((ch & ~15) | ((ch ^ c) & 15)) * 16);
+        acc[ht] = mfma16<BF16>(af, bf, acc[ht]);   // steps past the end of K meet the zero padding of the image
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
+    store_q(it + 1, next_chunk, qreg);  // the other buffer: last read one iteration ago, which every wavefront has left
     APS_WAIT_LGKM0();
-    APS_BARRIER();  // every wavefront has its fragments of tile kt: the stage can be refilled
-    if (kt + 2 < nk) issue(kt + 2);
+    APS_BARRIER();
   }
 
-  // lane holds head nt*32 + frow and tokens 8*(e/4) + 4*fhalf + e%4 of its wavefront's 32
+  // lane (g4, c) holds heads 16*ht + 4*g4 + i and token c of its wavefront
+  const int t = tile0 + wave * 16 + c;
+  if (t >= g.s_row_stride) return;
+  float* s_base = g.s + (int64_t)z * g.s_batch_stride + t;
 #pragma unroll
-  for (int nt = 0; nt < NHT; ++nt) {
-    const int head = nt * 32 + frow;
-    if (head >= g.heads) continue;
-    float* row = g.s + (int64_t)z * g.s_batch_stride + (int64_t)head * g.s_row_stride;
+  for (int ht = 0; ht < NHT; ++ht)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int t = tile0 + wave * 32 + 8 * q + 4 * fhalf;
-      if (t < g.s_row_stride)
-        *(float4v*)(row + t) = float4v{acc[nt][4 * q], acc[nt][4 * q + 1], acc[nt][4 * q + 2], acc[nt][4 * q + 3]};
+    for (int i = 0; i < 4; ++i) {
+      const int head = 16 * ht + 4 * g4 + i;
+      if (head < g.heads) s_base[(int64_t)head * g.s_row_stride] = acc[ht][i];
     }
-  }
 }
 
 // ------------------------------------------------------------------ softmax over the tokens of a row
@@ -392,7 +455,7 @@ struct Plan {
   int64_t lp;        // padded row length of S and P
   int kparts;        // token partitions of the weighted sum
   int k_per_part;
-  int64_t off_qt, off_s, off_p, off_ctx, off_partial, total;
+  int64_t off_qt, off_s, off_p, off_ctx, off_tiles, off_partial, total;
 };
 
 Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
@@ -410,6 +473,7 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   p.off_s = o; o += align_up(n_seqs * heads * p.lp * 4, 256);
   p.off_p = o; o += align_up(n_seqs * heads * p.lp * 2, 256);
   p.off_ctx = o; o += align_up(n_seqs * heads * hidden * 2, 256);
+  p.off_tiles = o; o += align_up((n_seqs + 1) * 4, 256);
   p.off_partial = o;
   if (p.kparts > 1) o += align_up((int64_t)p.kparts * n_seqs * heads * hidden * 4, 256);
   p.total = o;
@@ -483,20 +547,41 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
   {
     ScoreArgs g{};
     g.cache = (const char*)paged_cache; g.slot_stride_b = slot_stride * 2; g.num_slots = num_slots;
-    g.row_ids = hidden_slots; g.row_start = seq_start;
+    g.row_ids = hidden_slots; g.row_start = seq_start; g.order = nullptr;
     g.qt = qt; g.qt_batch_stride_b = (int64_t)num_heads * hidden * 2; g.qt_row_stride_b = hidden * 2;
     g.heads = num_heads;
     g.s = sc; g.s_batch_stride = (int64_t)num_heads * p.lp; g.s_row_stride = p.lp;
     g.k = hidden;
-    const dim3 grid((unsigned)((max_len + kScTokens - 1) / kScTokens), (unsigned)n_seqs);
-    const int nht = (num_heads + 31) / 32;
-#define APS_LAUNCH_SCORES(B, N) hipLaunchKernelGGL((hidden_scores_kernel<B, N>), grid, dim3(kScThreads), 0, s, g)
-    if (bf16) {
-      if (nht == 1) APS_LAUNCH_SCORES(true, 1); else if (nht == 2) APS_LAUNCH_SCORES(true, 2); else APS_LAUNCH_SCORES(true, 3);
-    } else {
-      if (nht == 1) APS_LAUNCH_SCORES(false, 1); else if (nht == 2) APS_LAUNCH_SCORES(false, 2); else APS_LAUNCH_SCORES(false, 3);
-    }
+    int32_t* tiles = (int32_t*)(ws + p.off_tiles);
+    hipLaunchKernelGGL(tile_prefix_kernel, dim3(1), dim3(256), 0, s, seq_start, (const int32_t*)nullptr, (int)n_seqs,
+                       kScTokens, tiles);
+    g.tile_start = tiles; g.n_seqs = (int)n_seqs;
+    // upper bound of the tile count that the host can know: every sequence at max_len
+    const int64_t max_tiles = ((max_len + kScTokens - 1) / kScTokens) * n_seqs;
+    if (max_tiles > 0x7fffffff) return APS_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)max_tiles);
+    const int nht = (num_heads + 15) / 16;
+    hipError_t e = hipSuccess;
+#define APS_LAUNCH_SCORES(B, N)                                                                                   \
+  do {                                                                                                            \
+    e = hipFuncSetAttribute((const void*)hidden_scores_kernel<B, N>, hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                            scores_lds_bytes<N>());                                                               \
+    if (e == hipSuccess)                                                                                          \
+      hipLaunchKernelGGL((hidden_scores_kernel<B, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g);      \
+  } while (0)
+#define APS_LAUNCH_SCORES_N(B)                                                                        \
+  switch (nht) {                                                                                      \
+    case 1: APS_LAUNCH_SCORES(B, 1); break;                                                           \
+    case 2: APS_LAUNCH_SCORES(B, 2); break;                                                           \
+    case 3: APS_LAUNCH_SCORES(B, 3); break;                                                           \
+    case 4: APS_LAUNCH_SCORES(B, 4); break;                                                           \
+    case 5: APS_LAUNCH_SCORES(B, 5); break;                                                           \
+    default: APS_LAUNCH_SCORES(B, 6); break;                                                          \
+  }
+    if (bf16) { APS_LAUNCH_SCORES_N(true) } else { APS_LAUNCH_SCORES_N(false) }
+#undef APS_LAUNCH_SCORES_N
 #undef APS_LAUNCH_SCORES
+    if (e != hipSuccess) return (int)e;
     const int st = launch_status();
     if (st != APS_OK) return st;
   }
