@@ -40,6 +40,7 @@ struct NnArgs {
   float* partial;  // non-null: fp32 partial sums [k part][batch][m_rows][n] instead of out
   int batches, k_per_part, m_tiles;
   float alpha;
+  const int32_t* batch_order;  // nullable: the y-th batch dispatched is batch_order[y] (longest first)
 };
 
 constexpr int kNnWaves = 4;   // one wavefront per SIMD: the register file holds a 4-deep ring of row blocks
@@ -52,7 +53,8 @@ __global__ __launch_bounds__(kNnWaves * 64) __attribute__((amdgpu_waves_per_eu(1
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int g4 = lane >> 4, c = lane & 15;
-  const int z = blockIdx.y / g.m_tiles;
+  const int zi = blockIdx.y / g.m_tiles;
+  const int z = g.batch_order ? g.batch_order[zi] : zi;
   const int m0 = (blockIdx.y % g.m_tiles) * (16 * MT);
   int64_t rs = 0;
   int K = g.k_fixed;
@@ -228,7 +230,7 @@ __global__ __launch_bounds__(256) void nn_reduce_kernel(const float* __restrict_
 // wait for every outstanding load, which empties the ring.
 struct ScoreArgs {
   const char* cache; int64_t slot_stride_b, num_slots;
-  const int64_t* row_ids; const int64_t* row_start; const int32_t* order;
+  const int64_t* row_ids; const int64_t* row_start;
   const char* qt; int64_t qt_batch_stride_b, qt_row_stride_b; int heads;
   float* s; int64_t s_batch_stride, s_row_stride;  // elements
   int64_t k;
@@ -237,20 +239,27 @@ struct ScoreArgs {
 
 constexpr int kScWaves = 8, kScTokens = kScWaves * 16, kScThreads = kScWaves * 64, kScChunk = 512, kScRing = 16;
 
-// tile_start[z] = sum over y < z of ceil(L(order ? order[y] : y) / tile_tokens); one workgroup.
-__global__ __launch_bounds__(256) void tile_prefix_kernel(const int64_t* __restrict__ row_start,
-                                                          const int32_t* __restrict__ order, int n_seqs,
-                                                          int tile_tokens, int32_t* __restrict__ tile_start) {
+// One workgroup plans the ragged batch:
+//   tile_start[z] = sum over y < z of ceil(L(y) / tile_tokens)   (n_seqs + 1 entries; the scores kernel's work list)
+//   order[r]      = the sequence with the r-th most rows, ties by index (nullable).  A workgroup of the weighted
+//                   sum works through all rows of its sequence and workgroups start in grid order: longest first
+//                   keeps the last ones short (list scheduling: within a few % of ideal instead of 20-35 % over).
+constexpr int kMaxOrderedSeqs = 4096;  // lengths are ranked out of LDS, quadratic work; larger batches balance anyway
+__global__ __launch_bounds__(256) void seq_plan_kernel(const int64_t* __restrict__ row_start, int n_seqs,
+                                                       int tile_tokens, int32_t* __restrict__ tile_start,
+                                                       int32_t* __restrict__ order) {
   __shared__ int32_t part[256];
   __shared__ int32_t carry;
+  __shared__ int32_t lens[kMaxOrderedSeqs];
   if (threadIdx.x == 0) { carry = 0; tile_start[0] = 0; }
   __syncthreads();
   for (int base = 0; base < n_seqs; base += 256) {
     const int y = base + threadIdx.x;
     int v = 0;
     if (y < n_seqs) {
-      const int z = order ? order[y] : y;
-      v = (int)((row_start[z + 1] - row_start[z] + tile_tokens - 1) / tile_tokens);
+      const int64_t len = row_start[y + 1] - row_start[y];
+      v = (int)((len + tile_tokens - 1) / tile_tokens);
+      if (order) lens[y] = (int32_t)len;
     }
     part[threadIdx.x] = v;
     __syncthreads();
@@ -264,6 +273,13 @@ __global__ __launch_bounds__(256) void tile_prefix_kernel(const int64_t* __restr
     __syncthreads();
     if (threadIdx.x == 0) carry += part[255];
     __syncthreads();
+  }
+  if (!order) return;
+  for (int z = threadIdx.x; z < n_seqs; z += 256) {
+    const int len = lens[z];
+    int rank = 0;
+    for (int y = 0; y < n_seqs; ++y) rank += (lens[y] > len || (lens[y] == len && y < z)) ? 1 : 0;
+    order[rank] = z;
   }
 }
 
@@ -289,7 +305,7 @@ __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreAr
     const int mid = (zlo + zhi + 1) >> 1;
     if (g.tile_start[mid] <= (int)blockIdx.x) zlo = mid; else zhi = mid - 1;
   }
-  const int z = g.order ? g.order[zlo] : zlo;
+  const int z = zlo;
   const int64_t rs = g.row_start[z];
   const int L = (int)(g.row_start[z + 1] - rs);
   const int tile0 = ((int)blockIdx.x - g.tile_start[zlo]) * kScTokens;
@@ -340,22 +356,14 @@ __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreAr
     }
   };
 
-  // Workgroups walk K in chunk order rotated by their index.  Slots are a whole number of 256-byte memory
-  // channels apart (10 KiB rows: 40 channels), so workgroups that all started at k = 0 would at every moment
-  // send the whole chip's loads to the few channels that hold that part of a row.
-  const int rot = (int)(blockIdx.x % (unsigned)nchunks);
-  auto chunk_at = [&](int i) { const int ch = i + rot; return ch >= nchunks ? ch - nchunks : ch; };  // i < nchunks
-  auto step_at = [&](int i) {  // the i-th step this workgroup takes (i clamped to the last one)
-    const int ii = min(i, nchunks * (kScChunk / 32) - 1);
-    return min(chunk_at(ii >> 4) * (kScChunk / 32) + (ii & 15), last_step);
-  };
+  auto step_at = [&](int i) { return min(i, last_step); };  // k step of the i-th loop step, clamped to the last one
 
   float4v acc[NHT];
 #pragma unroll
   for (int ht = 0; ht < NHT; ++ht) acc[ht] = float4v{0.f, 0.f, 0.f, 0.f};
   u32x4 qreg[kPerThread];
-  fetch_q(chunk_at(0), qreg);
-  store_q(0, chunk_at(0), qreg);
+  fetch_q(0, qreg);
+  store_q(0, 0, qreg);
   u32x4 ring[kScRing];
 #pragma unroll
   for (int d = 0; d < kScRing - 1; ++d)
@@ -364,7 +372,7 @@ __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreAr
   APS_BARRIER();     // chunk 0 of the query image is in LDS
 
   for (int it = 0; it < nchunks; ++it) {
-    const int next_chunk = chunk_at(min(it + 1, nchunks - 1));
+    const int next_chunk = min(it + 1, nchunks - 1);
     fetch_q(next_chunk, qreg);
     const char* qrow = lds + (it & 1) * kBuf + c * (kScChunk * 2);
     const int i0 = it * (kScChunk / 32);
@@ -455,7 +463,7 @@ struct Plan {
   int64_t lp;        // padded row length of S and P
   int kparts;        // token partitions of the weighted sum
   int k_per_part;
-  int64_t off_qt, off_s, off_p, off_ctx, off_tiles, off_partial, total;
+  int64_t off_qt, off_s, off_p, off_ctx, off_tiles, off_order, off_partial, total;
 };
 
 Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
@@ -474,6 +482,7 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   p.off_p = o; o += align_up(n_seqs * heads * p.lp * 2, 256);
   p.off_ctx = o; o += align_up(n_seqs * heads * hidden * 2, 256);
   p.off_tiles = o; o += align_up((n_seqs + 1) * 4, 256);
+  p.off_order = o; o += align_up(n_seqs * 4, 256);
   p.off_partial = o;
   if (p.kparts > 1) o += align_up((int64_t)p.kparts * n_seqs * heads * hidden * 4, 256);
   p.total = o;
@@ -547,14 +556,14 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
   {
     ScoreArgs g{};
     g.cache = (const char*)paged_cache; g.slot_stride_b = slot_stride * 2; g.num_slots = num_slots;
-    g.row_ids = hidden_slots; g.row_start = seq_start; g.order = nullptr;
+    g.row_ids = hidden_slots; g.row_start = seq_start;
     g.qt = qt; g.qt_batch_stride_b = (int64_t)num_heads * hidden * 2; g.qt_row_stride_b = hidden * 2;
     g.heads = num_heads;
     g.s = sc; g.s_batch_stride = (int64_t)num_heads * p.lp; g.s_row_stride = p.lp;
     g.k = hidden;
     int32_t* tiles = (int32_t*)(ws + p.off_tiles);
-    hipLaunchKernelGGL(tile_prefix_kernel, dim3(1), dim3(256), 0, s, seq_start, (const int32_t*)nullptr, (int)n_seqs,
-                       kScTokens, tiles);
+    int32_t* order = n_seqs > 1 && n_seqs <= kMaxOrderedSeqs ? (int32_t*)(ws + p.off_order) : nullptr;
+    hipLaunchKernelGGL(seq_plan_kernel, dim3(1), dim3(256), 0, s, seq_start, (int)n_seqs, kScTokens, tiles, order);
     g.tile_start = tiles; g.n_seqs = (int)n_seqs;
     // upper bound of the tile count that the host can know: every sequence at max_len
     const int64_t max_tiles = ((max_len + kScTokens - 1) / kScTokens) * n_seqs;
@@ -608,6 +617,7 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     g.batches = (int)n_seqs; g.k_per_part = p.k_per_part;
     g.m_tiles = (num_heads + 47) / 48;
     g.alpha = 1.f;
+    if (n_seqs > 1 && n_seqs <= kMaxOrderedSeqs) g.batch_order = (const int32_t*)(ws + p.off_order);  // from step 2
     int st = bf16 ? launch_nn<true>(g, p.kparts, s) : launch_nn<false>(g, p.kparts, s);
     if (st != APS_OK) return st;
     if (p.kparts > 1) {
