@@ -286,59 +286,38 @@ __global__ __launch_bounds__(256) void seq_plan_kernel(const int64_t* __restrict
 template <int NHT>
 constexpr int scores_lds_bytes() { return 2 * NHT * 16 * kScChunk * 2; }
 
+// acc[ht][i] (lane (g4, c)) = sum_k row_c[k] * image[16*ht + 4*g4 + i][k]: row_c = the c-th of the 16 rows that
+// this wavefront streams (rowp = this lane's row in the loading layout, + 16 bytes * (lane % 4)), image rows =
+// q_base + r * q_row_stride_b for r < q_rows (zero beyond), staged through lds (scores_lds_bytes<NHT>()).
+// Called by all 8 wavefronts of the workgroup (it contains barriers).
 template <bool BF16, int NHT>
-__global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreArgs g) {
-  extern __shared__ __attribute__((aligned(1024))) char lds[];  // [2][NHT*16 heads][1 KiB]
+__device__ __forceinline__ void stream_rows_times_image(const char* rowp, const char* q_base, int64_t q_row_stride_b,
+                                                        int q_rows, int64_t k, char* lds, float4v (&acc)[NHT]) {
   constexpr int kBuf = NHT * 16 * kScChunk * 2;
   constexpr int kPieces = NHT * 16 * 64;                          // 16-byte pieces of a chunk
   static_assert(kPieces % kScThreads == 0, "pieces are spread evenly over the threads");
   constexpr int kPerThread = kPieces / kScThreads;
   const int tid = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int lane = tid & 63;
   const int g4 = lane >> 4, c = lane & 15;
-  // Work item blockIdx.x = tile number in the list of all sequences' tiles; workgroups past the end of the list
-  // leave.  (A (tile, sequence) grid would hold mostly absent tiles of short sequences, and since workgroups
-  // are dealt to the 8 XCDs round-robin by linear index, the tiles that exist would crowd onto a few XCDs.)
-  if ((int)blockIdx.x >= g.tile_start[g.n_seqs]) return;
-  int zlo = 0, zhi = g.n_seqs - 1;
-  while (zlo < zhi) {  // last z with tile_start[z] <= blockIdx.x
-    const int mid = (zlo + zhi + 1) >> 1;
-    if (g.tile_start[mid] <= (int)blockIdx.x) zlo = mid; else zhi = mid - 1;
-  }
-  const int z = zlo;
-  const int64_t rs = g.row_start[z];
-  const int L = (int)(g.row_start[z + 1] - rs);
-  const int tile0 = ((int)blockIdx.x - g.tile_start[zlo]) * kScTokens;
-  const int nsteps = (int)(g.k / 32), last_step = nsteps - 1;
-  const int nchunks = (int)((g.k + kScChunk - 1) / kScChunk);
-
-  // row of this lane's token in the loading layout (rows past the sequence / padding slots: slot 0, never stored)
-  const char* rowp;
-  {
-    const int t = tile0 + wave * 16 + (lane >> 2);
-    int64_t slot = 0;
-    if (t < L) {
-      slot = g.row_ids[rs + t];
-      if (slot < 0 || slot >= g.num_slots) slot = 0;
-    }
-    rowp = g.cache + slot * g.slot_stride_b + (lane & 3) * 16;
-  }
+  const int nsteps = (int)(k / 32), last_step = nsteps - 1;
+  const int nchunks = (int)((k + kScChunk - 1) / kScChunk);
   const int from_lane = (4 * c + g4) * 4;  // byte address of the lane that loaded (row c, piece g4)
 
-  // query image: piece p = (head p / 64, chunk p % 64); thread tid moves pieces tid + j*threads.  Heads past
-  // the last one and k past the end of K re-read a valid address and are replaced by zeros.
+  // image: piece p = (row p / 64, chunk p % 64); thread tid moves pieces tid + j*threads.  Rows past the last
+  // one and k past the end of K re-read a valid address and are replaced by zeros.
   const char* qsrc[kPerThread];
   bool qok[kPerThread];
   uint32_t qdst[kPerThread];
 #pragma unroll
   for (int j = 0; j < kPerThread; ++j) {
     const int p = tid + j * kScThreads;
-    const int head = p >> 6, ch = p & 63;
-    qok[j] = head < g.heads;
-    qsrc[j] = g.qt + (int64_t)z * g.qt_batch_stride_b + (int64_t)(qok[j] ? head : 0) * g.qt_row_stride_b + ch * 16;
-    qdst[j] = (uint32_t)(head * (kScChunk * 2) + ((ch & ~15) | ((ch ^ head) & 15)) * 16);
+    const int r = p >> 6, ch = p & 63;
+    qok[j] = r < q_rows;
+    qsrc[j] = q_base + (int64_t)(qok[j] ? r : 0) * q_row_stride_b + ch * 16;
+    qdst[j] = (uint32_t)(r * (kScChunk * 2) + ((ch & ~15) | ((ch ^ r) & 15)) * 16);
   }
-  const int64_t k_bytes = g.k * 2;
+  const int64_t k_bytes = k * 2;
   auto fetch_q = [&](int chunk, u32x4(&q)[kPerThread]) {
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) {
@@ -355,10 +334,8 @@ __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreAr
       *(u32x4*)(dst + qdst[j]) = (qok[j] && in_k) ? q[j] : u32x4{0u, 0u, 0u, 0u};
     }
   };
-
   auto step_at = [&](int i) { return min(i, last_step); };  // k step of the i-th loop step, clamped to the last one
 
-  float4v acc[NHT];
 #pragma unroll
   for (int ht = 0; ht < NHT; ++ht) acc[ht] = float4v{0.f, 0.f, 0.f, 0.f};
   u32x4 qreg[kPerThread];
@@ -369,7 +346,7 @@ __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreAr
   for (int d = 0; d < kScRing - 1; ++d)
     ring[d] = __builtin_nontemporal_load((const u32x4*)(rowp + (int64_t)step_at(d) * 64));
   APS_WAIT_LGKM0();  // own LDS writes done; no fence: it would also wait for the row loads in flight
-  APS_BARRIER();     // chunk 0 of the query image is in LDS
+  APS_BARRIER();     // chunk 0 of the image is in LDS
 
   for (int it = 0; it < nchunks; ++it) {
     const int next_chunk = min(it + 1, nchunks - 1);
@@ -384,7 +361,7 @@ __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreAr
       u32x4 bf;
 #pragma unroll
       for (int d = 0; d < 4; ++d) bf[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane, (int)ring[u][d]);
-      const int ch = 4 * u + g4;  // chunk of the head row within the 512-element image
+      const int ch = 4 * u + g4;  // chunk of the image row within the 512-element chunk
 #pragma unroll
       for (int ht = 0; ht < NHT; ++ht) {
         const u32x4 af = *(const u32x4*)(qrow + ht * 16 * (kScChunk * 2) + ((ch & ~15) | ((ch ^ c) & 15)) * 16);
@@ -396,6 +373,42 @@ __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreAr
     APS_WAIT_LGKM0();
     APS_BARRIER();
   }
+}
+
+template <bool BF16, int NHT>
+__global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreArgs g) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];  // [2][NHT*16 heads][1 KiB]
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int g4 = lane >> 4, c = lane & 15;
+  // Work item blockIdx.x = tile number in the list of all sequences' tiles; workgroups past the end of the list
+  // leave.  (A (tile, sequence) grid would hold mostly absent tiles of short sequences, and since workgroups
+  // are dealt to the 8 XCDs round-robin by linear index, the tiles that exist would crowd onto a few XCDs.)
+  if ((int)blockIdx.x >= g.tile_start[g.n_seqs]) return;
+  int zlo = 0, zhi = g.n_seqs - 1;
+  while (zlo < zhi) {  // last z with tile_start[z] <= blockIdx.x
+    const int mid = (zlo + zhi + 1) >> 1;
+    if (g.tile_start[mid] <= (int)blockIdx.x) zlo = mid; else zhi = mid - 1;
+  }
+  const int z = zlo;
+  const int64_t rs = g.row_start[z];
+  const int L = (int)(g.row_start[z + 1] - rs);
+  const int tile0 = ((int)blockIdx.x - g.tile_start[zlo]) * kScTokens;
+
+  // row of this lane's token in the loading layout (rows past the sequence / padding slots: slot 0, never used)
+  const char* rowp;
+  {
+    const int t = tile0 + wave * 16 + (lane >> 2);
+    int64_t slot = 0;
+    if (t < L) {
+      slot = g.row_ids[rs + t];
+      if (slot < 0 || slot >= g.num_slots) slot = 0;
+    }
+    rowp = g.cache + slot * g.slot_stride_b + (lane & 3) * 16;
+  }
+  float4v acc[NHT];
+  stream_rows_times_image<BF16, NHT>(rowp, g.qt + (int64_t)z * g.qt_batch_stride_b, g.qt_row_stride_b, g.heads, g.k,
+                                     lds, acc);
 
   // lane (g4, c) holds heads 16*ht + 4*g4 + i and token c of its wavefront
   const int t = tile0 + wave * 16 + c;
@@ -407,6 +420,58 @@ __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreAr
     for (int i = 0; i < 4; ++i) {
       const int head = 16 * ht + 4 * g4 + i;
       if (head < g.heads) s_base[(int64_t)head * g.s_row_stride] = acc[ht][i];
+    }
+}
+
+// ------------------------------------------------------------------ per-head projection of many rows
+// out[map(m)][h*head_rows + d] = <W[h*head_rows + d], x[m][h]> + bias, for m < m_rows: the per-head value
+// projection of the context rows of many sequences.  The same streaming core as the scores: the streamed rows
+// are the head's weight rows (128 per workgroup), the image is x[m0 .. m0+16*NHT)[h] (16*NHT sequences), so the
+// weights are read once per 16*NHT sequences and x once per 128 weight rows.
+struct HeadProjArgs {
+  const char* w; int64_t w_stride_b; int head_rows, heads;
+  const char* x; int64_t x_row_stride_b, x_head_stride_b; int m_rows;
+  const char* bias;                                   // nullable, 16-bit
+  char* out; int64_t out_stride; const int64_t* out_row_map; int64_t out_rows;  // elements; map nullable
+  int64_t k;
+  int m_tiles, row_tiles;                             // per head
+};
+
+template <bool BF16, int NHT>
+__global__ __launch_bounds__(kScThreads) void head_proj_kernel(const HeadProjArgs g) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int g4 = lane >> 4, c = lane & 15;
+  // blockIdx.x = (m tile, head, row tile), row tile fastest: neighbours share the image through L2
+  const int row_tile = blockIdx.x % g.row_tiles;
+  const int h = (blockIdx.x / g.row_tiles) % g.heads;
+  const int m0 = (blockIdx.x / g.row_tiles / g.heads) * (16 * NHT);
+  const int tile0 = row_tile * kScTokens;
+  const char* rowp;
+  {
+    const int d = tile0 + wave * 16 + (lane >> 2);
+    const int64_t row = (int64_t)h * g.head_rows + (d < g.head_rows ? d : 0);  // rows past the head: never used
+    rowp = g.w + row * g.w_stride_b + (lane & 3) * 16;
+  }
+  float4v acc[NHT];
+  stream_rows_times_image<BF16, NHT>(rowp, g.x + (int64_t)m0 * g.x_row_stride_b + (int64_t)h * g.x_head_stride_b,
+                                     g.x_row_stride_b, min(16 * NHT, g.m_rows - m0), g.k, lds, acc);
+  // lane (g4, c) holds x rows m0 + 16*ht + 4*g4 + i and weight row tile0 + 16*wave + c of the head
+  const int d = tile0 + wave * 16 + c;
+  if (d >= g.head_rows) return;
+  const int64_t col = (int64_t)h * g.head_rows + d;
+  const float b = g.bias ? load_16bit_as_f32<BF16>(g.bias, col) : 0.f;
+#pragma unroll
+  for (int ht = 0; ht < NHT; ++ht)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + 16 * ht + 4 * g4 + i;
+      if (m >= g.m_rows) continue;
+      const int64_t r = g.out_row_map ? g.out_row_map[m] : m;
+      if (r < 0 || r >= g.out_rows) continue;
+      const float v = acc[ht][i] + b;
+      *(uint16_t*)(g.out + (r * g.out_stride + col) * 2) = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
     }
 }
 
@@ -634,8 +699,43 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     }
   }
   // 5. out[seq_rows[s]][h*D + d] = <W_v[h*D + d], ctx[s][h]> + b_v
-  return aps_internal_headwise_linear(ctx, w_v, b_v, out, n_seqs, hidden, hidden, (int64_t)num_heads * hidden, hidden,
-                                      head_size, w_stride, out_stride, seq_rows, out_rows, dtype, s);
+  if (n_seqs <= 16)  // few sequences: the weight-streaming kernels read W_v once
+    return aps_internal_headwise_linear(ctx, w_v, b_v, out, n_seqs, hidden, hidden, (int64_t)num_heads * hidden,
+                                        hidden, head_size, w_stride, out_stride, seq_rows, out_rows, dtype, s);
+  {
+    HeadProjArgs g{};
+    g.w = (const char*)w_v; g.w_stride_b = w_stride * 2; g.head_rows = head_size; g.heads = num_heads;
+    g.x = ctx; g.x_row_stride_b = (int64_t)num_heads * hidden * 2; g.x_head_stride_b = hidden * 2;
+    g.m_rows = (int)n_seqs;
+    g.bias = (const char*)b_v;
+    g.out = (char*)out; g.out_stride = out_stride; g.out_row_map = seq_rows; g.out_rows = out_rows;
+    g.k = hidden;
+    g.row_tiles = (head_size + kScTokens - 1) / kScTokens;
+    // image of 32 or 48 sequences: whichever needs fewer rounds of workgroups over the 256 CUs; on a tie the
+    // smaller one, which gives more workgroups (measured at 128 sequences x 40 heads: 56 us against 59 us)
+    auto rounds = [&](int nht) {
+      const int64_t wgs = (int64_t)num_heads * g.row_tiles * ((n_seqs + 16 * nht - 1) / (16 * nht));
+      return (wgs + 255) / 256;
+    };
+    const int nht = rounds(3) < rounds(2) ? 3 : 2;
+    g.m_tiles = (int)((n_seqs + 16 * nht - 1) / (16 * nht));
+    const dim3 grid((unsigned)(g.m_tiles * num_heads * g.row_tiles));
+    hipError_t e = hipSuccess;
+#define APS_LAUNCH_PROJ(B, N)                                                                                    \
+  do {                                                                                                           \
+    e = hipFuncSetAttribute((const void*)head_proj_kernel<B, N>, hipFuncAttributeMaxDynamicSharedMemorySize,     \
+                            scores_lds_bytes<N>());                                                              \
+    if (e == hipSuccess)                                                                                         \
+      hipLaunchKernelGGL((head_proj_kernel<B, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g);         \
+  } while (0)
+#define APS_LAUNCH_PROJ_N(B)                                                                          \
+  if (nht == 2) APS_LAUNCH_PROJ(B, 2); else APS_LAUNCH_PROJ(B, 3);
+    if (bf16) { APS_LAUNCH_PROJ_N(true) } else { APS_LAUNCH_PROJ_N(false) }
+#undef APS_LAUNCH_PROJ_N
+#undef APS_LAUNCH_PROJ
+    if (e != hipSuccess) return (int)e;
+    return launch_status();
+  }
 }
 
 }  // extern "C"

@@ -2,7 +2,7 @@
 
 Tolerance: the absorbed form never rounds K and V to 16 bits, so it differs from the
 re-projection flow by rounding only; against the float64 oracle on the same 16-bit inputs the
-bar is the stated 2e-2 absolute for a 16-bit attention output (checked at 1e-2)."""
+bar is the stated 2e-2 absolute for a 16-bit attention output (checked at 1e-2 for fp16)."""
 import numpy as np
 import pytest
 import torch
@@ -47,7 +47,8 @@ def run_case(dev, H, D, batch, frac, max_len, N, dtype=torch.float16, seed=0, ws
         ref = OA.absorbed_hidden_attention(q[pos].view(H, D), x, w_k, w_v, b_v, scale).reshape(-1)
         d = (out[pos].double() - ref).abs().max().item()
         worst = max(worst, d)
-    assert worst <= 1e-2, worst
+    # bf16 keeps 8 significant bits: outputs of magnitude ~1 round in steps of 7.8e-3, so it gets the stated bar
+    assert worst <= (2e-2 if dtype == torch.bfloat16 else 1e-2), worst
     # rows of K/V-cached sequences are not touched
     kv_pos = [i for i, h in enumerate(b.use_hidden) if not h]
     assert (out[kv_pos] == 7).all()
@@ -64,6 +65,17 @@ def test_absorbed_attention_bf16_and_many_sequences(dev):
     run_case(dev, 12, 64, 9, 0.6, 200, N=256, dtype=torch.bfloat16)
     # more than 48 hidden sequences: several row tiles in the query product, MFMA kernel in the value projection
     run_case(dev, 4, 64, 70, 0.9, 30, N=512, seed=3)
+
+
+@pytest.mark.parametrize("H,D,batch,dtype", [(12, 64, 30, torch.float16),     # 17..32 sequences: one 32-row image
+                                             (40, 128, 40, torch.float16),    # 128 weight rows per head
+                                             (8, 128, 100, torch.float16),    # four images, the last one partial
+                                             (8, 128, 100, torch.bfloat16),
+                                             (2, 256, 24, torch.float16),     # two 128-row tiles per head
+                                             (40, 64, 200, torch.float16)])   # enough workgroups for 48-row images
+def test_absorbed_attention_value_projection_of_many_sequences(dev, H, D, batch, dtype):
+    """More than 16 hidden-cached sequences: the per-head value projection runs on the row-streaming MFMA kernel."""
+    run_case(dev, H, D, batch, 1.0, 40, N=1024, dtype=dtype, seed=11)
 
 
 def test_absorbed_attention_equals_reprojection_flow(dev):
