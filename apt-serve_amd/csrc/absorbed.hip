@@ -235,6 +235,7 @@ struct ScoreArgs {
   float* s; int64_t s_batch_stride, s_row_stride;  // elements
   int64_t k;
   const int32_t* tile_start; int n_seqs;  // tile_start[z] = tiles of the sequences before z (n_seqs + 1 entries)
+  int64_t k_per_part, s_part_stride;      // blockIdx.y = part of K (whole image chunks); partial scores per part
 };
 
 constexpr int kScWaves = 8, kScTokens = kScWaves * 16, kScThreads = kScWaves * 64, kScChunk = 512, kScRing = 16;
@@ -406,14 +407,18 @@ __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreAr
     }
     rowp = g.cache + slot * g.slot_stride_b + (lane & 3) * 16;
   }
+  // few tiles (small batches): K is split over blockIdx.y so that the chip still has workgroups; the softmax
+  // adds the partial scores
+  const int64_t k0 = (int64_t)blockIdx.y * g.k_per_part;
+  const int64_t klen = min(g.k - k0, g.k_per_part);
   float4v acc[NHT];
-  stream_rows_times_image<BF16, NHT>(rowp, g.qt + (int64_t)z * g.qt_batch_stride_b, g.qt_row_stride_b, g.heads, g.k,
-                                     lds, acc);
+  stream_rows_times_image<BF16, NHT>(rowp + k0 * 2, g.qt + (int64_t)z * g.qt_batch_stride_b + k0 * 2,
+                                     g.qt_row_stride_b, g.heads, klen, lds, acc);
 
   // lane (g4, c) holds heads 16*ht + 4*g4 + i and token c of its wavefront
   const int t = tile0 + wave * 16 + c;
   if (t >= g.s_row_stride) return;
-  float* s_base = g.s + (int64_t)z * g.s_batch_stride + t;
+  float* s_base = g.s + (int64_t)blockIdx.y * g.s_part_stride + (int64_t)z * g.s_batch_stride + t;
 #pragma unroll
   for (int ht = 0; ht < NHT; ++ht)
 #pragma unroll
@@ -480,14 +485,19 @@ __global__ __launch_bounds__(kScThreads) void head_proj_kernel(const HeadProjArg
 template <bool BF16>
 __global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restrict__ s, uint16_t* __restrict__ p,
                                                            const int64_t* __restrict__ row_start, int heads,
-                                                           int64_t lp) {
+                                                           int64_t lp, int parts, int64_t part_stride) {
   __shared__ float red[4];
   const int z = blockIdx.y, h = blockIdx.x;
   const int L = (int)(row_start[z + 1] - row_start[z]);
   const float* row = s + ((int64_t)z * heads + h) * lp;
   uint16_t* out = p + ((int64_t)z * heads + h) * lp;
+  auto score = [&](int64_t t) {  // sum of the partial scores of the K parts
+    float v = row[t];
+    for (int kp = 1; kp < parts; ++kp) v += row[kp * part_stride + t];
+    return v;
+  };
   float mx = -INFINITY;
-  for (int t = threadIdx.x; t < L; t += 256) mx = fmaxf(mx, row[t]);
+  for (int t = threadIdx.x; t < L; t += 256) mx = fmaxf(mx, score(t));
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
@@ -495,7 +505,7 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restri
   mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   __syncthreads();
   float sum = 0.f;
-  for (int t = threadIdx.x; t < L; t += 256) sum += exp2f(row[t] - mx);
+  for (int t = threadIdx.x; t < L; t += 256) sum += exp2f(score(t) - mx);
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = sum;
@@ -503,7 +513,7 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restri
   sum = (red[0] + red[1]) + (red[2] + red[3]);
   const float inv = 1.f / sum;
   for (int64_t t = threadIdx.x; t < lp; t += 256) {
-    const float v = t < L ? exp2f(row[t] - mx) * inv : 0.f;
+    const float v = t < L ? exp2f(score(t) - mx) * inv : 0.f;
     out[t] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
   }
 }
@@ -527,6 +537,8 @@ inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 struct Plan {
   int64_t lp;        // padded row length of S and P
   int kparts;        // token partitions of the weighted sum
+  int score_parts;   // parts of K in the scores kernel (partial scores summed by the softmax)
+  int64_t score_k_per_part;
   int k_per_part;
   int64_t off_qt, off_s, off_p, off_ctx, off_tiles, off_order, off_partial, total;
 };
@@ -541,9 +553,19 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   while (p.lp / parts > kNnMaxPart) parts *= 2;
   p.k_per_part = (int)align_up((p.lp + parts - 1) / parts, 32);
   p.kparts = (int)((p.lp + p.k_per_part - 1) / p.k_per_part);
+  // scores: with few 128-token tiles, split K by whole 512-element chunks until ~2 workgroups per CU exist
+  {
+    const int64_t tiles = n_seqs * ((p.lp + kScTokens - 1) / kScTokens);
+    const int64_t chunks = (hidden + kScChunk - 1) / kScChunk;
+    int64_t parts = 1;
+    while (tiles * parts < 512 && parts < chunks) ++parts;
+    const int64_t per = (chunks + parts - 1) / parts;
+    p.score_parts = (int)((chunks + per - 1) / per);
+    p.score_k_per_part = per * kScChunk;
+  }
   int64_t o = 0;
   p.off_qt = o; o += align_up(n_seqs * heads * hidden * 2, 256);
-  p.off_s = o; o += align_up(n_seqs * heads * p.lp * 4, 256);
+  p.off_s = o; o += align_up(n_seqs * heads * p.lp * 4, 256) * p.score_parts;
   p.off_p = o; o += align_up(n_seqs * heads * p.lp * 2, 256);
   p.off_ctx = o; o += align_up(n_seqs * heads * hidden * 2, 256);
   p.off_tiles = o; o += align_up((n_seqs + 1) * 4, 256);
@@ -598,6 +620,7 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
   char* ws = (char*)workspace;
   char* qt = ws + p.off_qt;
   float* sc = (float*)(ws + p.off_s);
+  const int64_t s_part_stride = align_up(n_seqs * num_heads * p.lp * 4, 256) / 4;  // elements between K parts
   char* pr = ws + p.off_p;
   char* ctx = ws + p.off_ctx;
   float* partial = (float*)(ws + p.off_partial);
@@ -630,10 +653,11 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     int32_t* order = n_seqs > 1 && n_seqs <= kMaxOrderedSeqs ? (int32_t*)(ws + p.off_order) : nullptr;
     hipLaunchKernelGGL(seq_plan_kernel, dim3(1), dim3(256), 0, s, seq_start, (int)n_seqs, kScTokens, tiles, order);
     g.tile_start = tiles; g.n_seqs = (int)n_seqs;
+    g.k_per_part = p.score_k_per_part; g.s_part_stride = s_part_stride;
     // upper bound of the tile count that the host can know: every sequence at max_len
     const int64_t max_tiles = ((max_len + kScTokens - 1) / kScTokens) * n_seqs;
     if (max_tiles > 0x7fffffff) return APS_ERR_UNSUPPORTED;
-    const dim3 grid((unsigned)max_tiles);
+    const dim3 grid((unsigned)max_tiles, (unsigned)p.score_parts);
     const int nht = (num_heads + 15) / 16;
     hipError_t e = hipSuccess;
 #define APS_LAUNCH_SCORES(B, N)                                                                                   \
@@ -663,9 +687,11 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
   {
     const dim3 grid((unsigned)num_heads, (unsigned)n_seqs);
     if (bf16)
-      hipLaunchKernelGGL(softmax_rows_kernel<true>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp);
+      hipLaunchKernelGGL(softmax_rows_kernel<true>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp,
+                         p.score_parts, s_part_stride);
     else
-      hipLaunchKernelGGL(softmax_rows_kernel<false>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp);
+      hipLaunchKernelGGL(softmax_rows_kernel<false>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp,
+                         p.score_parts, s_part_stride);
     const int st = launch_status();
     if (st != APS_OK) return st;
   }
