@@ -288,22 +288,35 @@ template <int NHT>
 constexpr int scores_lds_bytes() { return 2 * NHT * 16 * kScChunk * 2; }
 
 // acc[ht][i] (lane (g4, c)) = sum_k row_c[k] * image[16*ht + 4*g4 + i][k]: row_c = the c-th of the 16 rows that
-// this wavefront streams (rowp = this lane's row in the loading layout, + 16 bytes * (lane % 4)), image rows =
-// q_base + r * q_row_stride_b for r < q_rows (zero beyond), staged through lds (scores_lds_bytes<NHT>()).
-// Called by all 8 wavefronts of the workgroup (it contains barriers).
+// this wavefront streams, image rows = q_base + r * q_row_stride_b for r < q_rows (zero beyond), staged through
+// lds (scores_lds_bytes<NHT>()).  k is a multiple of 64.  Called by all 8 wavefronts of the workgroup (barriers).
+//
+// Loading layout: a wave-wide load takes 128 contiguous bytes (64 k) of each of 8 rows, lane l = row l/8, piece
+// l%8; rowp0 is this lane's pointer into row l/8, rowp1 into row 8 + l/8 (both + 16 bytes * (l % 8)).  On this
+// part scattered rows stream a third faster in 128-byte visits than in 64-byte ones.  Two loads (a pair) hold
+// 16 rows x 64 k = two MFMA k-steps.  Operand order for a step is lane 16*g + c: row c, k piece g of the step's
+// four.  For the even step (pieces 0-3) one DPP move first puts pieces 0-3 of rows 8-15 (second load, lanes
+// with l%8 < 4) over the lanes with l%8 >= 4 of the first load, so that a single ds_bpermute per dword finds
+// every (row, piece) in one register; the odd step mirrors that.
 template <bool BF16, int NHT>
-__device__ __forceinline__ void stream_rows_times_image(const char* rowp, const char* q_base, int64_t q_row_stride_b,
-                                                        int q_rows, int64_t k, char* lds, float4v (&acc)[NHT]) {
+__device__ __forceinline__ void stream_rows_times_image(const char* rowp0, const char* rowp1, const char* q_base,
+                                                        int64_t q_row_stride_b, int q_rows, int64_t k, char* lds,
+                                                        float4v (&acc)[NHT]) {
   constexpr int kBuf = NHT * 16 * kScChunk * 2;
   constexpr int kPieces = NHT * 16 * 64;                          // 16-byte pieces of a chunk
   static_assert(kPieces % kScThreads == 0, "pieces are spread evenly over the threads");
   constexpr int kPerThread = kPieces / kScThreads;
+  constexpr int kPairs = kScRing / 2;                             // pairs of loads in the ring
+  constexpr int kChunkPairs = kScChunk / 64;
+  static_assert(kChunkPairs == kPairs, "ring positions are static because a chunk is one trip round the ring");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int g4 = lane >> 4, c = lane & 15;
-  const int nsteps = (int)(k / 32), last_step = nsteps - 1;
+  const int last_pair = (int)(k / 64) - 1;
   const int nchunks = (int)((k + kScChunk - 1) / kScChunk);
-  const int from_lane = (4 * c + g4) * 4;  // byte address of the lane that loaded (row c, piece g4)
+  const int upper = c >> 3;                                        // rows 8-15 come from the second load
+  const int src_even = (8 * (c & 7) + g4 + 4 * upper) * 4;         // byte address of the source lane, even step
+  const int src_odd = (8 * (c & 7) + g4 + 4 * (1 - upper)) * 4;
 
   // image: piece p = (row p / 64, chunk p % 64); thread tid moves pieces tid + j*threads.  Rows past the last
   // one and k past the end of K re-read a valid address and are replaced by zeros.
@@ -335,7 +348,7 @@ __device__ __forceinline__ void stream_rows_times_image(const char* rowp, const 
       *(u32x4*)(dst + qdst[j]) = (qok[j] && in_k) ? q[j] : u32x4{0u, 0u, 0u, 0u};
     }
   };
-  auto step_at = [&](int i) { return min(i, last_step); };  // k step of the i-th loop step, clamped to the last one
+  auto pair_at = [&](int i) { return (int64_t)min(i, last_pair) * 128; };  // byte offset of the i-th pair, clamped
 
 #pragma unroll
   for (int ht = 0; ht < NHT; ++ht) acc[ht] = float4v{0.f, 0.f, 0.f, 0.f};
@@ -344,8 +357,10 @@ __device__ __forceinline__ void stream_rows_times_image(const char* rowp, const 
   store_q(0, 0, qreg);
   u32x4 ring[kScRing];
 #pragma unroll
-  for (int d = 0; d < kScRing - 1; ++d)
-    ring[d] = __builtin_nontemporal_load((const u32x4*)(rowp + (int64_t)step_at(d) * 64));
+  for (int d = 0; d < kPairs - 1; ++d) {
+    ring[2 * d] = __builtin_nontemporal_load((const u32x4*)(rowp0 + pair_at(d)));
+    ring[2 * d + 1] = __builtin_nontemporal_load((const u32x4*)(rowp1 + pair_at(d)));
+  }
   APS_WAIT_LGKM0();  // own LDS writes done; no fence: it would also wait for the row loads in flight
   APS_BARRIER();     // chunk 0 of the image is in LDS
 
@@ -353,20 +368,31 @@ __device__ __forceinline__ void stream_rows_times_image(const char* rowp, const 
     const int next_chunk = min(it + 1, nchunks - 1);
     fetch_q(next_chunk, qreg);
     const char* qrow = lds + (it & 1) * kBuf + c * (kScChunk * 2);
-    const int i0 = it * (kScChunk / 32);
+    const int i0 = it * kChunkPairs;
 #pragma unroll
-    for (int u = 0; u < kScChunk / 32; ++u) {   // 16 steps = ring size: ring positions are static
-      const int ahead = step_at(i0 + u + kScRing - 1);
-      ring[(u + kScRing - 1) % kScRing] = __builtin_nontemporal_load((const u32x4*)(rowp + (int64_t)ahead * 64));
-      __builtin_amdgcn_sched_barrier(0);  // keep the load here: the scheduler would sink it to its use
-      u32x4 bf;
+    for (int u = 0; u < kChunkPairs; ++u) {
+      const int64_t ahead = pair_at(i0 + u + kPairs - 1);
+      ring[2 * ((u + kPairs - 1) % kPairs)] = __builtin_nontemporal_load((const u32x4*)(rowp0 + ahead));
+      ring[2 * ((u + kPairs - 1) % kPairs) + 1] = __builtin_nontemporal_load((const u32x4*)(rowp1 + ahead));
+      __builtin_amdgcn_sched_barrier(0);  // keep the loads here: the scheduler would sink them to their use
 #pragma unroll
-      for (int d = 0; d < 4; ++d) bf[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane, (int)ring[u][d]);
-      const int ch = 4 * u + g4;  // chunk of the image row within the 512-element chunk
+      for (int j = 0; j < 2; ++j) {
+        u32x4 bf;
 #pragma unroll
-      for (int ht = 0; ht < NHT; ++ht) {
-        const u32x4 af = *(const u32x4*)(qrow + ht * 16 * (kScChunk * 2) + ((ch & ~15) | ((ch ^ c) & 15)) * 16);
-        acc[ht] = mfma16<BF16>(af, bf, acc[ht]);   // steps past the end of K meet the zero padding of the image
+        for (int d = 0; d < 4; ++d) {
+          const int lo = (int)ring[2 * u][d], hi = (int)ring[2 * u + 1][d];
+          // even step: lanes l%8 >= 4 (banks 1, 3 of a 16-lane row) take the second load from 4 lanes below;
+          // odd step: lanes l%8 < 4 (banks 0, 2) take it from 4 lanes above
+          const int merged = j == 0 ? __builtin_amdgcn_update_dpp(lo, hi, 0x114 /* row_shr:4 */, 0xf, 0xa, false)
+                                    : __builtin_amdgcn_update_dpp(lo, hi, 0x104 /* row_shl:4 */, 0xf, 0x5, false);
+          bf[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(j == 0 ? src_even : src_odd, merged);
+        }
+        const int ch = 4 * (2 * u + j) + g4;  // 16-byte piece of the image row within the 512-element chunk
+#pragma unroll
+        for (int ht = 0; ht < NHT; ++ht) {
+          const u32x4 af = *(const u32x4*)(qrow + ht * 16 * (kScChunk * 2) + ((ch & ~15) | ((ch ^ c) & 15)) * 16);
+          acc[ht] = mfma16<BF16>(af, bf, acc[ht]);   // steps past the end of K meet the zero padding of the image
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -396,23 +422,23 @@ __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreAr
   const int L = (int)(g.row_start[z + 1] - rs);
   const int tile0 = ((int)blockIdx.x - g.tile_start[zlo]) * kScTokens;
 
-  // row of this lane's token in the loading layout (rows past the sequence / padding slots: slot 0, never used)
-  const char* rowp;
-  {
-    const int t = tile0 + wave * 16 + (lane >> 2);
+  // rows of this lane's two tokens in the loading layout (past the sequence / padding slots: slot 0, never used)
+  auto token_row = [&](int t) {
     int64_t slot = 0;
     if (t < L) {
       slot = g.row_ids[rs + t];
       if (slot < 0 || slot >= g.num_slots) slot = 0;
     }
-    rowp = g.cache + slot * g.slot_stride_b + (lane & 3) * 16;
-  }
+    return g.cache + slot * g.slot_stride_b + (lane & 7) * 16;
+  };
+  const char* rowp0 = token_row(tile0 + wave * 16 + (lane >> 3));
+  const char* rowp1 = token_row(tile0 + wave * 16 + 8 + (lane >> 3));
   // few tiles (small batches): K is split over blockIdx.y so that the chip still has workgroups; the softmax
   // adds the partial scores
   const int64_t k0 = (int64_t)blockIdx.y * g.k_per_part;
   const int64_t klen = min(g.k - k0, g.k_per_part);
   float4v acc[NHT];
-  stream_rows_times_image<BF16, NHT>(rowp + k0 * 2, g.qt + (int64_t)z * g.qt_batch_stride_b + k0 * 2,
+  stream_rows_times_image<BF16, NHT>(rowp0 + k0 * 2, rowp1 + k0 * 2, g.qt + (int64_t)z * g.qt_batch_stride_b + k0 * 2,
                                      g.qt_row_stride_b, g.heads, klen, lds, acc);
 
   // lane (g4, c) holds heads 16*ht + 4*g4 + i and token c of its wavefront
@@ -453,14 +479,14 @@ __global__ __launch_bounds__(kScThreads) void head_proj_kernel(const HeadProjArg
   const int h = (blockIdx.x / g.row_tiles) % g.heads;
   const int m0 = (blockIdx.x / g.row_tiles / g.heads) * (16 * NHT);
   const int tile0 = row_tile * kScTokens;
-  const char* rowp;
-  {
-    const int d = tile0 + wave * 16 + (lane >> 2);
-    const int64_t row = (int64_t)h * g.head_rows + (d < g.head_rows ? d : 0);  // rows past the head: never used
-    rowp = g.w + row * g.w_stride_b + (lane & 3) * 16;
-  }
+  auto weight_row = [&](int d) {  // rows past the head: its first row, never used
+    const int64_t row = (int64_t)h * g.head_rows + (d < g.head_rows ? d : 0);
+    return g.w + row * g.w_stride_b + (lane & 7) * 16;
+  };
   float4v acc[NHT];
-  stream_rows_times_image<BF16, NHT>(rowp, g.x + (int64_t)m0 * g.x_row_stride_b + (int64_t)h * g.x_head_stride_b,
+  stream_rows_times_image<BF16, NHT>(weight_row(tile0 + wave * 16 + (lane >> 3)),
+                                     weight_row(tile0 + wave * 16 + 8 + (lane >> 3)),
+                                     g.x + (int64_t)m0 * g.x_row_stride_b + (int64_t)h * g.x_head_stride_b,
                                      g.x_row_stride_b, min(16 * NHT, g.m_rows - m0), g.k, lds, acc);
   // lane (g4, c) holds x rows m0 + 16*ht + 4*g4 + i and weight row tile0 + 16*wave + c of the head
   const int d = tile0 + wave * 16 + c;
@@ -483,21 +509,23 @@ __global__ __launch_bounds__(kScThreads) void head_proj_kernel(const HeadProjArg
 // ------------------------------------------------------------------ softmax over the tokens of a row
 // P[z][h][t] = exp2(S - max) / sum for t < L(z), 0 for L <= t < lp; S already carries scale*log2(e).
 template <bool BF16>
-__global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restrict__ s, uint16_t* __restrict__ p,
+__global__ __launch_bounds__(256) void softmax_rows_kernel(float* __restrict__ s, uint16_t* __restrict__ p,
                                                            const int64_t* __restrict__ row_start, int heads,
                                                            int64_t lp, int parts, int64_t part_stride) {
   __shared__ float red[4];
   const int z = blockIdx.y, h = blockIdx.x;
   const int L = (int)(row_start[z + 1] - row_start[z]);
-  const float* row = s + ((int64_t)z * heads + h) * lp;
+  float* row = s + ((int64_t)z * heads + h) * lp;
   uint16_t* out = p + ((int64_t)z * heads + h) * lp;
-  auto score = [&](int64_t t) {  // sum of the partial scores of the K parts
+  // the first pass adds the partial scores of the K parts into part 0; a thread meets the same t in every pass
+  auto score = [&](int64_t t) { return row[t]; };
+  float mx = -INFINITY;
+  for (int t = threadIdx.x; t < L; t += 256) {
     float v = row[t];
     for (int kp = 1; kp < parts; ++kp) v += row[kp * part_stride + t];
-    return v;
-  };
-  float mx = -INFINITY;
-  for (int t = threadIdx.x; t < L; t += 256) mx = fmaxf(mx, score(t));
+    if (parts > 1) row[t] = v;
+    mx = fmaxf(mx, v);
+  }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
