@@ -17,6 +17,7 @@
 // gather, a 4*Hd*Hd-flop GEMM, a cache write and an attention read for the re-projection flow.
 #include "aps_common.h"
 #include "mfma_common.h"
+#include "row_stream_core.h"
 
 namespace aps {
 namespace {
@@ -238,7 +239,6 @@ struct ScoreArgs {
   int64_t k_per_part, s_part_stride;      // blockIdx.y = part of K (whole image chunks); partial scores per part
 };
 
-constexpr int kScWaves = 8, kScTokens = kScWaves * 16, kScThreads = kScWaves * 64, kScChunk = 512, kScRing = 16;
 
 // One workgroup plans the ragged batch:
 //   tile_start[z] = sum over y < z of ceil(L(y) / tile_tokens)   (n_seqs + 1 entries; the scores kernel's work list)
@@ -284,123 +284,6 @@ __global__ __launch_bounds__(256) void seq_plan_kernel(const int64_t* __restrict
   }
 }
 
-template <int NHT>
-constexpr int scores_lds_bytes() { return 2 * NHT * 16 * kScChunk * 2; }
-
-// acc[ht][i] (lane (g4, c)) = sum_k row_c[k] * image[16*ht + 4*g4 + i][k]: row_c = the c-th of the 16 rows that
-// this wavefront streams, image rows = q_base + r * q_row_stride_b for r < q_rows (zero beyond), staged through
-// lds (scores_lds_bytes<NHT>()).  k is a multiple of 64.  Called by all 8 wavefronts of the workgroup (barriers).
-//
-// Loading layout: a wave-wide load takes 128 contiguous bytes (64 k) of each of 8 rows, lane l = row l/8, piece
-// l%8; rowp0 is this lane's pointer into row l/8, rowp1 into row 8 + l/8 (both + 16 bytes * (l % 8)).  On this
-// part scattered rows stream a third faster in 128-byte visits than in 64-byte ones.  Two loads (a pair) hold
-// 16 rows x 64 k = two MFMA k-steps.  Operand order for a step is lane 16*g + c: row c, k piece g of the step's
-// four.  For the even step (pieces 0-3) one DPP move first puts pieces 0-3 of rows 8-15 (second load, lanes
-// with l%8 < 4) over the lanes with l%8 >= 4 of the first load, so that a single ds_bpermute per dword finds
-// every (row, piece) in one register; the odd step mirrors that.
-template <bool BF16, int NHT>
-__device__ __forceinline__ void stream_rows_times_image(const char* rowp0, const char* rowp1, const char* q_base,
-                                                        int64_t q_row_stride_b, int q_rows, int64_t k, char* lds,
-                                                        float4v (&acc)[NHT]) {
-  constexpr int kBuf = NHT * 16 * kScChunk * 2;
-  constexpr int kPieces = NHT * 16 * 64;                          // 16-byte pieces of a chunk
-  static_assert(kPieces % kScThreads == 0, "pieces are spread evenly over the threads");
-  constexpr int kPerThread = kPieces / kScThreads;
-  constexpr int kPairs = kScRing / 2;                             // pairs of loads in the ring
-  constexpr int kChunkPairs = kScChunk / 64;
-  static_assert(kChunkPairs == kPairs, "ring positions are static because a chunk is one trip round the ring");
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int g4 = lane >> 4, c = lane & 15;
-  const int last_pair = (int)(k / 64) - 1;
-  const int nchunks = (int)((k + kScChunk - 1) / kScChunk);
-  const int upper = c >> 3;                                        // rows 8-15 come from the second load
-  const int src_even = (8 * (c & 7) + g4 + 4 * upper) * 4;         // byte address of the source lane, even step
-  const int src_odd = (8 * (c & 7) + g4 + 4 * (1 - upper)) * 4;
-
-  // image: piece p = (row p / 64, chunk p % 64); thread tid moves pieces tid + j*threads.  Rows past the last
-  // one and k past the end of K re-read a valid address and are replaced by zeros.
-  const char* qsrc[kPerThread];
-  bool qok[kPerThread];
-  uint32_t qdst[kPerThread];
-#pragma unroll
-  for (int j = 0; j < kPerThread; ++j) {
-    const int p = tid + j * kScThreads;
-    const int r = p >> 6, ch = p & 63;
-    qok[j] = r < q_rows;
-    qsrc[j] = q_base + (int64_t)(qok[j] ? r : 0) * q_row_stride_b + ch * 16;
-    qdst[j] = (uint32_t)(r * (kScChunk * 2) + ((ch & ~15) | ((ch ^ r) & 15)) * 16);
-  }
-  const int64_t k_bytes = k * 2;
-  auto fetch_q = [&](int chunk, u32x4(&q)[kPerThread]) {
-#pragma unroll
-    for (int j = 0; j < kPerThread; ++j) {
-      int64_t off = (int64_t)chunk * (kScChunk * 2);
-      if (off + ((tid + j * kScThreads) & 63) * 16 >= k_bytes) off = 0;   // short last chunk: any valid address
-      q[j] = *(const u32x4*)(qsrc[j] + off);
-    }
-  };
-  auto store_q = [&](int buf, int chunk, const u32x4(&q)[kPerThread]) {
-    char* dst = lds + (buf & 1) * kBuf;
-#pragma unroll
-    for (int j = 0; j < kPerThread; ++j) {
-      const bool in_k = (int64_t)chunk * (kScChunk * 2) + ((tid + j * kScThreads) & 63) * 16 < k_bytes;
-      *(u32x4*)(dst + qdst[j]) = (qok[j] && in_k) ? q[j] : u32x4{0u, 0u, 0u, 0u};
-    }
-  };
-  auto pair_at = [&](int i) { return (int64_t)min(i, last_pair) * 128; };  // byte offset of the i-th pair, clamped
-
-#pragma unroll
-  for (int ht = 0; ht < NHT; ++ht) acc[ht] = float4v{0.f, 0.f, 0.f, 0.f};
-  u32x4 qreg[kPerThread];
-  fetch_q(0, qreg);
-  store_q(0, 0, qreg);
-  u32x4 ring[kScRing];
-#pragma unroll
-  for (int d = 0; d < kPairs - 1; ++d) {
-    ring[2 * d] = __builtin_nontemporal_load((const u32x4*)(rowp0 + pair_at(d)));
-    ring[2 * d + 1] = __builtin_nontemporal_load((const u32x4*)(rowp1 + pair_at(d)));
-  }
-  APS_WAIT_LGKM0();  // own LDS writes done; no fence: it would also wait for the row loads in flight
-  APS_BARRIER();     // chunk 0 of the image is in LDS
-
-  for (int it = 0; it < nchunks; ++it) {
-    const int next_chunk = min(it + 1, nchunks - 1);
-    fetch_q(next_chunk, qreg);
-    const char* qrow = lds + (it & 1) * kBuf + c * (kScChunk * 2);
-    const int i0 = it * kChunkPairs;
-#pragma unroll
-    for (int u = 0; u < kChunkPairs; ++u) {
-      const int64_t ahead = pair_at(i0 + u + kPairs - 1);
-      ring[2 * ((u + kPairs - 1) % kPairs)] = __builtin_nontemporal_load((const u32x4*)(rowp0 + ahead));
-      ring[2 * ((u + kPairs - 1) % kPairs) + 1] = __builtin_nontemporal_load((const u32x4*)(rowp1 + ahead));
-      __builtin_amdgcn_sched_barrier(0);  // keep the loads here: the scheduler would sink them to their use
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        u32x4 bf;
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          const int lo = (int)ring[2 * u][d], hi = (int)ring[2 * u + 1][d];
-          // even step: lanes l%8 >= 4 (banks 1, 3 of a 16-lane row) take the second load from 4 lanes below;
-          // odd step: lanes l%8 < 4 (banks 0, 2) take it from 4 lanes above
-          const int merged = j == 0 ? __builtin_amdgcn_update_dpp(lo, hi, 0x114 /* row_shr:4 */, 0xf, 0xa, false)
-                                    : __builtin_amdgcn_update_dpp(lo, hi, 0x104 /* row_shl:4 */, 0xf, 0x5, false);
-          bf[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(j == 0 ? src_even : src_odd, merged);
-        }
-        const int ch = 4 * (2 * u + j) + g4;  // 16-byte piece of the image row within the 512-element chunk
-#pragma unroll
-        for (int ht = 0; ht < NHT; ++ht) {
-          const u32x4 af = *(const u32x4*)(qrow + ht * 16 * (kScChunk * 2) + ((ch & ~15) | ((ch ^ c) & 15)) * 16);
-          acc[ht] = mfma16<BF16>(af, bf, acc[ht]);   // steps past the end of K meet the zero padding of the image
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    store_q(it + 1, next_chunk, qreg);  // the other buffer: last read one iteration ago, which every wavefront has left
-    APS_WAIT_LGKM0();
-    APS_BARRIER();
-  }
-}
 
 template <bool BF16, int NHT>
 __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreArgs g) {
@@ -581,15 +464,20 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   while (p.lp / parts > kNnMaxPart) parts *= 2;
   p.k_per_part = (int)align_up((p.lp + parts - 1) / parts, 32);
   p.kparts = (int)((p.lp + p.k_per_part - 1) / p.k_per_part);
-  // scores: with few 128-token tiles, split K by whole 512-element chunks until ~2 workgroups per CU exist
+  // scores: with few 128-token tiles, K is split by whole 512-element chunks into as many parts as still give
+  // at most one workgroup per CU (one round of long-lived workgroups streams fastest)
   {
     const int64_t tiles = n_seqs * ((p.lp + kScTokens - 1) / kScTokens);
     const int64_t chunks = (hidden + kScChunk - 1) / kScChunk;
-    int64_t parts = 1;
-    while (tiles * parts < 512 && parts < chunks) ++parts;
-    const int64_t per = (chunks + parts - 1) / parts;
-    p.score_parts = (int)((chunks + per - 1) / per);
-    p.score_k_per_part = per * kScChunk;
+    int64_t best_per = chunks;
+    for (int64_t per = chunks; per >= 1; --per) {
+      const int64_t parts = (chunks + per - 1) / per;
+      if (tiles * parts > 256) break;
+      if ((chunks - (parts - 1) * per) * 2 < per) continue;  // no stub of a last part
+      best_per = per;
+    }
+    p.score_parts = (int)((chunks + best_per - 1) / best_per);
+    p.score_k_per_part = best_per * kScChunk;
   }
   int64_t o = 0;
   p.off_qt = o; o += align_up(n_seqs * heads * hidden * 2, 256);

@@ -35,6 +35,7 @@
 // form an 8 x 4 block of tiles and share their A and W panels in that XCD's L2.
 #include "aps_common.h"
 #include "mfma_common.h"
+#include "row_stream_core.h"
 
 namespace aps {
 namespace {
@@ -52,7 +53,8 @@ constexpr int kLdsBytes =
     kWaves * kEpiWaveBytes > kStages * kStageBytes ? kWaves * kEpiWaveBytes : kStages * kStageBytes;
 constexpr int kNumXcd = 8;
 constexpr int kGroupM = 8;
-constexpr int kSkinnyMaxRows = 16;  // at most this many rows: the weight-streaming kernel
+constexpr int kSkinnyMaxRows = 16;  // at most this many rows: the weight-streaming MFMA kernel without workspace
+constexpr int kRsMaxRows = 2;       // at most this many rows: the dot-product kernel
 
 // Where a result row goes.  Plain: row t of C is row t (or map[t], negative skipped) of base[0], ld elements
 // apart.  Cache mode (n_split > 0): columns below n_split are the K part of the row and columns from n_split
@@ -300,11 +302,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 // its 8 wavefronts split K, each feeding v_mfma_f32_16x16x32 with the 16 weight rows as the A operand
 // (lane l: row l%16, k-chunk l/16 of 8 elements) and the <=16 activation rows as B (rows beyond m read
 // as zero through the buffer bounds); the 8 partial 16x16 results are added in LDS in a fixed order.
-// No workspace and no second launch; every lane keeps up to 2 x kSkU 16-byte weight loads in flight.
-constexpr int kSkWaves = 8, kSkU = 8;
+// No workspace and no second launch.
+// Weights are not loaded in operand order (a wave-wide load of 16 rows x 64 bytes streams at 4.4 TB/s on this
+// part) but as 8 rows x 128 bytes (lane l: row l/8, 16-byte piece l%8; 5.9 TB/s): two such loads hold
+// 16 rows x 64 k = two MFMA steps.  For the even step one DPP move puts pieces 0-3 of rows 8-15 (second
+// load, lanes with l%8 < 4) over the lanes with l%8 >= 4 of the first load, and one ds_bpermute per dword
+// then fetches (row, piece) for every lane from that single register; the odd step mirrors it.
+// The activations are small and stay in L2; they are loaded in operand order.
+constexpr int kSkWaves = 8, kSkU = 4;   // kSkU pairs of steps per register set
 
 template <bool BF16>
-__global__ __launch_bounds__(kSkWaves * 64) void skinny_nt_kernel(const GemmArgs g, int steps_per_wave) {
+__global__ __launch_bounds__(kSkWaves * 64) void skinny_nt_kernel(const GemmArgs g, int pairs_per_wave) {
   __shared__ float4v red[kSkWaves][64];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -314,38 +322,61 @@ __global__ __launch_bounds__(kSkWaves * 64) void skinny_nt_kernel(const GemmArgs
   const int64_t x_head_b = g.head_rows ? (n0 / g.head_rows) * g.x_head_stride_b : 0;
   const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(g.a + m0 * g.lda_b + x_head_b, (g.m - m0) * g.lda_b - x_head_b);
   const int row = lane & 15, kg = lane >> 4;
-  const uint32_t voff_w = (uint32_t)(row * g.ldw_b + kg * 16);
-  const uint32_t voff_x = (uint32_t)(row * g.lda_b + kg * 16);  // rows >= m are out of bounds: zero
-  const int total_steps = (int)(g.k / 32);
-  const int s_begin = wave * steps_per_wave;
-  const int s_end = min(total_steps, s_begin + steps_per_wave);
+  const uint32_t voff_w0 = (uint32_t)((lane >> 3) * g.ldw_b + (lane & 7) * 16);  // rows >= n: out of bounds, zero
+  const uint32_t voff_w1 = voff_w0 + (uint32_t)(8 * g.ldw_b);
+  const uint32_t voff_x = (uint32_t)(row * g.lda_b + kg * 16);                   // rows >= m: zero
+  const int upper = row >> 3;
+  const int src_even = (8 * (row & 7) + kg + 4 * upper) * 4;       // byte address of the source lane, even step
+  const int src_odd = (8 * (row & 7) + kg + 4 * (1 - upper)) * 4;
+  const int total_steps = (int)(g.k / 32);                         // k is a multiple of 32
+  const int total_pairs = (total_steps + 1) / 2;                   // an odd last step: its pair reads zeros past k
+  const int p_begin = wave * pairs_per_wave;
+  const int p_end = min(total_pairs, p_begin + pairs_per_wave);
   float4v acc = {0.f, 0.f, 0.f, 0.f};
-  u32x4 wa[kSkU], xa[kSkU], wb[kSkU], xb[kSkU];
-  auto load_block = [&](int s0, u32x4(&wq)[kSkU], u32x4(&xq)[kSkU]) {
+  struct Set { u32x4 w0[kSkU], w1[kSkU], x0[kSkU], x1[kSkU]; };
+  Set sa, sb;
+  // Loads are unconditional: pairs past the wavefront's range are clamped to its last pair and skipped in the
+  // multiply (a branch around a load makes the compiler wait for everything outstanding).  The row limit of
+  // the buffer descriptors cannot bound k, so the second step of an odd tail is zeroed by hand.
+  auto load_block = [&](int q0, Set& t) {
 #pragma unroll
     for (int u = 0; u < kSkU; ++u) {
-      if (s0 + u < s_end) {
-        const uint32_t koff = (uint32_t)(s0 + u) * 64;
-        wq[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, voff_w, koff, 2));
-        xq[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff_x, koff, 0));
+      const uint32_t koff = (uint32_t)min(q0 + u, p_end - 1) * 128;
+      t.w0[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, voff_w0, koff, 2));
+      t.w1[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, voff_w1, koff, 2));
+      t.x0[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff_x, koff, 0));
+      t.x1[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, voff_x, koff + 64, 0));
+    }
+  };
+  auto mac_block = [&](int q0, const Set& t) {
+#pragma unroll
+    for (int u = 0; u < kSkU; ++u) {
+      if (q0 + u >= p_end) continue;   // uniform
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (j == 1 && 2 * (q0 + u) + 1 >= total_steps) continue;  // odd number of steps: no second half
+        u32x4 wf;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const int lo = (int)t.w0[u][d], hi = (int)t.w1[u][d];
+          const int merged = j == 0 ? __builtin_amdgcn_update_dpp(lo, hi, 0x114 /* row_shr:4 */, 0xf, 0xa, false)
+                                    : __builtin_amdgcn_update_dpp(lo, hi, 0x104 /* row_shl:4 */, 0xf, 0x5, false);
+          wf[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(j == 0 ? src_even : src_odd, merged);
+        }
+        acc = mfma16<BF16>(wf, j == 0 ? t.x0[u] : t.x1[u], acc);
       }
     }
   };
-  auto mac_block = [&](int s0, const u32x4(&wq)[kSkU], const u32x4(&xq)[kSkU]) {
-#pragma unroll
-    for (int u = 0; u < kSkU; ++u)
-      if (s0 + u < s_end) acc = mfma16<BF16>(wq[u], xq[u], acc);
-  };
-  int s = s_begin;
-  if (s < s_end) load_block(s, wa, xa);
-  while (s < s_end) {
-    load_block(s + kSkU, wb, xb);
-    mac_block(s, wa, xa);
-    s += kSkU;
-    if (s >= s_end) break;
-    load_block(s + kSkU, wa, xa);
-    mac_block(s, wb, xb);
-    s += kSkU;
+  int q = p_begin;
+  if (q < p_end) load_block(q, sa);
+  while (q < p_end) {
+    load_block(q + kSkU, sb);
+    mac_block(q, sa);
+    q += kSkU;
+    if (q >= p_end) break;
+    load_block(q + kSkU, sa);
+    mac_block(q, sb);
+    q += kSkU;
   }
   red[wave][lane] = acc;
   __syncthreads();
@@ -536,6 +567,98 @@ int launch_rowstream_m(const GemmArgs& g, hipStream_t s) {
   }
 }
 
+// ---------------------------------------------------------------- 3 .. 48 rows: weight rows through the streaming core
+// Workgroup = 128 weight rows (8 wavefronts x 16) x one part of K x up to 16*NHT activation rows.  The weight
+// rows are the streamed operand (128-byte visits, 16 KiB in flight per wavefront), the activations the LDS image
+// shared by all wavefronts, so neither LDS nor L2 carries more than the weights themselves (the dot-product
+// kernel reads the activations from LDS once per weight row and slows down from 3 rows on).  n/128 row tiles
+// do not fill the chip: K is split over blockIdx.y into parts of whole 512-element chunks, and the fp32
+// partial tiles [part][m][n] are added by splitk_reduce_kernel.
+constexpr int kWsMaxRows = 48;
+constexpr int kNumCus = 256;
+
+template <bool BF16, int NHT>
+__global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArgs g, int64_t k_per_part) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int g4 = lane >> 4, c = lane & 15;
+  const int64_t n0 = (int64_t)blockIdx.x * kScTokens;
+  const int64_t k0 = (int64_t)blockIdx.y * k_per_part;
+  const int64_t klen = min(g.k - k0, k_per_part);
+  const int64_t m0 = (int64_t)blockIdx.z * (16 * NHT);
+  auto weight_row = [&](int64_t n) {  // rows past the matrix: row 0, never stored
+    return g.w + (n < g.n ? n : 0) * g.ldw_b + (lane & 7) * 16 + k0 * 2;
+  };
+  float4v acc[NHT];
+  stream_rows_times_image<BF16, NHT>(weight_row(n0 + wave * 16 + (lane >> 3)),
+                                     weight_row(n0 + wave * 16 + 8 + (lane >> 3)), g.a + m0 * g.lda_b + k0 * 2,
+                                     g.lda_b, (int)min((int64_t)(16 * NHT), g.m - m0), klen, lds, acc);
+  // lane (g4, c) holds activation rows m0 + 16*ht + 4*g4 + i and weight row n0 + 16*wave + c
+  const int64_t n = n0 + wave * 16 + c;
+  if (n >= g.n) return;
+  float b = 0.f;
+  if (!g.partial && g.bias) b = load_16bit_as_f32<BF16>(g.bias, n);
+  const int half = (g.out.n_split && n >= g.out.n_split) ? 1 : 0;
+#pragma unroll
+  for (int ht = 0; ht < NHT; ++ht)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t row = m0 + 16 * ht + 4 * g4 + i;
+      if (row >= g.m) continue;
+      if (g.partial) {
+        g.partial[((int64_t)blockIdx.y * g.m + row) * g.n + n] = acc[ht][i];
+      } else {
+        uint16_t* dst = out_row(g.out, row, half);
+        if (!dst) continue;
+        const float v = acc[ht][i] + b;
+        dst[n - (half ? g.out.n_split : 0)] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+      }
+    }
+}
+
+// Parts of K for the kernel above: whole chunks, as even as possible, and as many workgroups as still fit one
+// per CU.  Measured (13B layer shapes, 3..48 rows): one round of long-lived workgroups beats more, shorter
+// ones even when they could share a CU (n=5120, k=20480: 240 workgroups 38 us, 400 workgroups 50 us) and even
+// when it leaves CUs idle (n=20480, k=5120: 160 workgroups, no K split, 39 us; 480 workgroups 41-55 us): a
+// workgroup's first loads meet the full memory latency with nothing to overlap, and a CU streams at 34 GB/s
+// while the chip is not saturated.
+int weight_stream_parts(int64_t m, int64_t n, int64_t k, int64_t* k_per_part) {
+  const int nht = m <= 16 ? 1 : (m <= 32 ? 2 : 3);
+  const int64_t tiles = ((n + kScTokens - 1) / kScTokens) * ((m + 16 * nht - 1) / (16 * nht));
+  const int64_t chunks = (k + kScChunk - 1) / kScChunk;
+  int64_t best_per = chunks;  // one part
+  for (int64_t per = chunks; per >= 1; --per) {
+    const int64_t parts = (chunks + per - 1) / per;
+    if (tiles * parts > kNumCus) break;
+    const int64_t last = chunks - (parts - 1) * per;
+    if (last * 2 < per) continue;  // a last part under half a part leaves its workgroups idle early
+    best_per = per;
+  }
+  if (k_per_part) *k_per_part = best_per * kScChunk;
+  return (int)((chunks + best_per - 1) / best_per);
+}
+
+template <bool BF16>
+int launch_weight_stream(const GemmArgs& g, int parts, int64_t k_per_part, hipStream_t s) {
+  const int nht = g.m <= 16 ? 1 : (g.m <= 32 ? 2 : 3);
+  const dim3 grid((unsigned)((g.n + kScTokens - 1) / kScTokens), (unsigned)parts,
+                  (unsigned)((g.m + 16 * nht - 1) / (16 * nht)));
+  hipError_t e = hipSuccess;
+#define APS_LAUNCH_WS(N)                                                                                          \
+  do {                                                                                                            \
+    e = hipFuncSetAttribute((const void*)weight_stream_kernel<BF16, N>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                            scores_lds_bytes<N>());                                                               \
+    if (e == hipSuccess)                                                                                          \
+      hipLaunchKernelGGL((weight_stream_kernel<BF16, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g,    \
+                         k_per_part);                                                                             \
+  } while (0)
+  if (nht == 1) APS_LAUNCH_WS(1); else if (nht == 2) APS_LAUNCH_WS(2); else APS_LAUNCH_WS(3);
+#undef APS_LAUNCH_WS
+  if (e != hipSuccess) return (int)e;
+  return launch_status();
+}
+
 // out[m][n] = sum_z partial[z][m][n] + bias[n], rounded once; 4 columns per thread
 template <bool BF16>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, const void* bias,
@@ -572,7 +695,8 @@ int aps_linear_nt_splits(int64_t m, int64_t n, int64_t k) {
   // Few tiles (a decode step's handful of tokens) cannot pull the weights at HBM speed with one workgroup
   // per tile: split K until about two waves of workgroups exist, keeping at least 4 k-tiles per split.
   if (m <= 0 || n <= 0 || k <= 0 || n % BN != 0 || k % BK != 0) return 1;
-  if (m <= kSkinnyMaxRows) return 1;  // streamed in one launch
+  if (m <= kRsMaxRows) return 1;  // streamed in one launch
+  if (m <= kWsMaxRows) return weight_stream_parts(m, n, k, nullptr);
   if (m > 2 * BM) return 1;  // beyond two row tiles the fp32 partials cost more than the extra workgroups gain
   const int64_t tiles = ((m + BM - 1) / BM) * (n / BN);
   const int64_t nk = k / BK;
@@ -604,11 +728,33 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   g.tiles_m = (int)((m + BM - 1) / BM); g.tiles_n = (int)(n / BN);
   g.out = om;
   hipStream_t s = (hipStream_t)stream;
-  if (m <= 8) return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
+  if (m <= kRsMaxRows) return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
+  if (m <= kWsMaxRows) {
+    int64_t k_per_part = 0;
+    const int parts = weight_stream_parts(m, n, k, &k_per_part);
+    if (parts == 1 || (workspace && workspace_bytes >= (int64_t)parts * m * n * 4 && !(addr(workspace) & 15))) {
+      g.partial = parts > 1 ? (float*)workspace : nullptr;
+      int st = dtype == APS_BF16 ? launch_weight_stream<true>(g, parts, k_per_part, s)
+                                 : launch_weight_stream<false>(g, parts, k_per_part, s);
+      if (st != APS_OK || parts == 1) return st;
+      const int64_t quads = m * n / 4;
+      const dim3 rgrid((unsigned)((quads + 255) / 256));
+      if (dtype == APS_BF16)
+        hipLaunchKernelGGL(splitk_reduce_kernel<true>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m, n,
+                           parts);
+      else
+        hipLaunchKernelGGL(splitk_reduce_kernel<false>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m,
+                           n, parts);
+      return launch_status();
+    }
+    if (workspace) return APS_ERR_WORKSPACE;
+    // no workspace: the single-launch kernels below
+    if (m <= 8) return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
+  }
   if (m <= kSkinnyMaxRows && n / 16 < ((int64_t)1 << 31) && x_stride * 2 * 16 < ((int64_t)1 << 31) &&
       w_stride * 2 * 16 < ((int64_t)1 << 31)) {
-    const int steps = (int)(k / 32);
-    const int per_wave = (steps + kSkWaves - 1) / kSkWaves;
+    const int pairs = (int)((k / 32 + 1) / 2);
+    const int per_wave = (pairs + kSkWaves - 1) / kSkWaves;
     const dim3 grid((unsigned)(n / 16));
     if (dtype == APS_BF16)
       hipLaunchKernelGGL(skinny_nt_kernel<true>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
@@ -672,8 +818,8 @@ int aps_internal_headwise_linear(const void* x, const void* weight, const void* 
   g.x_head_stride_b = x_head_stride * 2; g.head_rows = head_rows;
   if (m <= 8 && n % (kRsWaves * kRsRows) == 0)
     return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
-  const int steps = (int)(k / 32);
-  const int per_wave = (steps + kSkWaves - 1) / kSkWaves;
+  const int pairs = (int)((k / 32 + 1) / 2);
+  const int per_wave = (pairs + kSkWaves - 1) / kSkWaves;
   const dim3 grid((unsigned)(n / 16), (unsigned)((m + 15) / 16));
   if (dtype == APS_BF16)
     hipLaunchKernelGGL(skinny_nt_kernel<true>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);

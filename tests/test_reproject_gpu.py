@@ -42,6 +42,54 @@ def test_linear_nt_small(dev, M, N, K, dtype):
     check(out2, OR._linear_fp32(x, w, None), dtype)
 
 
+@pytest.mark.parametrize("M", [3, 8, 16, 17, 32, 33, 48])
+@pytest.mark.parametrize("N,K", [(256, 64), (512, 1600), (1024, 2048), (2560, 5120)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_linear_nt_few_rows_weight_stream(dev, M, N, K, dtype):
+    """3..48 rows: weight rows through the row-streaming MFMA core (16-, 32- and 48-row images), K in one part
+    or in parts added by the reduce kernel, with a short last chunk (K = 64, 1600) and without (2048, 5120);
+    the same product without a workspace goes through the single-launch kernels and must agree."""
+    x = randn((M, K), M + 1, dtype)
+    w = (randn((N, K), N + 1) * 0.02).to(dtype)    # outputs of magnitude ~1: the absolute bar holds for bf16 too
+    b = (randn((N,), 5) * 0.2).to(dtype)
+    ref = OR._linear_fp32(x, w, b)
+    out = ops.linear_nt(x.to(dev), w.to(dev), b.to(dev))
+    check(out, ref, dtype)
+    if M <= 16:
+        check(ops.linear_nt(x.to(dev), w.to(dev), b.to(dev), split_k=False), ref, dtype)
+    check(ops.linear_nt(x.to(dev), w.to(dev), None), OR._linear_fp32(x, w, None), dtype)
+
+
+def test_few_rows_weight_stream_strides_row_map_and_workspace(dev):
+    K, N, M = 1024, 2560, 21
+    wide = randn((M, 2 * K + 8), 0)
+    x = wide[:, 8:8 + K]                                   # row stride 2K+8, 16-byte aligned start
+    wfull = (randn((N + 256, K), 1) * 0.05).half()
+    w = wfull[256:]                                        # a row slice of a larger weight
+    b = randn((N,), 2).half()
+    ref = OR._linear_fp32(x, w, b)
+    xd, wd, bd = wide.to(dev)[:, 8:8 + K], wfull.to(dev)[256:], b.to(dev)
+    assert ops._lib.load().aps_linear_nt_splits(M, N, K) > 1
+    check(ops.linear_nt(xd, wd, bd), ref)
+    rows = 64
+    perm = torch.from_numpy(np.random.default_rng(1).permutation(rows)[:M].astype(np.int64)); perm[3] = -1
+    dest = torch.full((rows, N), 7.0, dtype=torch.float16, device=dev)
+    ops.linear_nt(xd, wd, bd, out=dest, out_row_map=perm.to(dev))
+    dest = dest.cpu()
+    keep = perm >= 0
+    check(dest[perm[keep]], ref[keep])
+    untouched = torch.ones(rows, dtype=torch.bool); untouched[perm[keep]] = False
+    assert (dest[untouched] == 7).all()
+    # through the C ABI: a workspace that is too small is an error (-3), not a silent fallback
+    small = torch.empty(1024, dtype=torch.uint8, device=dev)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    st = ops._lib.load().aps_linear_nt(xd.data_ptr(), wd.data_ptr(), bd.data_ptr(), out.data_ptr(), M, N, K,
+                                       xd.stride(0), wd.stride(0), out.stride(0), None, M, 0, small.data_ptr(),
+                                       small.numel(), None)
+    torch.cuda.synchronize()
+    assert st == -3
+
+
 def test_identity_and_one_hot_weights_are_exact(dev):
     """W = I reproduces x bit for bit; a one-hot row picks one input column."""
     K = N = 256
@@ -49,6 +97,8 @@ def test_identity_and_one_hot_weights_are_exact(dev):
     w = torch.eye(N, K, dtype=torch.float16)
     out = ops.linear_nt(x.to(dev), w.to(dev)).cpu()
     assert torch.equal(out, x)
+    for m in (2, 5, 16, 40):                               # the few-row kernels as well
+        assert torch.equal(ops.linear_nt(x[:m].to(dev), w.to(dev)).cpu(), x[:m])
     w2 = torch.zeros(N, K, dtype=torch.float16); w2[:, 17] = 1
     out = ops.linear_nt(x.to(dev), w2.to(dev)).cpu()
     assert torch.equal(out, x[:, 17:18].expand(300, N))
