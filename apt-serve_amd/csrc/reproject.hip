@@ -40,18 +40,27 @@
 namespace aps {
 namespace {
 
-constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int BM = 256, BN = 256, BK = 64;      // BM: rows of the full-size tile (MI = 4)
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / 64;
-constexpr int WM = 128, WN = 64;                  // wavefront tile
-constexpr int kTileBytes = BM * BK * 2;          // 32 KiB, same for A and W tiles
-constexpr int kStageBytes = 2 * kTileBytes;      // A + W
+constexpr int WN = 64;                            // columns of a wavefront tile
+constexpr int kWTileBytes = BN * BK * 2;          // 32 KiB
 constexpr int kStages = 2;
 constexpr int kEpiPitch = WN * 2 + 16;            // bytes per row of a wave's epilogue image
-constexpr int kEpiWaveBytes = WM * kEpiPitch;     // 18 KiB
-constexpr int kLdsBytes =
-    kWaves * kEpiWaveBytes > kStages * kStageBytes ? kWaves * kEpiWaveBytes : kStages * kStageBytes;
+// The tile has 2 x 4 wavefronts of (32*MI rows) x 64 columns: 64*MI rows in all.  MI = 4 is the tile for large
+// M; with 49..128 rows it would spend most of its matrix-core time on rows that do not exist (and that time,
+// not the weight stream, bounds the product there), hence MI = 1, 2 and 3.
+template <int MI>
+struct TileShape {
+  static constexpr int kWm = 32 * MI, kBm = 2 * kWm;
+  static constexpr int kATileBytes = kBm * BK * 2;
+  static constexpr int kStageBytes = kATileBytes + kWTileBytes;
+  static constexpr int kEpiWaveBytes = kWm * kEpiPitch;
+  static constexpr int kLdsBytes =
+      kWaves * kEpiWaveBytes > kStages * kStageBytes ? kWaves * kEpiWaveBytes : kStages * kStageBytes;
+};
 constexpr int kNumXcd = 8;
+constexpr int kNumCus = 256;
 constexpr int kGroupM = 8;
 constexpr int kSkinnyMaxRows = 16;  // at most this many rows: the weight-streaming MFMA kernel without workspace
 constexpr int kRsMaxRows = 2;       // at most this many rows: the dot-product kernel
@@ -102,9 +111,12 @@ struct GemmArgs {
   int kt_per_split;
 };
 
-template <bool BF16>
+template <bool BF16, int MI>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_nt_kernel(
     const GemmArgs g) {
+  using T = TileShape<MI>;
+  constexpr int WM = T::kWm, TBM = T::kBm, kStageBytes = T::kStageBytes, kTileBytes = T::kATileBytes;
+  constexpr int kEpiWaveBytes = T::kEpiWaveBytes;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -128,7 +140,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
 
   // ---- global -> LDS DMA addressing
-  const int64_t row0 = (int64_t)pid_m * BM, col0 = (int64_t)pid_n * BN;
+  const int64_t row0 = (int64_t)pid_m * TBM, col0 = (int64_t)pid_n * BN;
   const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(g.a + row0 * g.lda_b, (g.m - row0) * g.lda_b);
   const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(g.w + col0 * g.ldw_b, (g.n - col0) * g.ldw_b);
   const int lrow = lane >> 3;  // row within the 8-row group of a wave-wide load
@@ -145,10 +157,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     char* sw = sa + kTileBytes;
     const uint32_t koff = (uint32_t)(kt_base_ + kt) * (BK * 2);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int i = wave * 4 + j;  // 8-row group of the tile handled by this wave-wide load
+    for (int j = 0; j < MI; ++j) {
+      const int i = wave * MI + j;  // 8-row group of the A tile handled by this wave-wide load (8*MI groups)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(sa + i * 1024), 16,
-                                               (j & 1) ? voff_a1 : voff_a0, koff + i * grp_a, 0, 0);
+                                               (i & 1) ? voff_a1 : voff_a0, koff + i * grp_a, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = wave * 4 + j;   // 8-row group of the W tile (32 groups)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (__attribute__((address_space(3))) void*)(sw + i * 1024), 16,
                                                (j & 1) ? voff_w1 : voff_w0, koff + i * grp_w, 0, 0);
     }
@@ -162,29 +178,30 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) chunk_off[ks] = (uint32_t)(((2 * ks + fhalf) ^ ((frow >> 1) & 7)) * 16);
 
-  float16v acc[4][2];
+  float16v acc[MI][2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  auto read_frags = [&](int kt, int ks, u32x4(&af)[4], u32x4(&wf)[2]) {
+  auto read_frags = [&](int kt, int ks, u32x4(&af)[MI], u32x4(&wf)[2]) {
     const char* sa = lds + (kt & 1) * kStageBytes;
     const char* sw = sa + kTileBytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) af[i] = *(const u32x4*)(sa + a_row_off + i * (32 * BK * 2) + chunk_off[ks]);
+    for (int i = 0; i < MI; ++i) af[i] = *(const u32x4*)(sa + a_row_off + i * (32 * BK * 2) + chunk_off[ks]);
 #pragma unroll
     for (int i = 0; i < 2; ++i) wf[i] = *(const u32x4*)(sw + w_row_off + i * (32 * BK * 2) + chunk_off[ks]);
   };
-  auto mfma8 = [&](const u32x4(&af)[4], const u32x4(&wf)[2]) {
+  auto mfma8 = [&](const u32x4(&af)[MI], const u32x4(&wf)[2]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j) acc[i][j] = mfma32<BF16>(af[i], wf[j], acc[i][j]);
   };
   auto interleave = [&]() {  // scheduling hint: the 6 LDS reads spread over the 8 MFMA of a k-step
+    if constexpr (MI != 4) return;  // the small tiles are bound by the weight stream: the compiler's order will do
     __builtin_amdgcn_sched_group_barrier(0x008, 2, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     __builtin_amdgcn_sched_group_barrier(0x008, 2, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
@@ -196,11 +213,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int nk_total = (int)(g.k / BK);
   const int kt_base = g.partial ? blockIdx.y * g.kt_per_split : 0;
   const int nk = g.partial ? min(g.kt_per_split, nk_total - kt_base) : nk_total;
-  u32x4 a0[4], w0[2], a1[4], w1[2];
+  u32x4 a0[MI], w0[2], a1[MI], w1[2];
   issue_loads(0);
   if (nk > 1) {
     issue_loads(1);
-    APS_WAIT_VM(8);  // tile 0 has landed, tile 1 may still be in flight
+    // tile 0 has landed, tile 1 (4 + MI loads per wavefront) may still be in flight
+    if constexpr (MI == 4) APS_WAIT_VM(8); else if constexpr (MI == 3) APS_WAIT_VM(7);
+    else if constexpr (MI == 2) APS_WAIT_VM(6); else APS_WAIT_VM(5);
   } else {
     APS_WAIT_VM(0);
   }
@@ -230,7 +249,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
   // ---- epilogue: bias, round once, transpose through LDS, 128-bit row stores.
   // Lane l of a 32x32 result tile holds column l%32 and rows 8*(e/4) + 4*(l/32) + e%4, e = 0..15.
-  // Each wave owns a [128 rows][64 cols] fp16 image (row pitch 144 B).  Neighbouring lanes swap one value
+  // Each wave owns a [32*MI rows][64 cols] fp16 image (row pitch 144 B).  Neighbouring lanes swap one value
   // so that every lane writes a 32-bit pair; the image is then read back 16 bytes per lane, 8 lanes per row.
   if (g.partial) {  // split-K: raw fp32 partial sums, lanes of a half-wave write 128 contiguous bytes
     float* pz = g.partial + (int64_t)blockIdx.y * g.m * g.n;
@@ -238,7 +257,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int j = 0; j < 2; ++j) {
       const int64_t col = col0 + wn * WN + j * 32 + frow;
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int64_t row = row0 + wm * WM + i * 32 + 8 * (e >> 2) + 4 * fhalf + (e & 3);
@@ -260,7 +279,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
       bv = BF16 ? __uint_as_float((uint32_t)bb << 16) : (float)__builtin_bit_cast(_Float16, bb);
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < MI; ++i) {
 #pragma unroll
       for (int e = 0; e < 16; e += 2) {
         const float v0 = acc[i][j][e] + bv, v1 = acc[i][j][e + 1] + bv;
@@ -575,7 +594,6 @@ int launch_rowstream_m(const GemmArgs& g, hipStream_t s) {
 // do not fill the chip: K is split over blockIdx.y into parts of whole 512-element chunks, and the fp32
 // partial tiles [part][m][n] are added by splitk_reduce_kernel.
 constexpr int kWsMaxRows = 48;
-constexpr int kNumCus = 256;
 
 template <bool BF16, int NHT>
 __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArgs g, int64_t k_per_part) {
@@ -691,18 +709,36 @@ using namespace aps;
 
 extern "C" {
 
+// Tile rows / 64 for m rows beyond the row-streaming kernels' range.  Up to 128 rows: the smallest tile that
+// covers m.  Beyond: 192 or 256 rows, whichever needs less time by the count "rounds of workgroups over the
+// CUs x rows per tile" (a tie goes to the 256-row tile, which is the one tuned for large products).  Measured
+// on the 13B layer shapes this rule picks the faster of the two at every m from 160 to 4096; the 192-row tile
+// wins most of that range because its rounds are shorter and rows past m cost it less matrix-core time.
+static int tile_mi(int64_t m, int64_t n) {
+  if (m <= 64) return 1;
+  if (m <= 128) return 2;
+  auto cost = [&](int mi) {
+    const int64_t tiles = ((m + 64 * mi - 1) / (64 * mi)) * (n / BN);
+    return ((tiles + kNumCus - 1) / kNumCus) * mi;
+  };
+  return cost(3) < cost(4) ? 3 : 4;
+}
+
 int aps_linear_nt_splits(int64_t m, int64_t n, int64_t k) {
   // Few tiles (a decode step's handful of tokens) cannot pull the weights at HBM speed with one workgroup
   // per tile: split K until about two waves of workgroups exist, keeping at least 4 k-tiles per split.
   if (m <= 0 || n <= 0 || k <= 0 || n % BN != 0 || k % BK != 0) return 1;
   if (m <= kRsMaxRows) return 1;  // streamed in one launch
   if (m <= kWsMaxRows) return weight_stream_parts(m, n, k, nullptr);
-  if (m > 2 * BM) return 1;  // beyond two row tiles the fp32 partials cost more than the extra workgroups gain
-  const int64_t tiles = ((m + BM - 1) / BM) * (n / BN);
+  const int64_t bm = 64 * tile_mi(m, n);
+  const int64_t tiles = ((m + bm - 1) / bm) * (n / BN);
   const int64_t nk = k / BK;
-  int64_t s = 1;
-  while (tiles * s < 384 && nk / (s * 2) >= 4 && s < 32) s *= 2;
-  return (int)s;
+  // as many splits as still give one workgroup per CU (a second, partly filled round costs more than it gains),
+  // at least 4 k-tiles each
+  int64_t s = kNumCus / tiles;
+  if (s > 32) s = 32;
+  while (s > 1 && nk / s < 4) --s;
+  return (int)(s < 1 ? 1 : s);
 }
 
 int64_t aps_linear_nt_workspace_bytes(int64_t m, int64_t n, int64_t k) {
@@ -725,7 +761,8 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   g.a = (const char*)x; g.w = (const char*)weight; g.bias = bias;
   g.lda_b = x_stride * 2; g.ldw_b = w_stride * 2;
   g.m = m; g.n = n; g.k = k;
-  g.tiles_m = (int)((m + BM - 1) / BM); g.tiles_n = (int)(n / BN);
+  const int mi = tile_mi(m, n);
+  g.tiles_m = (int)((m + 64 * mi - 1) / (64 * mi)); g.tiles_n = (int)(n / BN);
   g.out = om;
   hipStream_t s = (hipStream_t)stream;
   if (m <= kRsMaxRows) return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
@@ -776,13 +813,21 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   if (splits > 1) splits = (int)((nk_all + g.kt_per_split - 1) / g.kt_per_split);  // no empty split
   const dim3 grid((unsigned)(per_xcd * kNumXcd), (unsigned)splits);
   // more than 64 KiB of dynamic LDS has to be allowed per function (and per device)
-  const void* fn = dtype == APS_BF16 ? (const void*)gemm_nt_kernel<true> : (const void*)gemm_nt_kernel<false>;
-  const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  hipError_t e = hipSuccess;
+#define APS_LAUNCH_TILE(B, M_)                                                                                     \
+  do {                                                                                                            \
+    e = hipFuncSetAttribute((const void*)gemm_nt_kernel<B, M_>, hipFuncAttributeMaxDynamicSharedMemorySize,       \
+                            TileShape<M_>::kLdsBytes);                                                            \
+    if (e == hipSuccess)                                                                                          \
+      hipLaunchKernelGGL((gemm_nt_kernel<B, M_>), grid, dim3(kThreads), TileShape<M_>::kLdsBytes, s, g);          \
+  } while (0)
+#define APS_LAUNCH_TILE_MI(B)                                                                        \
+  if (mi == 1) APS_LAUNCH_TILE(B, 1); else if (mi == 2) APS_LAUNCH_TILE(B, 2);                        \
+  else if (mi == 3) APS_LAUNCH_TILE(B, 3); else APS_LAUNCH_TILE(B, 4)
+  if (dtype == APS_BF16) { APS_LAUNCH_TILE_MI(true); } else { APS_LAUNCH_TILE_MI(false); }
+#undef APS_LAUNCH_TILE_MI
+#undef APS_LAUNCH_TILE
   if (e != hipSuccess) return (int)e;
-  if (dtype == APS_BF16)
-    hipLaunchKernelGGL(gemm_nt_kernel<true>, grid, dim3(kThreads), kLdsBytes, s, g);
-  else
-    hipLaunchKernelGGL(gemm_nt_kernel<false>, grid, dim3(kThreads), kLdsBytes, s, g);
   int st = launch_status();
   if (st != APS_OK || splits <= 1) return st;
   const int64_t quads = (m * n + 3) / 4;

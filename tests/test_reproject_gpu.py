@@ -21,14 +21,15 @@ pytestmark = pytest.mark.gpu
 def check(out, ref32, dtype=torch.float16):
     out = out.float().cpu()
     d = (out - ref32).abs()
-    assert d.max().item() <= 2e-2, f"max abs error {d.max().item()}"
+    if dtype == torch.float16:   # bf16 rounds in steps of 2^-8 relative: above |4| half a step alone exceeds 2e-2
+        assert d.max().item() <= 2e-2, f"max abs error {d.max().item()}"
     ulp = 2 ** -10 if dtype == torch.float16 else 2 ** -7
     bound = (1e-3 + ulp) * ref32.abs() + 2e-3
     bad = (d > bound).sum().item()
     assert bad == 0, f"{bad} elements outside tolerance, worst {d.max().item()}"
 
 
-@pytest.mark.parametrize("M", [1, 7, 255, 256, 257, 700])
+@pytest.mark.parametrize("M", [1, 7, 49, 64, 65, 128, 129, 192, 193, 255, 256, 257, 384, 385, 700])   # 64- to 256-row tiles
 @pytest.mark.parametrize("N,K", [(256, 64), (512, 192), (1536, 768)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_linear_nt_small(dev, M, N, K, dtype):
