@@ -204,7 +204,16 @@ __global__ __launch_bounds__(256) void nn_reduce_kernel(const float* __restrict_
   const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (idx >= per_part) return;
   float4v s = *(const float4v*)(partial + idx);
-  for (int p = 1; p < parts; ++p) {
+  int p = 1;
+  for (; p + 3 < parts; p += 4) {  // four independent loads in flight; additions in the order of one at a time
+    const float4v v0 = *(const float4v*)(partial + p * per_part + idx);
+    const float4v v1 = *(const float4v*)(partial + (p + 1) * per_part + idx);
+    const float4v v2 = *(const float4v*)(partial + (p + 2) * per_part + idx);
+    const float4v v3 = *(const float4v*)(partial + (p + 3) * per_part + idx);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s[i] = (((s[i] + v0[i]) + v1[i]) + v2[i]) + v3[i];
+  }
+  for (; p < parts; ++p) {
     const float4v v = *(const float4v*)(partial + p * per_part + idx);
     s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
   }
@@ -217,18 +226,9 @@ __global__ __launch_bounds__(256) void nn_reduce_kernel(const float* __restrict_
 
 // ------------------------------------------------------------------ scores over paged hidden rows
 // S[z][h][t] = sum_k hidden[row_ids[row_start[z] + t]][k] * qt[z][h][k]  (fp32), t < L(z).
-// One workgroup = kScWaves x 16 tokens of one sequence x all heads x all of K.  What hides the memory latency
-// on this part is bytes in flight per CU (loaded latency ~7 us), so hidden rows go straight from HBM into a
-// 16-step register ring per wavefront (16 KiB in flight each) and never through LDS.  Loads use the
-// coalescing layout (lane l: row l/4, 16-byte piece l%4: four adjacent lanes read 64 contiguous bytes; in
-// MFMA operand order neighbouring lanes would each fetch 16 bytes of a different row, which the memory
-// pipeline serves at a third of the rate) and a ds_bpermute per dword moves a block into operand order
-// (lane 16*g + c: token c, k = 32*step + 8*g) when it is consumed by v_mfma_f32_16x16x32.
-// The query image is the small, reused operand: 512 elements of K at a time, [heads][512], double buffered in
-// LDS (chunk c+1 is fetched into registers at the start of chunk c and written to LDS at its end); the
-// 16-byte chunk ch of head row r sits at position ch ^ (r % 16) of its 16-chunk group (conflict-free fragment
-// reads).  Nothing in the loop is conditional per lane or per step: a guard around a load makes the compiler
-// wait for every outstanding load, which empties the ring.
+// One workgroup = 128 tokens (8 wavefronts x 16) of one sequence x all heads x a part of K (all of it unless the
+// batch has few tiles), on the row-streaming core: the hidden rows are the streamed operand, the absorbed
+// queries qt[z] the LDS image.
 struct ScoreArgs {
   const char* cache; int64_t slot_stride_b, num_slots;
   const int64_t* row_ids; const int64_t* row_start;
@@ -395,19 +395,30 @@ template <bool BF16>
 __global__ __launch_bounds__(256) void softmax_rows_kernel(float* __restrict__ s, uint16_t* __restrict__ p,
                                                            const int64_t* __restrict__ row_start, int heads,
                                                            int64_t lp, int parts, int64_t part_stride) {
+  // Rows up to kCached scores are summed over the K parts once, 4 tokens per thread and step with the loads of
+  // all parts of a step independent of each other, and kept in LDS for the other two passes; longer rows keep
+  // their sums in part 0 of the global buffer (a thread meets the same tokens in every pass).
+  constexpr int kCached = 4096;
+  __shared__ __attribute__((aligned(16))) float cache[kCached];
   __shared__ float red[4];
   const int z = blockIdx.y, h = blockIdx.x;
   const int L = (int)(row_start[z + 1] - row_start[z]);
-  float* row = s + ((int64_t)z * heads + h) * lp;
+  float* row = s + ((int64_t)z * heads + h) * lp;   // 16-byte aligned: lp is a multiple of 32
   uint16_t* out = p + ((int64_t)z * heads + h) * lp;
-  // the first pass adds the partial scores of the K parts into part 0; a thread meets the same t in every pass
-  auto score = [&](int64_t t) { return row[t]; };
+  const bool in_lds = L <= kCached;
   float mx = -INFINITY;
-  for (int t = threadIdx.x; t < L; t += 256) {
-    float v = row[t];
-    for (int kp = 1; kp < parts; ++kp) v += row[kp * part_stride + t];
-    if (parts > 1) row[t] = v;
-    mx = fmaxf(mx, v);
+  for (int t = threadIdx.x * 4; t < L; t += 1024) {
+    float4 v = *(const float4*)(row + t);
+    for (int kp = 1; kp < parts; ++kp) {
+      const float4 q = *(const float4*)(row + kp * part_stride + t);
+      v.x += q.x; v.y += q.y; v.z += q.z; v.w += q.w;
+    }
+    if (in_lds) *(float4*)(cache + t) = v;
+    else if (parts > 1) *(float4*)(row + t) = v;
+    mx = fmaxf(mx, v.x);                       // tokens t+1.. past L hold finite padding of the scores kernel or
+    if (t + 1 < L) mx = fmaxf(mx, v.y);        // stale values: only tokens below L count
+    if (t + 2 < L) mx = fmaxf(mx, v.z);
+    if (t + 3 < L) mx = fmaxf(mx, v.w);
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
@@ -415,17 +426,32 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(float* __restrict__ s
   __syncthreads();
   mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   __syncthreads();
+  const float* src = in_lds ? cache : row;     // each thread re-reads what it wrote itself
   float sum = 0.f;
-  for (int t = threadIdx.x; t < L; t += 256) sum += exp2f(score(t) - mx);
+  for (int t = threadIdx.x * 4; t < L; t += 1024) {
+    const float4 v = *(const float4*)(src + t);
+    sum += exp2f(v.x - mx);
+    if (t + 1 < L) sum += exp2f(v.y - mx);
+    if (t + 2 < L) sum += exp2f(v.z - mx);
+    if (t + 3 < L) sum += exp2f(v.w - mx);
+  }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = sum;
   __syncthreads();
   sum = (red[0] + red[1]) + (red[2] + red[3]);
   const float inv = 1.f / sum;
-  for (int64_t t = threadIdx.x; t < lp; t += 256) {
-    const float v = t < L ? exp2f(score(t) - mx) * inv : 0.f;
-    out[t] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+  for (int64_t t = threadIdx.x * 4; t < lp; t += 1024) {   // zero padded up to lp
+    float4 v = {0.f, 0.f, 0.f, 0.f};
+    if (t < L) v = *(const float4*)(src + t);
+    uint16_t o[4];
+    const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float pv = t + i < L ? exp2f(e[i] - mx) * inv : 0.f;
+      o[i] = BF16 ? f32_to_bf16_bits(pv) : f32_to_f16_bits(pv);
+    }
+    *(uint2*)(out + t) = uint2{(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
   }
 }
 
@@ -459,8 +485,8 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   p.lp = align_up(max_len > 0 ? max_len : 1, 32);
   const int64_t col_tiles = (hidden + kNnWaves * 128 - 1) / (kNnWaves * 128);
   int64_t parts = 1;
-  // few sequences: split the tokens so that about two workgroups per CU exist
-  while (n_seqs * col_tiles * parts < 512 && p.lp / (parts * 2) >= 64) parts *= 2;
+  // few sequences: split the tokens into as many parts (of at least 64) as still give one workgroup per CU
+  while (n_seqs * col_tiles * (parts + 1) <= 256 && p.lp / (parts + 1) >= 64) ++parts;
   while (p.lp / parts > kNnMaxPart) parts *= 2;
   p.k_per_part = (int)align_up((p.lp + parts - 1) / parts, 32);
   p.kparts = (int)((p.lp + p.k_per_part - 1) / p.k_per_part);

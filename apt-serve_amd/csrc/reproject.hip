@@ -684,9 +684,22 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (idx >= m * n) return;
   const int64_t row = idx / n, col = idx - row * n;
+  // four partials at a time: independent loads in flight instead of one memory latency per split
   float4 s = *(const float4*)(partial + idx);
-  for (int z = 1; z < splits; ++z) {
-    const float4 p = *(const float4*)(partial + (int64_t)z * m * n + idx);
+  const int64_t plane = m * n;
+  int z = 1;
+  for (; z + 3 < splits; z += 4) {
+    const float4 p0 = *(const float4*)(partial + (int64_t)z * plane + idx);
+    const float4 p1 = *(const float4*)(partial + (int64_t)(z + 1) * plane + idx);
+    const float4 p2 = *(const float4*)(partial + (int64_t)(z + 2) * plane + idx);
+    const float4 p3 = *(const float4*)(partial + (int64_t)(z + 3) * plane + idx);
+    s.x += p0.x; s.y += p0.y; s.z += p0.z; s.w += p0.w;   // same order of additions as one at a time
+    s.x += p1.x; s.y += p1.y; s.z += p1.z; s.w += p1.w;
+    s.x += p2.x; s.y += p2.y; s.z += p2.z; s.w += p2.w;
+    s.x += p3.x; s.y += p3.y; s.z += p3.z; s.w += p3.w;
+  }
+  for (; z < splits; ++z) {
+    const float4 p = *(const float4*)(partial + (int64_t)z * plane + idx);
     s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
   }
   if (bias) {
