@@ -402,7 +402,7 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(float* __restrict__ s
   __shared__ __attribute__((aligned(16))) float cache[kCached];
   __shared__ float red[4];
   const int z = blockIdx.y, h = blockIdx.x;
-  const int L = (int)(row_start[z + 1] - row_start[z]);
+  const int L = (int)min(row_start[z + 1] - row_start[z], lp);  // a sequence longer than the stated maximum: its head
   float* row = s + ((int64_t)z * heads + h) * lp;   // 16-byte aligned: lp is a multiple of 32
   uint16_t* out = p + ((int64_t)z * heads + h) * lp;
   const bool in_lds = L <= kCached;

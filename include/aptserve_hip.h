@@ -334,10 +334,12 @@ int aps_build_prefill_metadata(
  * out_stride elements; negative or >= out_rows: skipped) — the epilogue that
  * writes re-projected K/V rows straight into [blocks, BS, H, D] tiles by slot.
  * workspace (nullable): fp32 scratch of aps_linear_nt_workspace_bytes(m,n,k)
- * bytes, 16-byte aligned, owned by the caller.  With it, a problem of few
- * output tiles (a decode step's handful of rows) is split along K into
- * aps_linear_nt_splits(m,n,k) partial products that a second kernel adds (in
- * fp32, then bias, then one rounding); without it one workgroup per tile runs.
+ * bytes, 16-byte aligned, owned by the caller.  With it, a problem whose output
+ * tiles leave CUs idle (a decode step's rows: anything from 3 rows up to a few
+ * hundred) is split along K into aps_linear_nt_splits(m,n,k) partial products
+ * that a second kernel adds (in fp32, then bias, then one rounding); without it
+ * a single-launch kernel runs.  A workspace that is passed but too small or
+ * misaligned is an error (APS_ERR_WORKSPACE), never a silent fallback.
  * ------------------------------------------------------------------------ */
 int aps_linear_nt_splits(int64_t m, int64_t n, int64_t k);
 int64_t aps_linear_nt_workspace_bytes(int64_t m, int64_t n, int64_t k);
