@@ -485,8 +485,16 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   p.lp = align_up(max_len > 0 ? max_len : 1, 32);
   const int64_t col_tiles = (hidden + kNnWaves * 128 - 1) / (kNnWaves * 128);
   int64_t parts = 1;
-  // few sequences: split the tokens into as many parts (of at least 64) as still give one workgroup per CU
-  while (n_seqs * col_tiles * (parts + 1) <= 256 && p.lp / (parts + 1) >= 64) ++parts;
+  // Fewer workgroups than CUs (few sequences): split the tokens.  A workgroup walks its tokens one after the
+  // other at ~29 GB/s, so without a split the longest sequence sets the kernel's time.  The host knows only the
+  // longest length; with lengths spread like a serving batch's the rows in all are about a third of
+  // n_seqs * longest, and a part should hold about 1/256 of the work of one column tile.
+  if (n_seqs * col_tiles < 256) {
+    int64_t target = n_seqs * p.lp * col_tiles / 3 / 256;
+    if (target < 64) target = 64;
+    parts = (p.lp + target - 1) / target;
+    if (parts > 32) parts = 32;
+  }
   while (p.lp / parts > kNnMaxPart) parts *= 2;
   p.k_per_part = (int)align_up((p.lp + parts - 1) / parts, 32);
   p.kparts = (int)((p.lp + p.k_per_part - 1) / p.k_per_part);
