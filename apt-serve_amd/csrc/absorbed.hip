@@ -8,11 +8,13 @@
 // so the hidden rows are read twice (scores, then the weighted sum) and the projections shrink to
 // products with one row per sequence and head:
 //   1. qt[s][h][:]  = scale*log2(e) * W_k[h]^T q[s][h]            nn_few_rows_kernel (B = rows of W_k)
-//   2. S[s][h][t]   = <qt[s][h], h_t>                               hidden_scores_kernel (paged rows)
+//   2. S[s][h][t]   = <qt[s][h], h_t>                               seq_plan_kernel (work list of the ragged
+//                                                                   batch), hidden_scores_kernel (paged rows)
 //   3. P[s][h][:]   = softmax_t, 16-bit, zero padded                softmax_rows_kernel
 //   4. ctx[s][h][:] = sum_t P[s][h][t] h_t                          nn_few_rows_kernel (B = paged rows)
-//   5. out[s][h*D+d] = <W_v[h*D+d], ctx[s][h]> + b_v                the weight-streaming kernels of the
-//                                                                   projection file, x chosen per head
+//   5. out[s][h*D+d] = <W_v[h*D+d], ctx[s][h]> + b_v                head_proj_kernel; up to 16 sequences: the
+//                                                                   weight-streaming kernels of the projection
+//                                                                   file, x chosen per head
 // Per cached token and layer that is 2 x Hd x 2 bytes of HBM reads and ~4*H*Hd flops, against a
 // gather, a 4*Hd*Hd-flop GEMM, a cache write and an attention read for the re-projection flow.
 #include "aps_common.h"

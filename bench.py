@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip attention / re-projection figures")
-    ap.add_argument("--extras", default="attention,metadata,write,reproject,layer,step_loop",
+    ap.add_argument("--extras", default="attention,prefill,metadata,write,reproject,layer,step_loop",
                     help="comma-separated subset of the extra figures to run")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="first run the plain copy kernel on 1 GiB three times (known traffic for counter scaling)")
@@ -232,6 +232,8 @@ def main():
             extras["metadata_build_us_cpu_list_algorithm"] = median(t)
         if "write" in want:
             extras["kv_write_prefill_16384"] = write_figures(torch, ops, dev, args.seed)
+        if "prefill" in want:
+            extras["prompt_attention_4x2048"] = prompt_attention_figures(torch, ops, dev, args.seed)
         if "reproject" in want:
             extras.update(reproject_figures(torch, ops, dev, args.seed))
         torch.cuda.empty_cache()
@@ -251,6 +253,25 @@ def main():
         result["cpu_baseline"] = cpu_baseline(torch, np, batch, md, cache, hs, key, value, kv_seq_idx, new_slots,
                                               step_bytes, T, Hd)
     print(json.dumps(result))
+
+
+def prompt_attention_figures(torch, ops, dev, seed):
+    """Causal attention of a prompt step (the flash_attn_varlen_func call of the reference's prompt path) at
+    OPT-13B width: 4 prompts of 2048 tokens, packed.  FLOPs counted as the causal half of QK^T and PV."""
+    H, D, lens = 40, 128, [2048] * 4
+    T = sum(lens)
+    g = torch.Generator(device=dev).manual_seed(seed)
+    q, k, v = (torch.randn(T, H, D, generator=g, device=dev).half() for _ in range(3))
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=dev)
+    out = torch.empty_like(q)
+    ms = median(event_times(torch, lambda: ops.flash_attn_varlen_func(q, k, v, cu, cu, max(lens), max(lens),
+                                                                      causal=True, out=out), 10))
+    flops = sum(2 * 2 * L * L * H * D / 2 for L in lens)
+    tf = flops / ms / 1e9
+    return {"workload": "causal varlen attention, 4 prompts x 2048 tokens, 40 heads x 128, fp16", "ms": ms,
+            "tokens_per_s": T / ms * 1e3, "algorithmic_flops": flops,
+            "roofline": {"bound": "mfma", "achieved": tf, "peak": 2500.0, "unit": "TFLOP/s", "frac": tf / 2500.0,
+                         "traffic": None}}
 
 
 def write_figures(torch, ops, dev, seed):
