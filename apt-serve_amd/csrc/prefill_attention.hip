@@ -101,29 +101,58 @@ __global__ __launch_bounds__(kThreads) void prefill_attention_kernel(const Prefi
     for (int e = 0; e < 16; ++e) o[t][e] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  const int kv_end = min(len, q0 + BQ);  // causal: keys beyond the tile's last query are never needed
-  for (int kv0 = 0; kv0 < kv_end; kv0 += BKV) {
-    __syncthreads();  // previous tile fully consumed
-    // ---- stage K (row-major, swizzled) and V (transposed)
-    for (int c = tid; c < BKV * KCH; c += kThreads) {
-      const int key = c / KCH, ch = c % KCH;
-      const int gk = min(kv0 + key, len - 1);
-      const u32x4 kvv = *(const u32x4*)(a.k + (int64_t)(s0 + gk) * a.k_stride_b + (int64_t)head * D * 2 + ch * 16);
-      *(u32x4*)(k_lds + key * KROW + ((ch ^ (key & (KCH - 1) & 15)) * 16)) = kvv;
-    }
-    for (int c = tid; c < BKV * KCH; c += kThreads) {
-      const int key = c % BKV, ch = c / BKV;   // consecutive lanes -> consecutive keys of one d-chunk
-      const int gk = min(kv0 + key, len - 1);
-      const u32x4 vv = *(const u32x4*)(a.v + (int64_t)(s0 + gk) * a.v_stride_b + (int64_t)head * D * 2 + ch * 16);
-      const int pos = vt_pos(key);
+  // Staging: thread tid moves pieces tid + 256*j (j < PER) of the K tile and of the V tile; the pieces of the
+  // next tile are loaded into registers before the current tile is multiplied and written to LDS after it.
+  constexpr int PER = BKV * KCH / kThreads;
+  const char* k_base = a.k + (int64_t)s0 * a.k_stride_b + (int64_t)head * D * 2;
+  const char* v_base = a.v + (int64_t)s0 * a.v_stride_b + (int64_t)head * D * 2;
+  u32x4 kreg[PER], vreg[PER];
+  auto fetch_tile = [&](int kv0) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t w = vv[i];
-        *(uint16_t*)(vt_lds + (ch * 8 + 2 * i) * VPITCH + pos * 2) = (uint16_t)(w & 0xffffu);
-        *(uint16_t*)(vt_lds + (ch * 8 + 2 * i + 1) * VPITCH + pos * 2) = (uint16_t)(w >> 16);
+    for (int j = 0; j < PER; ++j) {
+      const int c = tid + j * kThreads;
+      {
+        const int key = c / KCH, ch = c % KCH;
+        const int gk = min(kv0 + key, len - 1);
+        kreg[j] = *(const u32x4*)(k_base + (int64_t)gk * a.k_stride_b + ch * 16);
+      }
+      {
+        const int key = c % BKV, ch = c / BKV;   // consecutive lanes -> consecutive keys of one d-chunk
+        const int gk = min(kv0 + key, len - 1);
+        vreg[j] = *(const u32x4*)(v_base + (int64_t)gk * a.v_stride_b + ch * 16);
       }
     }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int c = tid + j * kThreads;
+      {
+        const int key = c / KCH, ch = c % KCH;
+        *(u32x4*)(k_lds + key * KROW + ((ch ^ (key & (KCH - 1) & 15)) * 16)) = kreg[j];
+      }
+      {
+        const int key = c % BKV, ch = c / BKV;
+        const int pos = vt_pos(key);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t w = vreg[j][i];
+          *(uint16_t*)(vt_lds + (ch * 8 + 2 * i) * VPITCH + pos * 2) = (uint16_t)(w & 0xffffu);
+          *(uint16_t*)(vt_lds + (ch * 8 + 2 * i + 1) * VPITCH + pos * 2) = (uint16_t)(w >> 16);
+        }
+      }
+    }
+  };
+
+  const int kv_end = min(len, q0 + BQ);  // causal: keys beyond the tile's last query are never needed
+  const int wave_q0 = q0 + wave * 32;    // first query of this wavefront
+  fetch_tile(0);
+  for (int kv0 = 0; kv0 < kv_end; kv0 += BKV) {
+    __syncthreads();  // previous tile fully consumed
+    store_tile();
     __syncthreads();
+    if (kv0 + BKV < kv_end) fetch_tile(kv0 + BKV);  // in flight while this tile is multiplied
+    if (kv0 > wave_q0 + 31) continue;               // every key of the tile lies after this wavefront's queries
 
     // ---- S^T = K Q^T for the two 32-key tiles
     float16v st[2];
@@ -140,13 +169,18 @@ __global__ __launch_bounds__(kThreads) void prefill_attention_kernel(const Prefi
       }
     }
     // ---- online softmax for this lane's query (its 32 keys here, the other 32 in lane^32)
+    // Only a tile that reaches past the wavefront's first query or past the sequence needs the mask.
+    const bool masked = kv0 + BKV - 1 > wave_q0 || kv0 + BKV > len;
     float mx = m_run;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int key = kv0 + t * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
-        const float sc = (key <= my_q && key < len) ? st[t][e] * a.scale_log2 : -INFINITY;
+        float sc = st[t][e] * a.scale_log2;
+        if (masked) {
+          const int key = kv0 + t * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+          if (!(key <= my_q && key < len)) sc = -INFINITY;
+        }
         st[t][e] = sc;
         mx = fmaxf(mx, sc);
       }
