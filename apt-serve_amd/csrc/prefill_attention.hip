@@ -67,14 +67,21 @@ __device__ __forceinline__ int vt_pos(int key) {  // see the file comment
 }
 
 template <bool BF16, int D>
-__global__ __launch_bounds__(kThreads) void prefill_attention_kernel(const PrefillArgs a) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attention_kernel(const PrefillArgs a) {
   constexpr int KS = D / 16;          // k-steps of the score product
   constexpr int DT = D / 32;          // 32-row tiles of O^T
   constexpr int KROW = D * 2;         // bytes per key row in LDS
   constexpr int KCH = KROW / 16;      // 16-byte chunks per key row
-  constexpr int VPITCH = BKV * 2 + 16;  // bytes per d-row of V^T (padding keeps rows off the same banks)
+  // V^T in LDS: row d = 64 keys in stored order (8 chunks of 8 keys, 16 bytes each); chunk o of row d sits at
+  // slot o ^ ((d/8 ^ d/2) % 8), and rows 64.. start 128 bytes (32 banks) later.  With that both the fragment
+  // reads (16 lanes = 16 consecutive d, one chunk) and the transposed stores (16 lanes = rows 8 apart, one
+  // chunk) touch 16 different 16-byte bank groups.
+  constexpr int VROW = BKV * 2;
   __shared__ __attribute__((aligned(16))) char k_lds[BKV * KROW];
-  __shared__ __attribute__((aligned(16))) char vt_lds[D * VPITCH];
+  __shared__ __attribute__((aligned(16))) char vt_lds[D * VROW + 128];
+  auto vt_addr = [&](int d, int chunk) {
+    return vt_lds + d * VROW + ((d >> 6) << 7) + ((chunk ^ (((d >> 3) ^ (d >> 1)) & 7)) << 4);
+  };
 
   const int seq = blockIdx.z, head = blockIdx.y;
   const int s0 = a.cu_seqlens[seq], s1 = a.cu_seqlens[seq + 1];
@@ -101,45 +108,50 @@ __global__ __launch_bounds__(kThreads) void prefill_attention_kernel(const Prefi
     for (int e = 0; e < 16; ++e) o[t][e] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  // Staging: thread tid moves pieces tid + 256*j (j < PER) of the K tile and of the V tile; the pieces of the
-  // next tile are loaded into registers before the current tile is multiplied and written to LDS after it.
-  constexpr int PER = BKV * KCH / kThreads;
+  // Staging.  K: thread tid moves the 16-byte pieces tid + 256*j of the tile (row-major, swizzled).  V: thread
+  // (octet o, d-chunk ch), o = tid / KCH < 8, loads the 8 keys whose stored positions are 8o .. 8o+7 (16 bytes = 8 d
+  // each: 16 lanes read 256 contiguous bytes of a key row), transposes the 8x8 block in registers with v_perm and
+  // stores 8 rows d of 16 bytes (8 keys).  The pieces of the next tile are loaded into registers before the
+  // current tile is multiplied and written to LDS after it.
+  constexpr int PER_K = BKV * KCH / kThreads;
+  const bool v_thread = tid < 8 * KCH;           // whole wavefronts
+  const int vo = tid / KCH, vch = tid % KCH;
   const char* k_base = a.k + (int64_t)s0 * a.k_stride_b + (int64_t)head * D * 2;
-  const char* v_base = a.v + (int64_t)s0 * a.v_stride_b + (int64_t)head * D * 2;
-  u32x4 kreg[PER], vreg[PER];
+  const char* v_base = a.v + (int64_t)s0 * a.v_stride_b + (int64_t)head * D * 2 + vch * 16;
+  u32x4 kreg[PER_K], vreg[8];
   auto fetch_tile = [&](int kv0) {
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {
+    for (int j = 0; j < PER_K; ++j) {
       const int c = tid + j * kThreads;
-      {
-        const int key = c / KCH, ch = c % KCH;
+      const int key = c / KCH, ch = c % KCH;
+      const int gk = min(kv0 + key, len - 1);
+      kreg[j] = *(const u32x4*)(k_base + (int64_t)gk * a.k_stride_b + ch * 16);
+    }
+    if (v_thread) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {  // stored position 8*vo + j holds this key (see the file comment)
+        const int key = (vo >> 1) * 16 + (vo & 1) * 4 + (j & 3) + (j >> 2) * 8;
         const int gk = min(kv0 + key, len - 1);
-        kreg[j] = *(const u32x4*)(k_base + (int64_t)gk * a.k_stride_b + ch * 16);
-      }
-      {
-        const int key = c % BKV, ch = c / BKV;   // consecutive lanes -> consecutive keys of one d-chunk
-        const int gk = min(kv0 + key, len - 1);
-        vreg[j] = *(const u32x4*)(v_base + (int64_t)gk * a.v_stride_b + ch * 16);
+        vreg[j] = *(const u32x4*)(v_base + (int64_t)gk * a.v_stride_b);
       }
     }
   };
   auto store_tile = [&]() {
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {
+    for (int j = 0; j < PER_K; ++j) {
       const int c = tid + j * kThreads;
-      {
-        const int key = c / KCH, ch = c % KCH;
-        *(u32x4*)(k_lds + key * KROW + ((ch ^ (key & (KCH - 1) & 15)) * 16)) = kreg[j];
-      }
-      {
-        const int key = c % BKV, ch = c / BKV;
-        const int pos = vt_pos(key);
+      const int key = c / KCH, ch = c % KCH;
+      *(u32x4*)(k_lds + key * KROW + ((ch ^ (key & (KCH - 1) & 15)) * 16)) = kreg[j];
+    }
+    if (v_thread) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint32_t w = vreg[j][i];
-          *(uint16_t*)(vt_lds + (ch * 8 + 2 * i) * VPITCH + pos * 2) = (uint16_t)(w & 0xffffu);
-          *(uint16_t*)(vt_lds + (ch * 8 + 2 * i + 1) * VPITCH + pos * 2) = (uint16_t)(w >> 16);
-        }
+      for (int dd = 0; dd < 8; ++dd) {  // row d = 8*vch + dd: dword p = (key position 2p, 2p+1)
+        const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;
+        u32x4 col;
+#pragma unroll
+        for (int p4 = 0; p4 < 4; ++p4)
+          col[p4] = __builtin_amdgcn_perm(vreg[2 * p4 + 1][dd >> 1], vreg[2 * p4][dd >> 1], sel);
+        *(u32x4*)vt_addr(vch * 8 + dd, vo) = col;
       }
     }
   };
@@ -211,10 +223,10 @@ __global__ __launch_bounds__(kThreads) void prefill_attention_kernel(const Prefi
         u32x4 pf;
 #pragma unroll
         for (int i = 0; i < 4; ++i) pf[i] = pack2<BF16>(st[t32][8 * ks + 2 * i], st[t32][8 * ks + 2 * i + 1]);
-        const int kpos = (t32 * 2 + ks) * 16 + half * 8;  // this lane's 8 keys of the step, in stored order
+        const int chunk = (t32 * 2 + ks) * 2 + half;  // this lane's 8 keys of the step, in stored order
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
-          const u32x4 vf = *(const u32x4*)(vt_lds + (t * 32 + qcol) * VPITCH + kpos * 2);
+          const u32x4 vf = *(const u32x4*)vt_addr(t * 32 + qcol, chunk);
           o[t] = mfma32<BF16>(vf, pf, o[t]);
         }
       }
