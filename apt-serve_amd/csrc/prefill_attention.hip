@@ -83,10 +83,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     return vt_lds + d * VROW + ((d >> 6) << 7) + ((chunk ^ (((d >> 3) ^ (d >> 1)) & 7)) << 4);
   };
 
-  const int seq = blockIdx.z, head = blockIdx.y;
+  // Grid (head, sequence, query tile), the last query tiles first: under the causal mask a workgroup's work grows
+  // with its tile's position, and workgroups start in grid order, so the long ones go first and the short ones
+  // fill the end (list scheduling).
+  const int seq = blockIdx.y, head = blockIdx.x;
   const int s0 = a.cu_seqlens[seq], s1 = a.cu_seqlens[seq + 1];
   const int len = s1 - s0;
-  const int q0 = blockIdx.x * BQ;
+  const int q0 = (int)(gridDim.z - 1 - blockIdx.z) * BQ;
   if (q0 >= len) return;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int qcol = lane & 31, half = lane >> 5;
@@ -277,7 +280,9 @@ int aps_varlen_prefill_attention(void* out, const void* q, const void* k, const 
   a.q_stride_b = q_stride * 2; a.k_stride_b = k_stride * 2; a.v_stride_b = v_stride * 2; a.out_stride_b = out_stride * 2;
   a.num_heads = num_heads;
   a.scale_log2 = softmax_scale * kLog2e;
-  const dim3 grid((unsigned)((max_seqlen + BQ - 1) / BQ), (unsigned)num_heads, (unsigned)num_seqs);
+  const int64_t q_tiles = (max_seqlen + BQ - 1) / BQ;
+  if (q_tiles > 65535) return APS_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)num_heads, (unsigned)num_seqs, (unsigned)q_tiles);
   hipStream_t s = (hipStream_t)stream;
   if (dtype == APS_F16) {
     if (head_size == 64) hipLaunchKernelGGL((prefill_attention_kernel<false, 64>), grid, dim3(kThreads), 0, s, a);
