@@ -8,14 +8,10 @@ namespace aps {
 namespace {
 
 // A workgroup is 8 wavefronts x 16 streamed rows; the image is staged 512 elements of K at a time; every
-// wavefront keeps a ring of 16 or 32 wave-wide loads (16 or 32 KiB) in flight.
+// wavefront keeps a ring of 16 wave-wide loads (16 KiB) in flight, one trip round the ring per chunk (a ring of
+// 32 loads, tried with 32- and 48-row images where one workgroup fits a CU, made long products slower and short
+// ones no faster).
 constexpr int kScWaves = 8, kScTokens = kScWaves * 16, kScThreads = kScWaves * 64, kScChunk = 512;
-// Chunks per trip round the register ring: the ring holds 16 loads (16 KiB per wavefront) per chunk.  One chunk
-// for every image size: a 32-load ring (measured with 32- and 48-row images, where one workgroup fits a CU)
-// made the long products slower and the short ones no faster.
-template <int NHT>
-constexpr int ring_chunks() { return 1; }
-
 // dynamic LDS of a kernel that calls the core: two buffers of [16*NHT image rows][512 k]
 template <int NHT>
 constexpr int scores_lds_bytes() { return 2 * NHT * 16 * kScChunk * 2; }
@@ -31,7 +27,7 @@ constexpr int scores_lds_bytes() { return 2 * NHT * 16 * kScChunk * 2; }
 // four.  For the even step (pieces 0-3) one DPP move first puts pieces 0-3 of rows 8-15 (second load, lanes
 // with l%8 < 4) over the lanes with l%8 >= 4 of the first load, so that a single ds_bpermute per dword finds
 // every (row, piece) in one register; the odd step mirrors that.
-template <bool BF16, int NHT, int CPT = ring_chunks<NHT>()>
+template <bool BF16, int NHT>
 __device__ __forceinline__ void stream_rows_times_image(const char* rowp0, const char* rowp1, const char* q_base,
                                                         int64_t q_row_stride_b, int q_rows, int64_t k, char* lds,
                                                         float4v (&acc)[NHT]) {
@@ -40,8 +36,8 @@ __device__ __forceinline__ void stream_rows_times_image(const char* rowp0, const
   static_assert(kPieces % kScThreads == 0, "pieces are spread evenly over the threads");
   constexpr int kPerThread = kPieces / kScThreads;
   constexpr int kChunkPairs = kScChunk / 64;
-  constexpr int kPairs = kChunkPairs * CPT;                       // pairs of loads in the ring: CPT chunks, so that
-  constexpr int kScRing = 2 * kPairs;                             // ring positions are static in the unrolled body
+  constexpr int kPairs = kChunkPairs;                             // pairs of loads in the ring = pairs of a chunk, so
+  constexpr int kScRing = 2 * kPairs;                             // that ring positions are static in the unrolled body
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int g4 = lane >> 4, c = lane & 15;
@@ -114,39 +110,32 @@ __device__ __forceinline__ void stream_rows_times_image(const char* rowp0, const
       af[ht] = *(const u32x4*)(qrow + ht * 16 * (kScChunk * 2) + ((ch & ~15) | ((ch ^ c) & 15)) * 16);
   };
 
-  // A trip round the ring is CPT chunks.  A chunk past the end of K (nchunks not a multiple of CPT) multiplies
-  // clamped loads with an image of zeros.
-  for (int it = 0; it < nchunks; it += CPT) {
+  for (int chunk = 0; chunk < nchunks; ++chunk) {
+    fetch_q(min(chunk + 1, nchunks - 1), qreg);
+    const char* qrow = lds + (chunk & 1) * kBuf + c * (kScChunk * 2);
+    const int i0 = chunk * kChunkPairs;
+    // The operands of step st+1 (a DPP move, a ds_bpermute and NHT LDS reads) are fetched while the MFMAs of
+    // step st run.
+    u32x4 bf[2], af[2][NHT];
 #pragma unroll
-    for (int cc = 0; cc < CPT; ++cc) {
-      const int chunk = it + cc;
-      fetch_q(min(chunk + 1, nchunks - 1), qreg);
-      const char* qrow = lds + (chunk & 1) * kBuf + c * (kScChunk * 2);
-      const int i0 = chunk * kChunkPairs;
-      // The operands of step st+1 (a DPP move, a ds_bpermute and NHT LDS reads) are fetched while the MFMAs of
-      // step st run.
-      u32x4 bf[2], af[2][NHT];
-#pragma unroll
-      for (int st = 0; st < 2 * kChunkPairs; ++st) {
-        const int u = cc * kChunkPairs + (st >> 1);   // pair within the ring
-        if ((st & 1) == 0) {
-          const int64_t ahead = pair_at(i0 + (st >> 1) + kPairs - 1);
-          ring[2 * ((u + kPairs - 1) % kPairs)] = __builtin_nontemporal_load((const u32x4*)(rowp0 + ahead));
-          ring[2 * ((u + kPairs - 1) % kPairs) + 1] = __builtin_nontemporal_load((const u32x4*)(rowp1 + ahead));
-          __builtin_amdgcn_sched_barrier(0);  // keep the loads here: the scheduler would sink them to their use
-        }
-        if (st == 0) fetch_operands(qrow, u, 0, bf[0], af[0]);
-        if (st + 1 < 2 * kChunkPairs)
-          fetch_operands(qrow, cc * kChunkPairs + ((st + 1) >> 1), st + 1, bf[(st + 1) & 1], af[(st + 1) & 1]);
-#pragma unroll
-        for (int ht = 0; ht < NHT; ++ht)
-          acc[ht] = mfma16<BF16>(af[st & 1][ht], bf[st & 1], acc[ht]);  // k past the end meets the image's zeros
-        if (st & 1) __builtin_amdgcn_sched_barrier(0);
+    for (int st = 0; st < 2 * kChunkPairs; ++st) {
+      const int u = st >> 1;   // pair within the ring
+      if ((st & 1) == 0) {
+        const int64_t ahead = pair_at(i0 + u + kPairs - 1);
+        ring[2 * ((u + kPairs - 1) % kPairs)] = __builtin_nontemporal_load((const u32x4*)(rowp0 + ahead));
+        ring[2 * ((u + kPairs - 1) % kPairs) + 1] = __builtin_nontemporal_load((const u32x4*)(rowp1 + ahead));
+        __builtin_amdgcn_sched_barrier(0);  // keep the loads here: the scheduler would sink them to their use
       }
-      store_q(chunk + 1, chunk + 1, qreg);  // the other buffer: last read one chunk ago, which every wavefront has left
-      APS_WAIT_LGKM0();
-      APS_BARRIER();
+      if (st == 0) fetch_operands(qrow, u, 0, bf[0], af[0]);
+      if (st + 1 < 2 * kChunkPairs) fetch_operands(qrow, (st + 1) >> 1, st + 1, bf[(st + 1) & 1], af[(st + 1) & 1]);
+#pragma unroll
+      for (int ht = 0; ht < NHT; ++ht)
+        acc[ht] = mfma16<BF16>(af[st & 1][ht], bf[st & 1], acc[ht]);  // k past the end meets the image's zeros
+      if (st & 1) __builtin_amdgcn_sched_barrier(0);
     }
+    store_q(chunk + 1, chunk + 1, qreg);  // the other buffer: last read one chunk ago, which every wavefront has left
+    APS_WAIT_LGKM0();
+    APS_BARRIER();
   }
 }
 
