@@ -271,7 +271,7 @@ __global__ __launch_bounds__(256) void seq_plan_kernel(const int64_t* __restrict
     part[threadIdx.x] = v;
     __syncthreads();
     for (int d = 1; d < 256; d <<= 1) {  // inclusive scan
-      const int add = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+      const int add = (int)threadIdx.x >= d ? part[threadIdx.x - d] : 0;
       __syncthreads();
       part[threadIdx.x] += add;
       __syncthreads();

@@ -9,8 +9,10 @@
 // to the operand dtype, are directly the B operand (k = keys) of O^T = V^T P^T, provided V^T is laid
 // out in LDS in the key order the result layout produces:
 //     position (key/16)*16 + ((key%8)/4)*8 + (key%16/8)*4 + key%4   holds   key.
-// V is transposed while it is staged (16-byte global loads, 16-bit LDS stores); K is staged row-major
+// V is transposed on its way into LDS: a thread loads an 8x8 block (the 8 keys of one 16-byte run of stored
+// positions, 8 consecutive d), transposes it in registers and stores 8 rows of V^T; K is staged row-major
 // with its 16-byte chunks XOR-swizzled by key%16 so the fragment reads do not collide in the 64 banks.
+// The next tile's pieces travel global -> registers while the current tile is multiplied.
 #include "aps_common.h"
 
 #include <math.h>
@@ -62,12 +64,11 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
   }
 }
 
-__device__ __forceinline__ int vt_pos(int key) {  // see the file comment
-  return (key & ~15) + ((key & 7) >> 2) * 8 + ((key & 15) >> 3) * 4 + (key & 3);
-}
-
 template <bool BF16, int D>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attention_kernel(const PrefillArgs a) {
+// Two wavefronts per SIMD: the kernel needs ~244 registers, and left to itself the compiler splits them into
+// 244 + 64 accumulation registers, which leaves room for one.
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attention_kernel(
+    const PrefillArgs a) {
   constexpr int KS = D / 16;          // k-steps of the score product
   constexpr int DT = D / 32;          // 32-row tiles of O^T
   constexpr int KROW = D * 2;         // bytes per key row in LDS
