@@ -42,3 +42,28 @@ def test_argument_errors_return_without_launching():
     assert lib.aps_hidden_to_cache(None, None, None, None, None, 0, 768, 768, 768, 0, 0, 0, 2, None) == 0
     assert lib.aps_hidden_to_cache(None, None, None, None, None, 4, 768, 768, 768, 0, 0, 0, 2, None) == -1
     assert lib.aps_hidden_to_cache(None, None, None, None, None, 4, 768, 768, 768, 0, 0, 0, 3, None) == -1
+
+
+def test_linear_workspace_planning_is_host_only_and_consistent():
+    """aps_linear_nt_splits / _workspace_bytes are pure host functions (no launch): the workspace is the fp32
+    partial tiles of every split, few-row products are split into whole 512-element chunks of K, and no plan asks
+    for more workgroups than the part has CUs unless the output tiles alone already do."""
+    lib = _lib.load()
+    shapes = [(5120, 5120), (10240, 5120), (15360, 5120), (20480, 5120), (5120, 20480), (256, 64), (1536, 768)]
+    for n, k in shapes:
+        for m in (1, 2, 3, 5, 16, 17, 48, 49, 64, 128, 129, 192, 256, 300, 700, 1024, 4096, 16384):
+            s = lib.aps_linear_nt_splits(m, n, k)
+            assert s >= 1
+            assert lib.aps_linear_nt_workspace_bytes(m, n, k) == (s * m * n * 4 if s > 1 else 0)
+            if m <= 2:
+                assert s == 1                                  # one launch of the dot-product kernel
+            elif m <= 48:
+                chunks = -(-k // 512)
+                assert s <= chunks
+                rows = 16 if m <= 16 else (32 if m <= 32 else 48)
+                tiles = -(-n // 128) * -(-m // rows)
+                assert s == 1 or tiles * s <= 256
+            else:
+                assert s == 1 or (n // 256) * s <= 256         # at least one row of tiles
+    # degenerate arguments plan nothing
+    assert lib.aps_linear_nt_splits(0, 5120, 5120) == 1 and lib.aps_linear_nt_workspace_bytes(0, 5120, 5120) == 0
