@@ -67,3 +67,23 @@ def test_linear_workspace_planning_is_host_only_and_consistent():
                 assert s == 1 or (n // 256) * s <= 256         # at least one row of tiles
     # degenerate arguments plan nothing
     assert lib.aps_linear_nt_splits(0, 5120, 5120) == 1 and lib.aps_linear_nt_workspace_bytes(0, 5120, 5120) == 0
+
+
+def test_absorbed_attention_workspace_planning_is_host_only():
+    """The workspace of the attention on hidden rows covers at least its named buffers (query image and context
+    rows: n*H*Hd 16-bit each; scores fp32 and probabilities 16-bit over the padded longest sequence), grows with
+    the batch, and degenerate arguments plan nothing."""
+    lib = _lib.load()
+    f = lib.aps_absorbed_attention_workspace_bytes
+    for heads, d in ((12, 64), (40, 128)):
+        hd = heads * d
+        prev = 0
+        for n in (1, 2, 8, 16, 17, 128, 300, 5000):
+            for max_len in (1, 33, 700, 2048):
+                lp = -(-max_len // 32) * 32
+                need = 2 * n * heads * hd * 2 + n * heads * lp * 4 + n * heads * lp * 2
+                got = f(n, max_len, heads, d)
+                assert got >= need and got % 256 == 0, (n, max_len, heads, d, got, need)
+            assert f(n, 2048, heads, d) > prev
+            prev = f(n, 2048, heads, d)
+    assert f(0, 100, 40, 128) == 0 and f(4, 0, 40, 128) == 0
