@@ -98,6 +98,11 @@ class HybridAttentionImpl:
         allowed; ``ops.mixed_reshape_and_cache`` in a prompt step), only the attention runs."""
         assert kv_scale == 1.0, "kv_scale is not supported"            # :312
         md = attn_metadata
+        if md.num_prefills and md.max_prompt_context_len > 0:
+            # the reference's prefix branch (aptserve_flash_attn.py:431-447) attends over the cache through the
+            # block table; the prompt attention here reads only this step's q/k/v
+            raise ValueError("prompt steps with an already-cached prefix (context_lens != 0) are not supported: "
+                             "prefix / chunked-prompt attention over the cache is not built")
         num_tokens, hidden_size = query.shape
         H, D = self.num_heads, self.head_size
         query = query.view(-1, H, D)

@@ -67,6 +67,7 @@ class HybridAttentionMetadata:
     kv_seq_lens: Optional[torch.Tensor] = None          # int32 [batch]: seq_len, 0 for hidden-cached sequences
     max_kv_seq_len: int = 0
     private_block_tables: Optional[torch.Tensor] = None  # int32 [batch, W]: every sequence's private table
+    max_prompt_context_len: int = 0   # longest already-cached prefix of a prompt step (0: plain prompts)
     _cached_prefill_metadata: Optional["HybridAttentionMetadata"] = None
     _cached_decode_metadata: Optional["HybridAttentionMetadata"] = None
 
@@ -91,7 +92,8 @@ class HybridAttentionMetadata:
                 seq_start_loc=self.seq_start_loc[:self.num_prefills + 1],
                 context_lens_tensor=self.context_lens_tensor[:self.num_prefills],
                 block_tables=self.block_tables[:self.num_prefills], use_cuda_graph=False,
-                input_positions=self.input_positions, block_types=None, token_is_hidden=self.token_is_hidden)
+                input_positions=self.input_positions, block_types=None, token_is_hidden=self.token_is_hidden,
+                max_prompt_context_len=self.max_prompt_context_len)
         return self._cached_prefill_metadata
 
     @property
@@ -324,7 +326,7 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
         max_prefill_seq_len=int(lens.max()), max_decode_seq_len=0, query_start_loc=query_start,
         seq_start_loc=seq_start, context_lens_tensor=ctx,
         block_tables=torch.empty(B, 0, **i32), use_cuda_graph=False, input_positions=positions, block_types=None,
-        token_is_hidden=token_is_hidden)
+        token_is_hidden=token_is_hidden, max_prompt_context_len=int(ctxs.max()))
 
 
 def build_from_batch(batch, device, **kw) -> HybridAttentionMetadata:

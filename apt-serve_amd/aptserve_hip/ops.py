@@ -590,7 +590,7 @@ def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_se
     with torch.cuda.device(dev):
         st = _lib.load().aps_varlen_prefill_attention(
             out.data_ptr() if T else None, q.data_ptr() if T else None, k.data_ptr() if T else None,
-            v.data_ptr() if T else None, _ptr(cu_seqlens_q), n_seq if T else 0, max_len, H, D, q.stride(0),
+            v.data_ptr() if T else None, _ptr(cu_seqlens_q), n_seq if T else 0, T, max_len, H, D, q.stride(0),
             k.stride(0), v.stride(0), out.stride(0), float(softmax_scale), _DTYPE_CODE[q.dtype], _stream(q))
     _lib.check(st, "flash_attn_varlen_func")
     return out

@@ -35,6 +35,7 @@ struct PrefillArgs {
   const int32_t* cu_seqlens;
   int64_t q_stride_b, k_stride_b, v_stride_b, out_stride_b;  // token row strides in bytes
   int num_heads;
+  int64_t num_tokens;  // rows of q / k / v / out: sequence boundaries outside [0, num_tokens] are not followed
   float scale_log2;
 };
 
@@ -89,6 +90,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   // fill the end (list scheduling).
   const int seq = blockIdx.y, head = blockIdx.x;
   const int s0 = a.cu_seqlens[seq], s1 = a.cu_seqlens[seq + 1];
+  if (s0 < 0 || s1 < s0 || s1 > a.num_tokens) return;  // boundaries come from device memory: never follow bad ones
   const int len = s1 - s0;
   const int q0 = (int)(gridDim.z - 1 - blockIdx.z) * BQ;
   if (q0 >= len) return;
@@ -260,11 +262,11 @@ using namespace aps;
 extern "C" {
 
 int aps_varlen_prefill_attention(void* out, const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
-                                 int64_t num_seqs, int64_t max_seqlen, int num_heads, int head_size,
-                                 int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t out_stride,
+                                 int64_t num_seqs, int64_t num_tokens, int64_t max_seqlen, int num_heads,
+                                 int head_size, int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t out_stride,
                                  float softmax_scale, int dtype, aps_stream_t stream) {
-  if (num_seqs < 0 || max_seqlen < 0 || num_heads <= 0 || head_size <= 0) return APS_ERR_INVALID_ARG;
-  if (num_seqs == 0 || max_seqlen == 0) return APS_OK;
+  if (num_seqs < 0 || num_tokens < 0 || max_seqlen < 0 || num_heads <= 0 || head_size <= 0) return APS_ERR_INVALID_ARG;
+  if (num_seqs == 0 || num_tokens == 0 || max_seqlen == 0) return APS_OK;
   if (!out || !q || !k || !v || !cu_seqlens) return APS_ERR_INVALID_ARG;
   if (dtype != APS_F16 && dtype != APS_BF16) return APS_ERR_UNSUPPORTED;
   if (head_size != 64 && head_size != 128) return APS_ERR_UNSUPPORTED;
@@ -280,6 +282,7 @@ int aps_varlen_prefill_attention(void* out, const void* q, const void* k, const 
   a.cu_seqlens = cu_seqlens;
   a.q_stride_b = q_stride * 2; a.k_stride_b = k_stride * 2; a.v_stride_b = v_stride * 2; a.out_stride_b = out_stride * 2;
   a.num_heads = num_heads;
+  a.num_tokens = num_tokens;
   a.scale_log2 = softmax_scale * kLog2e;
   const int64_t q_tiles = (max_seqlen + BQ - 1) / BQ;
   if (q_tiles > 65535) return APS_ERR_UNSUPPORTED;

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define APS_ABI_VERSION 3
+#define APS_ABI_VERSION 4
 
 typedef void* aps_stream_t; /* a hipStream_t; NULL = the null stream */
 
@@ -238,12 +238,16 @@ int aps_paged_decode_attention(
  * [num_seqs+1], leading 0); query i of a sequence attends to keys 0..i of the
  * same sequence; softmax in fp32; result in the operand dtype.
  * q/k/v/out: [tokens, H, D] with token-row strides (elements), heads
- * contiguous; f16 or bf16; D in {64, 128}.  max_seqlen: host-side bound of
- * the sequence lengths (sizes the grid).
+ * contiguous; f16 or bf16; D in {64, 128}.  num_tokens: rows of q/k/v/out; a
+ * sequence whose boundaries do not satisfy 0 <= cu[i] <= cu[i+1] <= num_tokens
+ * is skipped (its rows of out are not written).  max_seqlen: host-side bound
+ * of the sequence lengths (sizes the grid): queries at positions >= max_seqlen
+ * of a longer sequence are not computed, so it must not be an underestimate.
  * ------------------------------------------------------------------------ */
 int aps_varlen_prefill_attention(void* out, const void* q, const void* k,
                                  const void* v, const int32_t* cu_seqlens,
-                                 int64_t num_seqs, int64_t max_seqlen,
+                                 int64_t num_seqs, int64_t num_tokens,
+                                 int64_t max_seqlen,
                                  int num_heads, int head_size,
                                  int64_t q_stride, int64_t k_stride,
                                  int64_t v_stride, int64_t out_stride,
