@@ -360,7 +360,8 @@ def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
 def paged_decode_attention(q, k_cache, v_cache, block_tables, seq_lens, softmax_scale=None, *,
                            block_types=None, ws_k_cache=None, ws_v_cache=None, k_scale: float = 1.0,
                            v_scale: float = 1.0, max_seq_len: Optional[int] = None, partition_size: int = 0,
-                           out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):
+                           out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+                           static_scratch: bool = False):
     """Decode attention of one query token per sequence over paged K/V.
 
     ``q`` ``[B, H, D]`` f16/bf16; caches ``[blocks, BS, H, D]`` in ``q``'s dtype or
@@ -369,6 +370,9 @@ def paged_decode_attention(q, k_cache, v_cache, block_tables, seq_lens, softmax_
     (uint8 ``[B, W]``, optional) sends a logical block to ``ws_k_cache``/``ws_v_cache``
     when non-zero.  ``max_seq_len`` is a host-side bound on ``seq_lens`` (default
     ``W * BS``, which needs no device read-back).  Returns ``[B, H, D]``.
+    ``static_scratch=True`` (with ``out`` given) takes the entry point that allocates
+    nothing: partial results go to the library's static device array, and a problem
+    that does not fit it raises.
     """
     dev = q.device
     _check_data("q", q, dev)
@@ -419,6 +423,19 @@ def paged_decode_attention(q, k_cache, v_cache, block_tables, seq_lens, softmax_
     lib = _lib.load()
     if partition_size <= 0:
         partition_size = lib.aps_decode_attention_partition_size(B, H, max(max_seq_len, 1), BS)
+    if static_scratch:
+        with torch.cuda.device(dev):
+            st = lib.aps_paged_decode_attention_static(
+                out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                None if block_types is None else ws_k_cache.data_ptr(),
+                None if block_types is None else ws_v_cache.data_ptr(),
+                _ptr(block_tables), None if block_types is None else _ptr(block_types), _ptr(seq_lens), B, H, D, BS,
+                W, block_tables.stride(0) if W else 0, types_stride, q.stride(0), out.stride(0), k_cache.stride(0),
+                k_cache.size(0), ws_stride, ws_blocks, max_seq_len, partition_size, float(softmax_scale),
+                _DTYPE_CODE[q.dtype], APS_FP8_E4M3 if fp8 else _DTYPE_CODE[q.dtype], float(k_scale),
+                float(v_scale), _stream(q))
+        _lib.check(st, "paged_decode_attention_static")
+        return out
     need = lib.aps_decode_attention_workspace_bytes(B, H, D, max(max_seq_len, 1), partition_size)
     if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)

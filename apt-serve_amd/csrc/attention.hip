@@ -19,6 +19,8 @@
 
 #include <math.h>
 
+#include <mutex>
+
 #include "aps_common.h"
 
 namespace aps {
@@ -425,15 +427,16 @@ int64_t aps_decode_attention_workspace_bytes(int64_t batch, int num_heads, int h
   return align_up(n * head_size * 4, 256) + align_up(n * 4, 256);
 }
 
-int aps_paged_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
-                               const void* ws_k_cache, const void* ws_v_cache, const int32_t* block_tables,
-                               const uint8_t* block_types, const int32_t* seq_lens, int64_t batch, int num_heads,
-                               int head_size, int block_size, int64_t table_width, int64_t table_stride,
-                               int64_t types_stride, int64_t q_stride, int64_t out_stride,
-                               int64_t cache_block_stride, int64_t num_cache_blocks, int64_t ws_block_stride,
-                               int64_t num_ws_blocks, int64_t max_seq_len, int partition_size, float softmax_scale,
-                               int q_dtype, int kv_dtype, float k_scale, float v_scale, void* workspace,
-                               int64_t workspace_bytes, aps_stream_t stream) {
+// Both entry points: the scratch for the partial results is the caller's workspace or the library's static array.
+static int decode_attention_impl(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                 const void* ws_k_cache, const void* ws_v_cache, const int32_t* block_tables,
+                                 const uint8_t* block_types, const int32_t* seq_lens, int64_t batch, int num_heads,
+                                 int head_size, int block_size, int64_t table_width, int64_t table_stride,
+                                 int64_t types_stride, int64_t q_stride, int64_t out_stride,
+                                 int64_t cache_block_stride, int64_t num_cache_blocks, int64_t ws_block_stride,
+                                 int64_t num_ws_blocks, int64_t max_seq_len, int partition_size, float softmax_scale,
+                                 int q_dtype, int kv_dtype, float k_scale, float v_scale, void* workspace,
+                                 int64_t workspace_bytes, int too_small_status, aps_stream_t stream) {
   if (batch < 0 || num_heads <= 0 || head_size <= 0 || block_size <= 0 || table_width < 0) return APS_ERR_INVALID_ARG;
   if (batch == 0) return APS_OK;
   if (!out || !q || !seq_lens) return APS_ERR_INVALID_ARG;
@@ -476,7 +479,8 @@ int aps_paged_decode_attention(void* out, const void* q, const void* k_cache, co
   a.part_out = nullptr; a.part_lse = nullptr;
   if (np > 1) {
     const int64_t need = aps_decode_attention_workspace_bytes(batch, num_heads, head_size, max_seq_len, partition_size);
-    if (!workspace || workspace_bytes < need || (addr(workspace) & 15)) return APS_ERR_WORKSPACE;
+    if (workspace && workspace_bytes < need) return too_small_status;
+    if (!workspace || (addr(workspace) & 15)) return APS_ERR_WORKSPACE;
     const int64_t n = batch * num_heads * np;
     a.part_out = (float*)workspace;
     a.part_lse = (float*)((char*)workspace + align_up(n * head_size * 4, 256));
@@ -490,4 +494,66 @@ int aps_paged_decode_attention(void* out, const void* q, const void* k_cache, co
                                   : launch_decode<APS_BF16, KV_BF16>(a, head_size, batch, s);
 }
 
+int aps_paged_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
+                               const void* ws_k_cache, const void* ws_v_cache, const int32_t* block_tables,
+                               const uint8_t* block_types, const int32_t* seq_lens, int64_t batch, int num_heads,
+                               int head_size, int block_size, int64_t table_width, int64_t table_stride,
+                               int64_t types_stride, int64_t q_stride, int64_t out_stride,
+                               int64_t cache_block_stride, int64_t num_cache_blocks, int64_t ws_block_stride,
+                               int64_t num_ws_blocks, int64_t max_seq_len, int partition_size, float softmax_scale,
+                               int q_dtype, int kv_dtype, float k_scale, float v_scale, void* workspace,
+                               int64_t workspace_bytes, aps_stream_t stream) {
+  return decode_attention_impl(out, q, k_cache, v_cache, ws_k_cache, ws_v_cache, block_tables, block_types, seq_lens,
+                               batch, num_heads, head_size, block_size, table_width, table_stride, types_stride,
+                               q_stride, out_stride, cache_block_stride, num_cache_blocks, ws_block_stride,
+                               num_ws_blocks, max_seq_len, partition_size, softmax_scale, q_dtype, kv_dtype, k_scale,
+                               v_scale, workspace, workspace_bytes, APS_ERR_WORKSPACE, stream);
+}
+
 }  // extern "C"
+
+// ---------------------------------------------------------------- the entry point that allocates nothing
+// The partial results of split sequences live in a device array that is part of the library image: every GPU
+// the library runs on holds its own copy until the process ends.  In host code the array's name is only a
+// handle; the device address is looked up once per device and that pointer is what the kernels receive.
+static __device__ __align__(256) unsigned char scratch[APS_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[kMaxDevices];  // device address of `scratch` on every device seen so far
+
+// Device address of the scratch array on the current device (status != 0: the runtime's error code).
+void* scratch_on_current_device(int* status) {
+  *status = APS_OK;
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) { *status = (int)e; return nullptr; }
+  if (device < 0 || device >= kMaxDevices) { *status = APS_ERR_UNSUPPORTED; return nullptr; }
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[device]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) { *status = e != hipSuccess ? (int)e : APS_ERR_UNSUPPORTED; return nullptr; }
+    scratch_ptr[device] = p;
+  }
+  return scratch_ptr[device];
+}
+}  // namespace
+
+extern "C" int aps_paged_decode_attention_static(
+    void* out, const void* q, const void* k_cache, const void* v_cache, const void* ws_k_cache,
+    const void* ws_v_cache, const int32_t* block_tables, const uint8_t* block_types, const int32_t* seq_lens,
+    int64_t batch, int num_heads, int head_size, int block_size, int64_t table_width, int64_t table_stride,
+    int64_t types_stride, int64_t q_stride, int64_t out_stride, int64_t cache_block_stride, int64_t num_cache_blocks,
+    int64_t ws_block_stride, int64_t num_ws_blocks, int64_t max_seq_len, int partition_size, float softmax_scale,
+    int q_dtype, int kv_dtype, float k_scale, float v_scale, aps_stream_t stream) {
+  int st = APS_OK;
+  void* ws = scratch_on_current_device(&st);
+  if (st != APS_OK) return st;
+  return decode_attention_impl(out, q, k_cache, v_cache, ws_k_cache, ws_v_cache, block_tables, block_types, seq_lens,
+                               batch, num_heads, head_size, block_size, table_width, table_stride, types_stride,
+                               q_stride, out_stride, cache_block_stride, num_cache_blocks, ws_block_stride,
+                               num_ws_blocks, max_seq_len, partition_size, softmax_scale, q_dtype, kv_dtype, k_scale,
+                               v_scale, ws, APS_STATIC_SCRATCH_BYTES, APS_ERR_SCRATCH_LIMIT, stream);
+}

@@ -479,6 +479,7 @@ const char* aps_status_string(int status) {
     case APS_ERR_INVALID_ARG: return "invalid argument";
     case APS_ERR_UNSUPPORTED: return "unsupported shape or dtype";
     case APS_ERR_WORKSPACE: return "workspace too small";
+    case APS_ERR_SCRATCH_LIMIT: return "problem needs more scratch than the library's static array holds";
     default: return status > 0 ? hipGetErrorString((hipError_t)status) : "unknown status";
   }
 }

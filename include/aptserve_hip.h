@@ -4,7 +4,8 @@
  * One shared library, libaptserve_hip.so, exports every function below with C
  * linkage.  All pointers are device pointers unless a parameter says "host".
  * All tensors are owned by the caller; the library never allocates, frees or
- * retains device memory and keeps no global state, so calls are re-entrant.
+ * retains device memory and keeps no global state, so calls are re-entrant
+ * (one exception, documented there: aps_paged_decode_attention_static).
  * Work is enqueued on the given stream and the call returns without waiting.
  *
  * Return value: 0 on success; a negative aps_status on an argument error
@@ -32,7 +33,9 @@ enum aps_status {
   APS_OK = 0,
   APS_ERR_INVALID_ARG = -1, /* null pointer, negative size, bad enum */
   APS_ERR_UNSUPPORTED = -2, /* shape / dtype combination not built */
-  APS_ERR_WORKSPACE = -3    /* workspace too small */
+  APS_ERR_WORKSPACE = -3,    /* workspace too small */
+  APS_ERR_SCRATCH_LIMIT = -4 /* aps_paged_decode_attention_static: the problem
+                                needs more than APS_STATIC_SCRATCH_BYTES */
 };
 
 enum aps_dtype {
@@ -229,6 +232,33 @@ int aps_paged_decode_attention(
     int partition_size, float softmax_scale, int q_dtype, int kv_dtype,
     float k_scale, float v_scale, void* workspace, int64_t workspace_bytes,
     aps_stream_t stream);
+
+/* aps_paged_decode_attention for callers that cannot allocate device memory
+ * or bring a workspace: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same
+ * arguments and bit-identical results; the partial results of split sequences
+ * go to a device array of APS_STATIC_SCRATCH_BYTES that is part of the library
+ * image (one copy per GPU, held until the process ends) instead of a caller
+ * workspace.  The call allocates and frees nothing.  A problem that needs more
+ * (aps_decode_attention_workspace_bytes(...) > APS_STATIC_SCRATCH_BYTES) is
+ * rejected with APS_ERR_SCRATCH_LIMIT before anything is launched.  The device
+ * of the call is the current device.  Every call on a GPU uses that GPU's one
+ * array: calls that overlap in time on the same GPU (two streams, two
+ * threads) race; calls on one stream are ordered and safe.  Nothing in the
+ * array has to start at zero (every partial that is read was written by the
+ * same call), so it is never cleared. */
+#define APS_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)
+int aps_paged_decode_attention_static(
+    void* out, const void* q, const void* k_cache, const void* v_cache,
+    const void* ws_k_cache, const void* ws_v_cache,
+    const int32_t* block_tables, const uint8_t* block_types,
+    const int32_t* seq_lens, int64_t batch, int num_heads, int head_size,
+    int block_size, int64_t table_width, int64_t table_stride,
+    int64_t types_stride, int64_t q_stride, int64_t out_stride,
+    int64_t cache_block_stride, int64_t num_cache_blocks,
+    int64_t ws_block_stride, int64_t num_ws_blocks, int64_t max_seq_len,
+    int partition_size, float softmax_scale, int q_dtype, int kv_dtype,
+    float k_scale, float v_scale, aps_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Prompt-step attention on freshly projected q/k/v (no cache read).
