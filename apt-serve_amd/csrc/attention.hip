@@ -22,11 +22,11 @@
 #include <mutex>
 
 #include "aps_common.h"
+#include "mfma_common.h"
 
 namespace aps {
 namespace {
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float float2_t __attribute__((ext_vector_type(2)));
@@ -116,25 +116,41 @@ __device__ __forceinline__ uint16_t f32_to_q(float x) {
 }
 
 struct AttnArgs {
-  void* out;                 // [B, H, D] (q dtype) — written when num_partitions == 1
-  float* part_out;           // [B, H, P, D] fp32
+  void* out;                 // [B, H, D] (q dtype)
+  float* part_out;           // [B, H, P, D] fp32   (flat path only)
   float* part_lse;           // [B, H, P]   fp32 (log2 domain)
   const void* q;
   const char* k_cache; const char* v_cache;
   const char* ws_k_cache; const char* ws_v_cache;
   const int32_t* block_tables; const uint8_t* block_types; const int32_t* seq_lens;
+  const int32_t* seq_order;  // group path: sequence handled by workgroup row y (nullptr: rank in the kernel, or y itself)
   int64_t q_stride, out_stride, table_stride, types_stride;
   int64_t cache_block_stride_b, ws_block_stride_b;  // bytes
   int64_t num_cache_blocks, num_ws_blocks;
   int num_heads, block_size, partition_size, num_partitions, table_width;
+  int batch, rank_in_kernel;
   float scale_log2;  // softmax_scale * k_scale * log2(e)
   float v_scale;
 };
 
-// HPW adjacent heads share a wavefront: the LPT lanes of head h+1 sit next to those of head h, so one
-// token contributes HPW*D contiguous elements to a wave-wide load (longer DRAM bursts per token row).
-template <int QT, int KV, int D, int HPW>
-__global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
+// State of one wavefront after it has walked its partition: the LPR lanes of token row 0 hold, for their
+// (head, 16-byte chunk of the head vector), the running maximum m (log2 domain), the sum l of 2^(s - m) and the
+// unnormalised weighted sum acc of V.
+template <int EPL>
+struct WaveResult {
+  float m, l;
+  float acc[EPL];
+};
+
+// One wavefront walks tokens [start, end) of sequence `seq` for HPW adjacent heads starting at head0.
+// HPW adjacent heads share the wavefront: the LPT lanes of head h+1 sit next to those of head h, so one token
+// contributes HPW*D contiguous elements to a wave-wide load (longer DRAM bursts per token row).
+// DEPTH tiles of 16 tokens are in flight: the ring is filled with unconditional buffer loads (a tile past the
+// end of the partition, or one whose block id is unusable, gets a zero-length descriptor: its loads touch no
+// memory and return zeros), so no load sits under a branch and the compiler's wait counts stay exact.
+template <int QT, int KV, int D, int HPW, int DEPTH>
+__device__ __forceinline__ void decode_wave(const AttnArgs& a, int seq, int head0, int start, int end, int lane,
+                                            WaveResult<Unpack<KV>::EPL>& res) {
   constexpr int EPL = Unpack<KV>::EPL;        // elements per lane
   constexpr int LPT = D / EPL;                // lanes per (token, head)
   constexpr int LPR = LPT * HPW;              // lanes per token row of the wave
@@ -143,17 +159,9 @@ __global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
   static_assert(LPT >= 2 && LPR <= 32 && NG >= 1, "unsupported head size");
   constexpr int KV_ELEM_B = (KV == KV_FP8) ? 1 : 2;
 
-  const int part = blockIdx.y;
-  const int seq = blockIdx.z;
-  const int lane = threadIdx.x;
   const int tl = lane / LPR;                            // token row of this lane
-  const int head = blockIdx.x * HPW + (lane % LPR) / LPT;
+  const int head = head0 + (lane % LPR) / LPT;
   const int dl = lane % LPT;                            // 16-byte chunk of the head vector
-
-  const int seq_len = a.seq_lens[seq];
-  const int start = part * a.partition_size;
-  if (start >= seq_len && !(part == 0 && seq_len <= 0)) return;
-  const int end = min(seq_len, start + a.partition_size);
   const int n_tiles = (end > start) ? (end - start + kTile - 1) / kTile : 0;
 
   // query fragment of this lane: fp32, or, when the cache holds the query's 16-bit type, the packed pairs as
@@ -190,38 +198,44 @@ __global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
   }
 
   const int64_t row_b = (int64_t)a.num_heads * D * KV_ELEM_B;       // one token, all heads
-  const int64_t lane_off = (int64_t)head * D * KV_ELEM_B + dl * 16;  // this lane's chunk in a token row
+  const uint32_t tile_b = (uint32_t)(kTile * row_b);                // the 16 token rows of a tile
+  const uint32_t lane_voff = (uint32_t)(tl * row_b + (int64_t)head * D * KV_ELEM_B + dl * 16);
+  const uint32_t group_b = (uint32_t)(TPL * row_b);
+  const int tiles_per_block = a.block_size / kTile;                 // start is a multiple of the block size
 
   float m = -INFINITY, l = 0.f;
   float acc[EPL];
 #pragma unroll
   for (int i = 0; i < EPL; ++i) acc[i] = 0.f;
 
-  u32x4 kA[NG], vA[NG], kB[NG], vB[NG];
+  u32x4 kr[DEPTH][NG], vr[DEPTH][NG];
+  bool ok[DEPTH];
 
-  // Issue the loads of tile t into (kr, vr); returns false if the tile's block is unusable.
-  auto load_tile = [&](int t, u32x4(&kr)[NG], u32x4(&vr)[NG]) -> bool {
-    const int tok0 = start + t * kTile;
-    const int bi = tok0 / a.block_size - first_blk;
+  // Issue the loads of tile t; returns false if the tile does not exist or its block is unusable.
+  auto load_tile = [&](int t, u32x4(&kq)[NG], u32x4(&vq)[NG]) -> bool {
+    const bool in = t < n_tiles;
+    const int tt = in ? t : 0;
+    const int bi = tiles_per_block == 1 ? tt : tt / tiles_per_block;
+    const int in_blk = tiles_per_block == 1 ? 0 : tt - bi * tiles_per_block;
     const int blk = __builtin_amdgcn_readlane(my_blk, bi);
     const int type = __builtin_amdgcn_readlane(my_type, bi);
     const bool ws = type != 0;
     const int64_t nblk = ws ? a.num_ws_blocks : a.num_cache_blocks;
-    if (blk < 0 || blk >= nblk) return false;
-    const int64_t base = (int64_t)blk * (ws ? a.ws_block_stride_b : a.cache_block_stride_b) +
-                         (int64_t)(tok0 % a.block_size + tl) * row_b + lane_off;
-    const char* kp = (ws ? a.ws_k_cache : a.k_cache) + base;
-    const char* vp = (ws ? a.ws_v_cache : a.v_cache) + base;
+    const bool valid = in && blk >= 0 && blk < nblk;
+    const int64_t base = valid ? (int64_t)blk * (ws ? a.ws_block_stride_b : a.cache_block_stride_b) +
+                                     (int64_t)in_blk * tile_b
+                               : 0;
+    const __amdgpu_buffer_rsrc_t rk = make_rsrc((ws ? a.ws_k_cache : a.k_cache) + base, valid ? tile_b : 0);
+    const __amdgpu_buffer_rsrc_t rv = make_rsrc((ws ? a.ws_v_cache : a.v_cache) + base, valid ? tile_b : 0);
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
-      kr[g] = __builtin_nontemporal_load((const u32x4*)(kp + (int64_t)g * TPL * row_b));
-      vr[g] = __builtin_nontemporal_load((const u32x4*)(vp + (int64_t)g * TPL * row_b));
+      kq[g] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rk, lane_voff + g * group_b, 0, 2));
+      vq[g] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rv, lane_voff + g * group_b, 0, 2));
     }
-    return true;
+    return valid;
   };
 
-  auto consume_tile = [&](int t, bool ok, const u32x4(&kr)[NG], const u32x4(&vr)[NG]) {
-    if (!ok) return;
+  auto consume_tile = [&](int t, const u32x4(&kq)[NG], const u32x4(&vq)[NG]) {
     const int tok0 = start + t * kTile;
     const bool partial = tok0 + kTile > end;
     float s[NG];
@@ -231,7 +245,7 @@ __global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
       if constexpr (kDot2) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const uint32_t kw = kr[g][i], qw = qpk[i];
+          const uint32_t kw = kq[g][i], qw = qpk[i];
           if constexpr (KV == KV_F16)
             d = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, kw), __builtin_bit_cast(half2_t, qw), d, false);
           else
@@ -240,7 +254,7 @@ __global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
         }
       } else {
         float kf[EPL];
-        Unpack<KV>::run(kr[g], kf);
+        Unpack<KV>::run(kq[g], kf);
 #pragma unroll
         for (int i = 0; i < EPL; ++i) d = fmaf(qf[i], kf[i], d);
       }
@@ -265,7 +279,7 @@ __global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
       float vf[EPL];
-      Unpack<KV>::run(vr[g], vf);
+      Unpack<KV>::run(vq[g], vf);
       if (partial) {  // slots past the end of the sequence may hold anything, NaN included
         const bool live = tok0 + g * TPL + tl < end;
 #pragma unroll
@@ -277,13 +291,16 @@ __global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
     m = m_new;
   };
 
-  bool okA = false, okB = false;
-  if (n_tiles > 0) okA = load_tile(0, kA, vA);
-  for (int t = 0; t < n_tiles; t += 2) {
-    if (t + 1 < n_tiles) okB = load_tile(t + 1, kB, vB);
-    consume_tile(t, okA, kA, vA);
-    if (t + 2 < n_tiles) okA = load_tile(t + 2, kA, vA);
-    if (t + 1 < n_tiles) consume_tile(t + 1, okB, kB, vB);
+#pragma unroll
+  for (int i = 0; i < DEPTH - 1; ++i) ok[i] = load_tile(i, kr[i], vr[i]);
+  for (int t0 = 0; t0 < n_tiles; t0 += DEPTH) {
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) {
+      constexpr int kAhead = DEPTH - 1;
+      const int fill = (j + kAhead) % DEPTH;
+      ok[fill] = load_tile(t0 + j + kAhead, kr[fill], vr[fill]);
+      if (ok[j]) consume_tile(t0 + j, kr[j], vr[j]);  // uniform; a tile that does not exist is never ok
+    }
   }
 
   // merge the TPL token rows (lanes that share dl)
@@ -299,30 +316,147 @@ __global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
     for (int i = 0; i < EPL; ++i) acc[i] = acc[i] * wa + __shfl_xor(acc[i], off) * wb;
     m = m_n;
   }
+  res.m = m;
+  res.l = l;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) res.acc[i] = acc[i];
+}
 
-  if (tl != 0) return;
-  const float inv = (l > 0.f) ? a.v_scale / l : 0.f;
+// Rounded result of lane (head, dl): acc * inv -> out[seq, head, dl*EPL ...]
+template <int QT, int EPL, int D>
+__device__ __forceinline__ void store_out(const AttnArgs& a, int seq, int head, int dl, const float (&acc)[EPL],
+                                          float inv) {
+  uint16_t* op = (uint16_t*)a.out + (int64_t)seq * a.out_stride + (int64_t)head * D + dl * EPL;
+#pragma unroll
+  for (int i = 0; i < EPL; i += 8) {
+    u32x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      r[j] = (uint32_t)f32_to_q<QT>(acc[i + 2 * j] * inv) | ((uint32_t)f32_to_q<QT>(acc[i + 2 * j + 1] * inv) << 16);
+    *(u32x4*)(op + i) = r;
+  }
+}
+
+// Flat path: one wavefront (one 64-thread workgroup) per (head group, partition, sequence); partitions of one
+// (sequence, head) are combined by combine_partitions_kernel.  Used when a sequence has more partitions than a
+// workgroup has wavefronts.
+template <int QT, int KV, int D, int HPW, int DEPTH>
+__global__ __launch_bounds__(64) void paged_decode_kernel(const AttnArgs a) {
+  constexpr int EPL = Unpack<KV>::EPL, LPT = D / EPL, LPR = LPT * HPW;
+  const int part = blockIdx.y, seq = blockIdx.z, lane = threadIdx.x;
+  const int seq_len = a.seq_lens[seq];
+  const int start = part * a.partition_size;
+  if (start >= seq_len && !(part == 0 && seq_len <= 0)) return;
+  const int end = min(seq_len, start + a.partition_size);
+  WaveResult<EPL> r;
+  decode_wave<QT, KV, D, HPW, DEPTH>(a, seq, blockIdx.x * HPW, start, end, lane, r);
+  if (lane >= LPR) return;
+  const int head = blockIdx.x * HPW + lane / LPT, dl = lane % LPT;
+  const float inv = (r.l > 0.f) ? a.v_scale / r.l : 0.f;
   if (a.num_partitions == 1) {
-    uint16_t* op = (uint16_t*)a.out + (int64_t)seq * a.out_stride + (int64_t)head * D + dl * EPL;
-#pragma unroll
-    for (int i = 0; i < EPL; i += 8) {
-      u32x4 r;
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        r[j] = (uint32_t)f32_to_q<QT>(acc[i + 2 * j] * inv) |
-               ((uint32_t)f32_to_q<QT>(acc[i + 2 * j + 1] * inv) << 16);
-      *(u32x4*)(op + i) = r;
-    }
+    store_out<QT, EPL, D>(a, seq, head, dl, r.acc, inv);
   } else {
     const int64_t ph = ((int64_t)seq * a.num_heads + head) * a.num_partitions + part;
     float* po = a.part_out + ph * D + dl * EPL;
 #pragma unroll
     for (int i = 0; i < EPL; i += 4) {
-      float4 r = make_float4(acc[i] * inv, acc[i + 1] * inv, acc[i + 2] * inv, acc[i + 3] * inv);
-      *(float4*)(po + i) = r;
+      float4 v = make_float4(r.acc[i] * inv, r.acc[i + 1] * inv, r.acc[i + 2] * inv, r.acc[i + 3] * inv);
+      *(float4*)(po + i) = v;
     }
-    if (dl == 0) a.part_lse[ph] = (l > 0.f) ? m + log2f(l) : -INFINITY;
+    if (dl == 0) a.part_lse[ph] = (r.l > 0.f) ? r.m + log2f(r.l) : -INFINITY;
   }
+}
+
+constexpr int kRankInKernelMax = 512;  // up to this many sequences a workgroup ranks the lengths itself
+
+// Group path: one workgroup per (head group, sequence); wavefront w walks partition w of the sequence and the
+// wavefront that finishes last merges the partial results through LDS: no partials in HBM, no second launch.
+// Wavefronts whose partition is empty leave at once (their registers and wave slot are free from then on).
+// Workgroup rows are dealt out longest sequence first (list scheduling): the order comes from seq_order, or,
+// for batches up to kRankInKernelMax, from ranking the lengths in LDS at the start of every workgroup.
+template <int QT, int KV, int D, int HPW, int DEPTH, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void paged_decode_group_kernel(const AttnArgs a) {
+  constexpr int EPL = Unpack<KV>::EPL, LPT = D / EPL, LPR = LPT * HPW;
+  __shared__ int s_arrived, s_seq;
+  __shared__ int s_len[kRankInKernelMax];
+  __shared__ float s_part[WAVES][LPR][EPL + 2];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+
+  if (tid == 0) {
+    s_arrived = 0;
+    s_seq = a.seq_order ? a.seq_order[blockIdx.y] : (int)blockIdx.y;
+  }
+  if (a.rank_in_kernel) {
+    for (int j = tid; j < a.batch; j += 64 * WAVES) s_len[j] = a.seq_lens[j];
+    __syncthreads();
+    for (int j = tid; j < a.batch; j += 64 * WAVES) {
+      const int mine = s_len[j];
+      int rank = 0;
+      for (int k = 0; k < a.batch; ++k) {
+        const int other = s_len[k];
+        rank += (other > mine || (other == mine && k < j)) ? 1 : 0;
+      }
+      if (rank == (int)blockIdx.y) s_seq = j;
+    }
+  }
+  __syncthreads();
+  const int seq = s_seq;
+  const int seq_len = a.rank_in_kernel ? s_len[seq] : a.seq_lens[seq];
+  int np = (seq_len + a.partition_size - 1) / a.partition_size;
+  np = np < 1 ? 1 : (np > WAVES ? WAVES : np);
+  if (wave >= np) return;
+  const int start = wave * a.partition_size;
+  const int end = min(seq_len, start + a.partition_size);
+  WaveResult<EPL> r;
+  decode_wave<QT, KV, D, HPW, DEPTH>(a, seq, blockIdx.x * HPW, start, end, lane, r);
+  const int head = blockIdx.x * HPW + lane / LPT, dl = lane % LPT;
+  if (np == 1) {
+    if (lane < LPR) store_out<QT, EPL, D>(a, seq, head, dl, r.acc, (r.l > 0.f) ? a.v_scale / r.l : 0.f);
+    return;
+  }
+  if (lane < LPR) {
+    float* sp = s_part[wave][lane];
+    sp[0] = r.m;
+    sp[1] = r.l;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) sp[2 + i] = r.acc[i];
+  }
+  // LDS operations of a wavefront execute in order, and the counter is an LDS atomic: whoever reads np - 1 has
+  // every other wavefront's partial result in LDS already
+  int arrived = 0;
+  if (lane == 0) arrived = __hip_atomic_fetch_add(&s_arrived, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
+  arrived = __builtin_amdgcn_readfirstlane(arrived);
+  if (arrived != np - 1 || lane >= LPR) return;
+  // fixed order of the merge (partition 0, 1, ...), whoever is last: the result does not depend on timing
+  float m = -INFINITY;
+  for (int p = 0; p < np; ++p) m = fmaxf(m, s_part[p][lane][0]);
+  const float m_u = (m == -INFINITY) ? 0.f : m;
+  float l = 0.f, acc[EPL];
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) acc[i] = 0.f;
+  for (int p = 0; p < np; ++p) {
+    const float* sp = s_part[p][lane];
+    const float w = __builtin_amdgcn_exp2f(sp[0] - m_u);
+    l = fmaf(sp[1], w, l);
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) acc[i] = fmaf(sp[2 + i], w, acc[i]);
+  }
+  store_out<QT, EPL, D>(a, seq, head, dl, acc, (l > 0.f) ? a.v_scale / l : 0.f);
+}
+
+// seq_order[r] = the sequence with the r-th longest length (ties by index): one thread per sequence.
+__global__ __launch_bounds__(256) void rank_sequences_kernel(const int32_t* __restrict__ seq_lens, int batch,
+                                                             int32_t* __restrict__ seq_order) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= batch) return;
+  const int mine = seq_lens[j];
+  int rank = 0;
+  for (int k = 0; k < batch; ++k) {
+    const int other = seq_lens[k];
+    rank += (other > mine || (other == mine && k < j)) ? 1 : 0;
+  }
+  seq_order[rank] = j;
 }
 
 // out[b,h,:] = sum_p w_p * part_out[b,h,p,:] / sum_p w_p,  w_p = 2^(lse_p - max lse)
@@ -359,39 +493,100 @@ __global__ __launch_bounds__(256) void combine_partitions_kernel(void* out, cons
 #ifndef APS_HPW_FP8
 #define APS_HPW_FP8 2
 #endif
+// Tiles of 16 tokens a wavefront keeps in flight.  Measured at 128 sequences x 40 heads x 128, lognormal
+// lengths: 2, 3 and 4 run within 2 % of each other (the kernel is not short of bytes in flight), and 2 keeps
+// the register count low enough for four wavefronts per SIMD.
+#ifndef APS_DEPTH_F16
+#define APS_DEPTH_F16 2
+#endif
+#ifndef APS_DEPTH_FP8
+#define APS_DEPTH_FP8 2
+#endif
+
+// wavefronts (= partitions of a sequence) of a group-path workgroup; 16 would cap the kernel at 128 registers
+constexpr int kMaxGroupWaves = 8;
+
+// Path and scratch of a problem, shared by the launcher and the workspace query.
+struct DecodePlan {
+  int64_t np;          // partitions of the longest sequence
+  bool group;          // one workgroup per (head group, sequence), merge in LDS
+  int waves;           // group path: wavefronts per workgroup
+  bool sorted;         // group path: workgroup rows dealt out longest sequence first
+  bool order_scratch;  // the order comes from rank_sequences_kernel (int32 per sequence in the scratch)
+};
+
+inline DecodePlan plan_decode(int64_t batch, int num_heads, int64_t max_seq_len, int partition_size) {
+  DecodePlan p{};
+  p.np = (max_seq_len + partition_size - 1) / partition_size;
+  if (p.np < 1) p.np = 1;
+  p.group = p.np <= kMaxGroupWaves;
+  p.waves = 1;
+  while (p.waves < p.np) p.waves <<= 1;
+  // more than one round of resident wavefronts (256 compute units x 16): the order of the workgroups decides
+  // how long the last ones run alone
+  p.sorted = p.group && batch > 1 && batch * num_heads * p.np > 4096;
+  p.order_scratch = p.sorted && batch > kRankInKernelMax;
+  return p;
+}
+
+template <int QT, int KV, int D, int HPW, int DEPTH>
+void launch_group(const AttnArgs& a, int64_t batch, int waves, hipStream_t s) {
+  const dim3 grid((unsigned)(a.num_heads / HPW), (unsigned)batch);
+  switch (waves) {
+    case 1: hipLaunchKernelGGL((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 1>), grid, dim3(64), 0, s, a); break;
+    case 2: hipLaunchKernelGGL((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 2>), grid, dim3(128), 0, s, a); break;
+    case 4: hipLaunchKernelGGL((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 4>), grid, dim3(256), 0, s, a); break;
+    default: hipLaunchKernelGGL((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 8>), grid, dim3(512), 0, s, a); break;
+  }
+}
 
 // Heads per wavefront: adjacent heads of one token are contiguous in memory, so HPW heads per wave make
 // the contiguous piece a wave-wide load takes from one token row HPW times longer.
 template <int QT, int KV, int D>
-void launch_head_size(const AttnArgs& a, int64_t batch, hipStream_t s) {
+void launch_head_size(const AttnArgs& a, int64_t batch, const DecodePlan& plan, hipStream_t s) {
   constexpr int kWant = (KV == KV_FP8) ? APS_HPW_FP8 : APS_HPW_F16;
+  constexpr int DEPTH = (KV == KV_FP8) ? APS_DEPTH_FP8 : APS_DEPTH_F16;
   constexpr int LPT = D / Unpack<KV>::EPL;
   constexpr int HPW = (LPT * kWant <= 32) ? kWant : 1;
   if constexpr (HPW > 1) {
     if (a.num_heads % HPW == 0) {
-      const dim3 grid((unsigned)(a.num_heads / HPW), (unsigned)a.num_partitions, (unsigned)batch);
-      hipLaunchKernelGGL((paged_decode_kernel<QT, KV, D, HPW>), grid, dim3(64), 0, s, a);
+      if (plan.group) {
+        launch_group<QT, KV, D, HPW, DEPTH>(a, batch, plan.waves, s);
+      } else {
+        const dim3 grid((unsigned)(a.num_heads / HPW), (unsigned)a.num_partitions, (unsigned)batch);
+        hipLaunchKernelGGL((paged_decode_kernel<QT, KV, D, HPW, DEPTH>), grid, dim3(64), 0, s, a);
+      }
       return;
     }
   }
-  const dim3 grid((unsigned)a.num_heads, (unsigned)a.num_partitions, (unsigned)batch);
-  hipLaunchKernelGGL((paged_decode_kernel<QT, KV, D, 1>), grid, dim3(64), 0, s, a);
+  if (plan.group) {
+    launch_group<QT, KV, D, 1, DEPTH>(a, batch, plan.waves, s);
+  } else {
+    const dim3 grid((unsigned)a.num_heads, (unsigned)a.num_partitions, (unsigned)batch);
+    hipLaunchKernelGGL((paged_decode_kernel<QT, KV, D, 1, DEPTH>), grid, dim3(64), 0, s, a);
+  }
 }
 
 template <int QT, int KV>
-int launch_decode(const AttnArgs& a, int head_size, int64_t batch, hipStream_t s) {
+int launch_decode(const AttnArgs& a, int head_size, int64_t batch, const DecodePlan& plan, hipStream_t s) {
+  if (plan.order_scratch) {
+    hipLaunchKernelGGL(rank_sequences_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, a.seq_lens,
+                       (int)batch, const_cast<int32_t*>(a.seq_order));
+    const int st = launch_status();
+    if (st != APS_OK) return st;
+  }
   switch (head_size) {
-    case 64: launch_head_size<QT, KV, 64>(a, batch, s); break;
-    case 128: launch_head_size<QT, KV, 128>(a, batch, s); break;
-    case 256: launch_head_size<QT, KV, 256>(a, batch, s); break;
+    case 64: launch_head_size<QT, KV, 64>(a, batch, plan, s); break;
+    case 128: launch_head_size<QT, KV, 128>(a, batch, plan, s); break;
+    case 256: launch_head_size<QT, KV, 256>(a, batch, plan, s); break;
     case 32:
       if constexpr (KV == KV_FP8) return APS_ERR_UNSUPPORTED;
-      else launch_head_size<QT, KV, 32>(a, batch, s);
+      else launch_head_size<QT, KV, 32>(a, batch, plan, s);
       break;
     default: return APS_ERR_UNSUPPORTED;
   }
   int st = launch_status();
-  if (st != APS_OK || a.num_partitions == 1) return st;
+  if (st != APS_OK || plan.group || a.num_partitions == 1) return st;
   const int threads = head_size >= 256 ? 256 : (head_size + 63) / 64 * 64;
   hipLaunchKernelGGL((combine_partitions_kernel<QT>), dim3((unsigned)a.num_heads, (unsigned)batch), dim3(threads), 0,
                      s, a.out, a.part_out, a.part_lse, a.seq_lens, a.out_stride, a.num_heads, head_size,
@@ -411,19 +606,25 @@ extern "C" {
 int aps_decode_attention_partition_size(int64_t batch, int num_heads, int64_t max_seq_len, int block_size) {
   if (batch <= 0 || num_heads <= 0 || max_seq_len <= 0 || block_size <= 0) return 256;
   // Aim for a few thousand wavefronts (256 compute units x 8-16 resident waves);
-  // shorten the partitions of small batches, never below two tiles.
-  int64_t part = 256;
+  // shorten the partitions of small batches, never below two tiles.  512 tokens = at most four wavefronts per
+  // workgroup for sequences up to 2048: workgroups of four pack the 12 or 16 wave slots of a compute unit
+  // without a remainder (8-wavefront workgroups left a third of the slots empty with the fp8 kernel).
+  int64_t part = 512;
   while (part > 32 && batch * num_heads * ((max_seq_len + part - 1) / part) < 4096) part >>= 1;
   if (part % block_size != 0) part = (part + block_size - 1) / block_size * block_size;
+  // plenty of sequences: lengthen the partitions until a sequence fits the wavefronts of one workgroup (the
+  // partial results then merge in LDS), as far as the 64 block ids a wavefront holds allow
+  if (batch * num_heads >= 1024)
+    while ((max_seq_len + part - 1) / part > kMaxGroupWaves && 2 * part / block_size <= 64) part *= 2;
   return (int)part;
 }
 
 int64_t aps_decode_attention_workspace_bytes(int64_t batch, int num_heads, int head_size, int64_t max_seq_len,
                                              int partition_size) {
   if (batch <= 0 || num_heads <= 0 || head_size <= 0 || max_seq_len <= 0 || partition_size <= 0) return 0;
-  const int64_t np = (max_seq_len + partition_size - 1) / partition_size;
-  if (np <= 1) return 0;
-  const int64_t n = batch * num_heads * np;
+  const DecodePlan plan = plan_decode(batch, num_heads, max_seq_len, partition_size);
+  if (plan.group) return plan.order_scratch ? align_up(batch * 4, 256) : 0;
+  const int64_t n = batch * num_heads * plan.np;
   return align_up(n * head_size * 4, 256) + align_up(n * 4, 256);
 }
 
@@ -459,7 +660,8 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
   if (partition_size <= 0)
     partition_size = aps_decode_attention_partition_size(batch, num_heads, max_seq_len, block_size);
   if (partition_size % block_size != 0 || partition_size / block_size > 64) return APS_ERR_INVALID_ARG;
-  const int64_t np = (max_seq_len + partition_size - 1) / partition_size;
+  const DecodePlan plan = plan_decode(batch, num_heads, max_seq_len, partition_size);
+  const int64_t np = plan.np;
   if (np > 65535 || batch > 65535) return APS_ERR_UNSUPPORTED;
 
   AttnArgs a;
@@ -476,22 +678,28 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
   const float ks = kv_dtype == APS_FP8_E4M3 ? k_scale : 1.f;
   a.scale_log2 = softmax_scale * ks * kLog2e;
   a.v_scale = kv_dtype == APS_FP8_E4M3 ? v_scale : 1.f;
-  a.part_out = nullptr; a.part_lse = nullptr;
-  if (np > 1) {
-    const int64_t need = aps_decode_attention_workspace_bytes(batch, num_heads, head_size, max_seq_len, partition_size);
+  a.part_out = nullptr; a.part_lse = nullptr; a.seq_order = nullptr;
+  a.batch = (int)batch;
+  a.rank_in_kernel = plan.sorted && !plan.order_scratch;
+  const int64_t need = aps_decode_attention_workspace_bytes(batch, num_heads, head_size, max_seq_len, partition_size);
+  if (need > 0) {
     if (workspace && workspace_bytes < need) return too_small_status;
     if (!workspace || (addr(workspace) & 15)) return APS_ERR_WORKSPACE;
-    const int64_t n = batch * num_heads * np;
-    a.part_out = (float*)workspace;
-    a.part_lse = (float*)((char*)workspace + align_up(n * head_size * 4, 256));
+    if (plan.group) {
+      a.seq_order = (const int32_t*)workspace;
+    } else {
+      const int64_t n = batch * num_heads * np;
+      a.part_out = (float*)workspace;
+      a.part_lse = (float*)((char*)workspace + align_up(n * head_size * 4, 256));
+    }
   }
   hipStream_t s = (hipStream_t)stream;
   if (q_dtype == APS_F16) {
-    return kv_dtype == APS_FP8_E4M3 ? launch_decode<APS_F16, KV_FP8>(a, head_size, batch, s)
-                                    : launch_decode<APS_F16, KV_F16>(a, head_size, batch, s);
+    return kv_dtype == APS_FP8_E4M3 ? launch_decode<APS_F16, KV_FP8>(a, head_size, batch, plan, s)
+                                    : launch_decode<APS_F16, KV_F16>(a, head_size, batch, plan, s);
   }
-  return kv_dtype == APS_FP8_E4M3 ? launch_decode<APS_BF16, KV_FP8>(a, head_size, batch, s)
-                                  : launch_decode<APS_BF16, KV_BF16>(a, head_size, batch, s);
+  return kv_dtype == APS_FP8_E4M3 ? launch_decode<APS_BF16, KV_FP8>(a, head_size, batch, plan, s)
+                                  : launch_decode<APS_BF16, KV_BF16>(a, head_size, batch, plan, s);
 }
 
 int aps_paged_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,

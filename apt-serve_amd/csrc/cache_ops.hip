@@ -22,27 +22,49 @@ struct RowDesc {
   char* dst;        // nullptr: skip the row
 };
 
-// One thread moves one VB-byte chunk: chunk g of the launch belongs to row
-// g / cpr (cpr = chunks per row).  Measured on MI355X this flat shape streams
-// faster than workgroups that loop over whole rows (6.4 vs 5.3-6.0 TB/s for
-// 10 KiB rows): every lane is busy, consecutive lanes touch consecutive 16-byte
-// chunks even across row boundaries, and the many small workgroups spread
-// evenly over the memory channels.  grid.y splits the rows into groups small
-// enough for 32-bit chunk arithmetic.
-template <int VB, class Op>
-__global__ __launch_bounds__(kMaxThreads) void row_mover(Op op, int64_t n_items, uint32_t cpr, uint32_t row_bytes,
-                                                         uint32_t items_per_y) {
+// A segment is one wave-wide access: 64 consecutive VB-byte chunks of one row.  A wavefront owns U consecutive
+// segments (of one row, or of two when U does not divide the segments per row): it resolves the U row
+// descriptors first (their index loads are independent and go out together), then issues its U loads, then its
+// U stores.  With one chunk per thread a compute unit has at most 32 wavefronts x 1 KiB of loads in flight,
+// which at this part's memory latency is about 3 TB/s of reads however many workgroups are queued; U chunks
+// per thread put U times as much in flight for the same number of resident wavefronts.  Loads and stores stay
+// fully coalesced (a 10 KiB row of OPT-13B is ten 1 KiB segments) and non-temporal.  grid.y splits the rows
+// into groups small enough for 32-bit segment arithmetic.
+// Measured on MI355X (OPT-13B rows, random fp16 data): operators with one index level run fastest with U = 1
+// (292 us for the config-2 gather against 299 / 317 us with U = 2 / 4: the chain index -> data is short enough
+// for the 32 resident wavefronts of a compute unit to hide), the ones with two dependent index levels with
+// U = 2 (312 against 341 us).  Each operator names its U as kChunks.
+
+template <int VB, int U, class Op>
+__global__ __launch_bounds__(kMaxThreads) void row_mover(Op op, int64_t n_items, uint32_t segs_per_row,
+                                                         uint32_t row_bytes, uint32_t items_per_y) {
   typedef typename VecOf<VB>::type vec_t;
-  const uint32_t g = blockIdx.x * kMaxThreads + threadIdx.x;
-  const uint32_t local_item = g / cpr;
-  const uint32_t c = (g - local_item * cpr) * VB;
-  const int64_t item = (int64_t)blockIdx.y * items_per_y + local_item;
-  if (local_item >= items_per_y || item >= n_items || c >= row_bytes) return;
-  const RowDesc rd = op(item);
-  if (rd.dst == nullptr) return;
-  vec_t v = vec_t{};
-  if (rd.src != nullptr) v = load_vec_stream<VB>(rd.src + c);
-  store_vec_stream<VB>(rd.dst + c, v);
+  const uint32_t lane = threadIdx.x & 63u;
+  // wave-uniform on purpose: the row of a segment, its index loads and its pointers are then scalar work
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * (kMaxThreads / 64) + (threadIdx.x >> 6));
+  uint32_t local_item = (wave * U) / segs_per_row;
+  uint32_t seg = wave * U - local_item * segs_per_row;
+  const int64_t item0 = (int64_t)blockIdx.y * items_per_y;
+  RowDesc rd[U];
+  uint32_t c[U];
+#pragma unroll
+  for (int j = 0; j < U; ++j) {
+    c[j] = (seg * 64u + lane) * VB;
+    const int64_t item = item0 + local_item;
+    rd[j] = RowDesc{nullptr, nullptr};
+    if (local_item < items_per_y && item < n_items) rd[j] = op(item);
+    if (c[j] >= row_bytes) rd[j].dst = nullptr;
+    if (++seg == segs_per_row) { seg = 0; ++local_item; }
+  }
+  vec_t v[U];
+#pragma unroll
+  for (int j = 0; j < U; ++j) {
+    v[j] = vec_t{};
+    if (rd[j].dst != nullptr && rd[j].src != nullptr) v[j] = load_vec_stream<VB>(rd[j].src + c[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < U; ++j)
+    if (rd[j].dst != nullptr) store_vec_stream<VB>(rd[j].dst + c[j], v[j]);
 }
 
 // ---------------------------------------------------------------- descriptors
@@ -67,6 +89,7 @@ struct BlockSplit {
 };
 
 struct HiddenToCacheOp {
+  static constexpr int kChunks = 2;
   const char* hidden; char* cache;
   const int64_t* slot_mapping; const int64_t* src_idx; const int64_t* tgt_idx;
   int64_t hidden_stride_b, slot_stride_b, num_slots, num_hidden_rows, slot_mapping_len;
@@ -84,6 +107,7 @@ struct HiddenToCacheOp {
 };
 
 struct CacheToHiddenOp {
+  static constexpr int kChunks = 2;
   char* hidden; const char* cache;
   const int64_t* slot_mapping; const int64_t* dst_idx;
   int64_t hidden_stride_b, slot_stride_b, num_slots, num_hidden_rows, slot_mapping_len;
@@ -100,6 +124,7 @@ struct CacheToHiddenOp {
 };
 
 struct HybridDecodeGatherOp {
+  static constexpr int kChunks = 2;
   char* holder; const char* hidden_states; char* cache;
   const int64_t* slot_mapping; const int64_t* upd; const int64_t* pull;
   const int64_t* use_input; const int64_t* store_tot;
@@ -137,6 +162,7 @@ struct HybridDecodeGatherOp {
 // below -num_inputs is a padding row (zero filled).  One dependent index load
 // per chunk instead of two: 6.4 instead of 5.6 TB/s on MI355X for 10 KiB rows.
 struct ResolvedGatherOp {
+  static constexpr int kChunks = 1;
   char* holder; const char* hidden_states; char* cache;
   const int64_t* row_src; const int64_t* slot_mapping;
   const int64_t* use_input; const int64_t* store_tot;
@@ -168,6 +194,7 @@ struct ResolvedGatherOp {
 
 // item = 2*t + plane (0 = K, 1 = V)
 struct KvScatterOp {
+  static constexpr int kChunks = 1;
   const char* key; const char* value; char* k_cache; char* v_cache;
   const int64_t* slot_mapping; const int64_t* token_idx;
   int64_t num_tokens, key_stride_b, value_stride_b, block_stride_b, row_b, num_blocks;
@@ -193,6 +220,7 @@ struct KvScatterOp {
 // and V row (plane 1) by block; a hidden token stores its hidden row (plane 0 only) at its slot of the
 // flattened cache.  A null source pointer switches that kind of row off.
 struct MixedTokenOp {
+  static constexpr int kChunks = 1;
   const char* key; const char* value; const char* hidden;
   char* k_cache; char* v_cache; char* hidden_cache;
   const int64_t* slot_mapping; const uint8_t* is_hidden;
@@ -225,6 +253,7 @@ struct MixedTokenOp {
 // A K/V block (kind 0) is both planes of block id b < N; a hidden block (kind 1) is one plane slab, its id
 // runs over the flattened 2N plane slabs (b < N: K plane of block b, b >= N: V plane of block b - N).
 struct BlockCopyOp {
+  static constexpr int kChunks = 1;
   const int64_t* layer_base;   // device array: base address of every layer's (2, N, BS, H, D) cache
   const int64_t* pairs;        // [n][2] (source, destination)
   const uint8_t* kinds;        // nullable: all K/V blocks
@@ -259,6 +288,7 @@ struct BlockCopyOp {
 
 // item = 2*blk + plane over the reference's grid of 2*nkv + nh blocks
 struct MixedKvOp {
+  static constexpr int kChunks = 2;
   const char* key; const char* value;
   char* k_cache; char* v_cache; char* sk_cache; char* sv_cache;
   const int64_t* slot_mapping; const int64_t* slot_mapping_shared;
@@ -305,14 +335,16 @@ struct MixedKvOp {
 
 template <int VB, class Op>
 int launch_rows_vb(const Op& op, int64_t n_items, int64_t row_bytes, hipStream_t s) {
-  const int64_t cpr = (row_bytes + VB - 1) / VB;
-  int64_t items_per_y = ((int64_t)1 << 30) / cpr;
+  constexpr int U = VB == 16 ? Op::kChunks : 1;
+  const int64_t segs_per_row = (row_bytes + 64 * VB - 1) / (64 * VB);
+  int64_t items_per_y = ((int64_t)1 << 30) / (segs_per_row * 64);
   if (items_per_y > n_items) items_per_y = n_items;
   const int64_t grid_y = (n_items + items_per_y - 1) / items_per_y;
   if (grid_y > 65535) return APS_ERR_UNSUPPORTED;
-  const int64_t grid_x = (items_per_y * cpr + kMaxThreads - 1) / kMaxThreads;
-  hipLaunchKernelGGL((row_mover<VB, Op>), dim3((unsigned)grid_x, (unsigned)grid_y), dim3(kMaxThreads), 0, s, op,
-                     n_items, (uint32_t)cpr, (uint32_t)row_bytes, (uint32_t)items_per_y);
+  const int64_t waves = (items_per_y * segs_per_row + U - 1) / U;
+  const int64_t grid_x = (waves + kMaxThreads / 64 - 1) / (kMaxThreads / 64);
+  hipLaunchKernelGGL((row_mover<VB, U, Op>), dim3((unsigned)grid_x, (unsigned)grid_y), dim3(kMaxThreads), 0, s, op,
+                     n_items, (uint32_t)segs_per_row, (uint32_t)row_bytes, (uint32_t)items_per_y);
   return launch_status();
 }
 
@@ -455,12 +487,50 @@ int dispatch_kv_scatter_fp8(const void* key, const void* value, void* key_cache,
   }
 }
 
+// Plain streams in the shape of the row movers: a workgroup owns 256 * U consecutive 16-byte chunks and every
+// thread moves U of them (all loads, then all stores); no loop, workgroups are dispatched in address order.
+template <int U>
 __global__ __launch_bounds__(kMaxThreads) void copy_bytes_kernel(VecOf<16>::type* __restrict__ dst,
                                                                   const VecOf<16>::type* __restrict__ src,
                                                                   int64_t n_vec) {
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec; i += stride) {
-    __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+  const int64_t base = (int64_t)blockIdx.x * (kMaxThreads * U) + threadIdx.x;
+  VecOf<16>::type v[U];
+#pragma unroll
+  for (int j = 0; j < U; ++j)
+    if (base + j * kMaxThreads < n_vec) v[j] = __builtin_nontemporal_load(src + base + j * kMaxThreads);
+#pragma unroll
+  for (int j = 0; j < U; ++j)
+    if (base + j * kMaxThreads < n_vec) __builtin_nontemporal_store(v[j], dst + base + j * kMaxThreads);
+}
+
+template <int U>
+__global__ __launch_bounds__(kMaxThreads) void read_bytes_kernel(uint32_t* __restrict__ sink,
+                                                                  const VecOf<16>::type* __restrict__ src,
+                                                                  int64_t n_vec) {
+  const int64_t base = (int64_t)blockIdx.x * (kMaxThreads * U) + threadIdx.x;
+  uint32_t x = 0;
+  VecOf<16>::type v[U];
+#pragma unroll
+  for (int j = 0; j < U; ++j) {
+    v[j] = VecOf<16>::type{0u, 0u, 0u, 0u};
+    if (base + j * kMaxThreads < n_vec) v[j] = __builtin_nontemporal_load(src + base + j * kMaxThreads);
+  }
+#pragma unroll
+  for (int j = 0; j < U; ++j) x ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+  if (x == 0x9e3779b9u && sink) *sink = x;  // keeps the loads alive; practically never taken
+}
+
+template <int U>
+__global__ __launch_bounds__(kMaxThreads) void fill_bytes_kernel(VecOf<16>::type* __restrict__ dst, int64_t n_vec,
+                                                                  uint32_t seed) {
+  const int64_t base = (int64_t)blockIdx.x * (kMaxThreads * U) + threadIdx.x;
+#pragma unroll
+  for (int j = 0; j < U; ++j) {
+    const int64_t i = base + j * kMaxThreads;
+    // not a constant pattern: what the memory sustains depends on the data
+    const uint32_t h = ((uint32_t)i * 2654435761u) ^ seed;
+    const VecOf<16>::type v = {h, h * 0x85ebca6bu, h ^ 0xc2b2ae35u, h * 0x27d4eb2fu};
+    if (i < n_vec) __builtin_nontemporal_store(v, dst + i);
   }
 }
 
@@ -719,15 +789,33 @@ int aps_swap_cache_blocks(const void* src_cache, void* dst_cache, const int64_t*
 }
 
 int aps_copy_bytes(void* dst, const void* src, int64_t nbytes, aps_stream_t stream) {
-  if (nbytes < 0) return APS_ERR_INVALID_ARG;
+  return aps_stream_probe(0, 1, dst, src, nbytes, stream);
+}
+
+int aps_stream_probe(int mode, int chunks_per_thread, void* dst, const void* src, int64_t nbytes,
+                     aps_stream_t stream) {
+  if (nbytes < 0 || mode < 0 || mode > 2) return APS_ERR_INVALID_ARG;
+  if (chunks_per_thread != 1 && chunks_per_thread != 4) return APS_ERR_INVALID_ARG;
   if (nbytes == 0) return APS_OK;
-  if (!dst || !src) return APS_ERR_INVALID_ARG;
-  if (common_vec_bytes({addr(dst), addr(src), (uint64_t)nbytes}) != 16) return APS_ERR_UNSUPPORTED;
+  if ((mode != 2 && !src) || !dst) return APS_ERR_INVALID_ARG;
+  if (common_vec_bytes({mode == 1 ? 0 : addr(dst), addr(src), (uint64_t)nbytes}) != 16) return APS_ERR_UNSUPPORTED;
   const int64_t n_vec = nbytes / 16;
-  int64_t grid = (n_vec + kMaxThreads * 4 - 1) / (kMaxThreads * 4);
-  if (grid > 256 * 64) grid = 256 * 64;
-  hipLaunchKernelGGL(copy_bytes_kernel, dim3((unsigned)grid), dim3(kMaxThreads), 0, (hipStream_t)stream,
-                     (VecOf<16>::type*)dst, (const VecOf<16>::type*)src, n_vec);
+  const int64_t per_block = (int64_t)kMaxThreads * chunks_per_thread;
+  const int64_t grid = (n_vec + per_block - 1) / per_block;
+  if (grid >= (int64_t)1 << 31) return APS_ERR_UNSUPPORTED;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 g((unsigned)grid), b(kMaxThreads);
+  VecOf<16>::type* d = (VecOf<16>::type*)dst;
+  const VecOf<16>::type* sp = (const VecOf<16>::type*)src;
+  if (chunks_per_thread == 1) {
+    if (mode == 0) hipLaunchKernelGGL(copy_bytes_kernel<1>, g, b, 0, s, d, sp, n_vec);
+    else if (mode == 1) hipLaunchKernelGGL(read_bytes_kernel<1>, g, b, 0, s, (uint32_t*)dst, sp, n_vec);
+    else hipLaunchKernelGGL(fill_bytes_kernel<1>, g, b, 0, s, d, n_vec, 0x3c003c00u);
+  } else {
+    if (mode == 0) hipLaunchKernelGGL(copy_bytes_kernel<4>, g, b, 0, s, d, sp, n_vec);
+    else if (mode == 1) hipLaunchKernelGGL(read_bytes_kernel<4>, g, b, 0, s, (uint32_t*)dst, sp, n_vec);
+    else hipLaunchKernelGGL(fill_bytes_kernel<4>, g, b, 0, s, d, n_vec, 0x3c003c00u);
+  }
   return launch_status();
 }
 

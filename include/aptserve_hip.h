@@ -474,6 +474,15 @@ int aps_swap_cache_blocks(const void* src_cache, void* dst_cache,
 int aps_copy_bytes(void* dst, const void* src, int64_t nbytes,
                    aps_stream_t stream);
 
+/* Plain streams over nbytes (16-byte aligned), for measuring what the part
+ * sustains: mode 0 copies src to dst (as aps_copy_bytes), mode 1 only reads
+ * src (dst: 4 bytes that are practically never written), mode 2 only writes
+ * dst with a non-constant pattern (src unused).  chunks_per_thread 1 or 4
+ * 16-byte chunks in flight per thread.  The ceilings the row movers and the
+ * attention are compared against come from these. */
+int aps_stream_probe(int mode, int chunks_per_thread, void* dst,
+                     const void* src, int64_t nbytes, aps_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

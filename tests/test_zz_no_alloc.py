@@ -28,8 +28,23 @@ def _both(c, dev, partition_size, **kw):
 def test_static_scratch_matches_workspace_entry_on_two_calls_in_a_row(dev):
     big = make_case(6, 8, 128, 16, [2048, 700, 1, 257, 1500, 31], 21, hybrid=True)
     small = make_case(3, 8, 128, 16, [300, 40, 129], 22, hybrid=True)
-    for case, ps in ((big, 256), (small, 64), (big, 0)):
+    # partition sizes that split a sequence into more partitions than a workgroup has wavefronts: the partial
+    # results go through the scratch; (big, 256) merges in LDS and touches no scratch
+    for case, ps in ((big, 64), (small, 16), (big, 256), (big, 32)):
         out, ref = _both(case, dev, ps)
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
+def test_static_scratch_holds_the_sequence_order_of_a_large_batch(dev):
+    """More than 512 sequences: the longest-first order of the workgroups is computed by a kernel into the
+    scratch.  Second call: fewer sequences (ranked inside the attention kernel, no scratch)."""
+    rng = np.random.default_rng(5)
+    lib = _lib.load()
+    for B in (600, 40):
+        lens = [int(x) for x in rng.integers(1, 65, B)]
+        c = make_case(B, 8, 64, 16, lens, 24)
+        assert (lib.aps_decode_attention_workspace_bytes(B, 8, 64, max(lens), 256) > 0) == (B > 512)
+        out, ref = _both(c, dev, 256)
         assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
 
 
@@ -46,7 +61,7 @@ def test_static_scratch_fp8_and_single_partition(dev):
 def test_static_scratch_rejects_a_problem_beyond_its_limit(dev):
     lib = _lib.load()
     B, H, D, BS, W = 512, 40, 128, 16, 128
-    need = lib.aps_decode_attention_workspace_bytes(B, H, D, W * BS, 256)
+    need = lib.aps_decode_attention_workspace_bytes(B, H, D, W * BS, 64)
     assert need > 32 * 1024 * 1024
     q = torch.zeros(B, H, D, dtype=torch.float16, device=dev)
     kc = torch.zeros(4, BS, H, D, dtype=torch.float16, device=dev)
@@ -54,7 +69,7 @@ def test_static_scratch_rejects_a_problem_beyond_its_limit(dev):
     sl = torch.ones(B, dtype=torch.int32, device=dev)
     out = torch.empty_like(q)
     with pytest.raises(RuntimeError, match="static array"):
-        ops.paged_decode_attention(q, kc, kc, bt, sl, partition_size=256, out=out, static_scratch=True)
+        ops.paged_decode_attention(q, kc, kc, bt, sl, partition_size=64, out=out, static_scratch=True)
     # the same problem with a caller workspace is fine
-    ops.paged_decode_attention(q, kc, kc, bt, sl, partition_size=256, out=out)
+    ops.paged_decode_attention(q, kc, kc, bt, sl, partition_size=64, out=out)
     torch.cuda.synchronize()
