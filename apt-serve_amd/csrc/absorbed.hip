@@ -623,8 +623,7 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     hipError_t e = hipSuccess;
 #define APS_LAUNCH_SCORES(B, N)                                                                                   \
   do {                                                                                                            \
-    e = hipFuncSetAttribute((const void*)hidden_scores_kernel<B, N>, hipFuncAttributeMaxDynamicSharedMemorySize,  \
-                            scores_lds_bytes<N>());                                                               \
+    e = allow_dynamic_lds((const void*)hidden_scores_kernel<B, N>, scores_lds_bytes<N>(), (B ? 6 : 0) + N - 1);   \
     if (e == hipSuccess)                                                                                          \
       hipLaunchKernelGGL((hidden_scores_kernel<B, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g);      \
   } while (0)
@@ -710,8 +709,7 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     hipError_t e = hipSuccess;
 #define APS_LAUNCH_PROJ(B, N)                                                                                    \
   do {                                                                                                           \
-    e = hipFuncSetAttribute((const void*)head_proj_kernel<B, N>, hipFuncAttributeMaxDynamicSharedMemorySize,     \
-                            scores_lds_bytes<N>());                                                              \
+    e = allow_dynamic_lds((const void*)head_proj_kernel<B, N>, scores_lds_bytes<N>(), 12 + (B ? 2 : 0) + N - 2); \
     if (e == hipSuccess)                                                                                         \
       hipLaunchKernelGGL((head_proj_kernel<B, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g);         \
   } while (0)

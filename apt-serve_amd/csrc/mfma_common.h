@@ -1,6 +1,8 @@
 // Shared pieces of the matrix-core kernels (gfx950): operand vector types, MFMA wrappers,
 // buffer descriptors, rounding to the 16-bit output types, hand-placed wait points.
 #pragma once
+#include <atomic>
+
 #include "aps_common.h"
 
 namespace aps {
@@ -55,6 +57,20 @@ template <bool BF16>
 __device__ __forceinline__ float load_16bit_as_f32(const void* p, int64_t i) {
   const uint16_t v = ((const uint16_t*)p)[i];
   return BF16 ? __uint_as_float((uint32_t)v << 16) : (float)__builtin_bit_cast(_Float16, v);
+}
+
+// More than 64 KiB of dynamic LDS has to be allowed per function and device: done once per (kernel, device)
+// instead of on every launch.  `slot` numbers the kernel instantiations of one source file that need it.
+inline hipError_t allow_dynamic_lds(const void* fn, int bytes, int slot) {
+  static std::atomic<uint64_t> done[16];
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = device >= 0 && device < 64 ? (uint64_t)1 << device : 0;
+  if (bit && (done[slot].load(std::memory_order_relaxed) & bit)) return hipSuccess;
+  e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && bit) done[slot].fetch_or(bit, std::memory_order_relaxed);
+  return e;
 }
 
 }  // namespace

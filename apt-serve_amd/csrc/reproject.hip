@@ -109,7 +109,23 @@ struct GemmArgs {
   // partial tile to partial[z][m][n]; a second kernel adds the splits and the bias
   float* partial;
   int kt_per_split;
+  // tail split (large M): logical tiles from tail_from on are cut into tail_ways parts of tail_kt k-tiles each;
+  // part p of tail tile i stores its fp32 result tile at tail_partial[(i * tail_ways + p)][256][256]
+  float* tail_partial;
+  int tail_from, tail_ways, tail_kt;
 };
+
+// Logical tile number -> tile coordinates: groups of kGroupM tile rows, column-major inside a group, so that
+// consecutive logical tiles share their A and W panels.
+__host__ __device__ __forceinline__ void tile_coords(int logical, int tiles_m, int tiles_n, int& pid_m, int& pid_n) {
+  const int in_group = kGroupM * tiles_n;
+  const int group = logical / in_group;
+  const int first_m = group * kGroupM;
+  const int gsz = (tiles_m - first_m) < kGroupM ? (tiles_m - first_m) : kGroupM;
+  const int r = logical - group * in_group;
+  pid_m = first_m + r % gsz;
+  pid_n = r / gsz;
+}
 
 template <bool BF16, int MI>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_nt_kernel(
@@ -122,21 +138,33 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int wm = wave >> 2, wn = wave & 3;
 
-  // ---- tile assignment: XCD-contiguous, grouped 8 tiles along M
-  int pid_m, pid_n;
+  // ---- tile assignment: XCD-contiguous, grouped 8 tiles along M.  Workgroups go to the XCDs round-robin by
+  // their linear id, so XCD x gets the ids x, x+8, ...: it is given a contiguous run of logical tiles (and, with
+  // a tail split, a contiguous run of the tail parts, which come last).
+  int pid_m, pid_n, tail_part = -1, tail_slot = 0;
   {
     const int total = g.tiles_m * g.tiles_n;
-    const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
     const int w = blockIdx.x;
-    const int logical = (w % kNumXcd) * per_xcd + w / kNumXcd;
-    if (logical >= total) return;
-    const int in_group = kGroupM * g.tiles_n;
-    const int group = logical / in_group;
-    const int first_m = group * kGroupM;
-    const int gsz = min(g.tiles_m - first_m, kGroupM);
-    const int r = logical - group * in_group;
-    pid_m = first_m + r % gsz;
-    pid_n = r / gsz;
+    const int xcd = w % kNumXcd, idx = w / kNumXcd;
+    int logical;
+    if (g.tail_ways > 1) {
+      const int full_per_xcd = g.tail_from / kNumXcd;  // tail_from is a multiple of the CU count
+      const int tail_items = (total - g.tail_from) * g.tail_ways;
+      const int tail_per_xcd = (tail_items + kNumXcd - 1) / kNumXcd;
+      if (idx < full_per_xcd) {
+        logical = xcd * full_per_xcd + idx;
+      } else {
+        tail_slot = xcd * tail_per_xcd + (idx - full_per_xcd);
+        if (idx - full_per_xcd >= tail_per_xcd || tail_slot >= tail_items) return;
+        logical = g.tail_from + tail_slot / g.tail_ways;
+        tail_part = tail_slot % g.tail_ways;
+      }
+    } else {
+      const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
+      logical = xcd * per_xcd + idx;
+      if (logical >= total) return;
+    }
+    tile_coords(logical, g.tiles_m, g.tiles_n, pid_m, pid_n);
   }
 
   // ---- global -> LDS DMA addressing
@@ -151,7 +179,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   const uint32_t voff_w0 = (uint32_t)(lrow * g.ldw_b + lchunk0 * 16), voff_w1 = (uint32_t)(lrow * g.ldw_b + lchunk1 * 16);
   const uint32_t grp_a = (uint32_t)(8 * g.lda_b), grp_w = (uint32_t)(8 * g.ldw_b);
 
-  const int kt_base_ = g.partial ? (int)blockIdx.y * g.kt_per_split : 0;
+  const int kt_base_ = tail_part >= 0 ? tail_part * g.tail_kt : (g.partial ? (int)blockIdx.y * g.kt_per_split : 0);
   auto issue_loads = [&](int kt) {
     char* sa = lds + (kt & 1) * kStageBytes;
     char* sw = sa + kTileBytes;
@@ -211,8 +239,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   };
 
   const int nk_total = (int)(g.k / BK);
-  const int kt_base = g.partial ? blockIdx.y * g.kt_per_split : 0;
-  const int nk = g.partial ? min(g.kt_per_split, nk_total - kt_base) : nk_total;
+  const int kt_base = kt_base_;
+  const int nk = tail_part >= 0 ? min(g.tail_kt, nk_total - kt_base)
+                                : (g.partial ? min(g.kt_per_split, nk_total - kt_base) : nk_total);
   u32x4 a0[MI], w0[2], a1[MI], w1[2];
   issue_loads(0);
   if (nk > 1) {
@@ -251,6 +280,21 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   // Lane l of a 32x32 result tile holds column l%32 and rows 8*(e/4) + 4*(l/32) + e%4, e = 0..15.
   // Each wave owns a [32*MI rows][64 cols] fp16 image (row pitch 144 B).  Neighbouring lanes swap one value
   // so that every lane writes a 32-bit pair; the image is then read back 16 bytes per lane, 8 lanes per row.
+  if (tail_part >= 0) {  // part of a tail tile: raw fp32 sums into its own [TBM][256] image
+    float* pz = g.tail_partial + (int64_t)tail_slot * (TBM * BN);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = wn * WN + j * 32 + frow;
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = wm * WM + i * 32 + 8 * (e >> 2) + 4 * fhalf + (e & 3);
+          pz[row * BN + col] = acc[i][j][e];
+        }
+    }
+    return;
+  }
   if (g.partial) {  // split-K: raw fp32 partial sums, lanes of a half-wave write 128 contiguous bytes
     float* pz = g.partial + (int64_t)blockIdx.y * g.m * g.n;
 #pragma unroll
@@ -665,8 +709,7 @@ int launch_weight_stream(const GemmArgs& g, int parts, int64_t k_per_part, hipSt
   hipError_t e = hipSuccess;
 #define APS_LAUNCH_WS(N)                                                                                          \
   do {                                                                                                            \
-    e = hipFuncSetAttribute((const void*)weight_stream_kernel<BF16, N>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            scores_lds_bytes<N>());                                                               \
+    e = allow_dynamic_lds((const void*)weight_stream_kernel<BF16, N>, scores_lds_bytes<N>(), 8 + (BF16 ? 3 : 0) + N - 1); \
     if (e == hipSuccess)                                                                                          \
       hipLaunchKernelGGL((weight_stream_kernel<BF16, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g,    \
                          k_per_part);                                                                             \
@@ -715,6 +758,57 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   else { o[0] = f32_to_f16_bits(s.x); o[1] = f32_to_f16_bits(s.y); o[2] = f32_to_f16_bits(s.z); o[3] = f32_to_f16_bits(s.w); }
 }
 
+// Tail tiles of a large product: out tile = sum of its parts + bias, rounded once.  One thread per 4 columns of a
+// row of a tile; 64 workgroups of 256 threads per 256 x 256 tile.
+template <bool BF16>
+__global__ __launch_bounds__(256) void tail_reduce_kernel(const GemmArgs g) {
+  const int tile = blockIdx.x >> 6;  // index among the tail tiles
+  const int q = ((blockIdx.x & 63) << 8) + threadIdx.x;  // quad of the tile: row q / 64, columns 4 * (q % 64)
+  const int r = q >> 6, c = (q & 63) << 2;
+  int pid_m, pid_n;
+  tile_coords(g.tail_from + tile, g.tiles_m, g.tiles_n, pid_m, pid_n);
+  const int64_t row = (int64_t)pid_m * BM + r, col = (int64_t)pid_n * BN + c;
+  if (row >= g.m) return;
+  const float* p = g.tail_partial + (int64_t)tile * g.tail_ways * (BM * BN) + r * BN + c;
+  float4 s = *(const float4*)p;
+  for (int z = 1; z < g.tail_ways; ++z) {
+    const float4 t = *(const float4*)(p + (int64_t)z * (BM * BN));
+    s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+  }
+  if (g.bias) {
+    s.x += load_16bit_as_f32<BF16>(g.bias, col); s.y += load_16bit_as_f32<BF16>(g.bias, col + 1);
+    s.z += load_16bit_as_f32<BF16>(g.bias, col + 2); s.w += load_16bit_as_f32<BF16>(g.bias, col + 3);
+  }
+  const int half = (g.out.n_split && col >= g.out.n_split) ? 1 : 0;
+  uint16_t* o = out_row(g.out, row, half);
+  if (!o) return;
+  o += col - (half ? g.out.n_split : 0);
+  const uint32_t lo = BF16 ? (f32_to_bf16_bits(s.x) | ((uint32_t)f32_to_bf16_bits(s.y) << 16))
+                           : (f32_to_f16_bits(s.x) | ((uint32_t)f32_to_f16_bits(s.y) << 16));
+  const uint32_t hi = BF16 ? (f32_to_bf16_bits(s.z) | ((uint32_t)f32_to_bf16_bits(s.w) << 16))
+                           : (f32_to_f16_bits(s.z) | ((uint32_t)f32_to_f16_bits(s.w) << 16));
+  ((uint32_t*)o)[0] = lo;   // rows and column offsets are at least 4-byte aligned (checked by the entry points)
+  ((uint32_t*)o)[1] = hi;
+}
+
+// Tail split of a product of full-size tiles: when the tiles fill the compute units a whole number of times
+// plus a remainder of at most half a round, the remaining tiles are cut along K into `ways` parts so that
+// their parts fill one short round instead of leaving most compute units idle for a full one (4096 x 10240:
+// 640 tiles on 256 compute units = 2.5 rounds run as 3; with the last 128 tiles cut in two, as 2.5).
+struct TailPlan { int from, ways, kt; int64_t bytes; };
+inline TailPlan plan_tail(int64_t tiles, int64_t nk) {
+  TailPlan t{0, 1, 0, 0};
+  const int64_t full = tiles / kNumCus * kNumCus, rest = tiles - full;
+  if (full == 0 || rest == 0 || tiles >= ((int64_t)1 << 28)) return t;
+  int ways = (int)(kNumCus / rest);
+  if (ways > 4) ways = 4;
+  while (ways > 1 && nk / ways < 8) --ways;
+  if (ways < 2) return t;
+  t.from = (int)full; t.ways = ways; t.kt = (int)((nk + ways - 1) / ways);
+  t.bytes = rest * ways * (int64_t)(BM * BN) * 4;
+  return t;
+}
+
 }  // namespace
 }  // namespace aps
 
@@ -754,9 +848,18 @@ int aps_linear_nt_splits(int64_t m, int64_t n, int64_t k) {
   return (int)(s < 1 ? 1 : s);
 }
 
+// Tail plan of a product, or none: only full-size tiles without a uniform K split are cut.
+static TailPlan tail_plan_of(int64_t m, int64_t n, int64_t k) {
+  if (m <= kWsMaxRows || n <= 0 || k <= 0 || n % BN != 0 || k % BK != 0 || tile_mi(m, n) != 4 ||
+      aps_linear_nt_splits(m, n, k) > 1)
+    return TailPlan{0, 1, 0, 0};
+  return plan_tail(((m + BM - 1) / BM) * (n / BN), k / BK);
+}
+
 int64_t aps_linear_nt_workspace_bytes(int64_t m, int64_t n, int64_t k) {
   const int s = aps_linear_nt_splits(m, n, k);
-  return s > 1 ? (int64_t)s * m * n * 4 : 0;
+  if (s > 1) return (int64_t)s * m * n * 4;
+  return tail_plan_of(m, n, k).bytes;
 }
 
 static int launch_gemm(const void* x, const void* weight, const void* bias, const OutMap& om, int64_t m, int64_t n,
@@ -824,13 +927,23 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   g.partial = splits > 1 ? (float*)workspace : nullptr;
   g.kt_per_split = (int)((nk_all + splits - 1) / splits);
   if (splits > 1) splits = (int)((nk_all + g.kt_per_split - 1) / g.kt_per_split);  // no empty split
-  const dim3 grid((unsigned)(per_xcd * kNumXcd), (unsigned)splits);
+  dim3 grid((unsigned)(per_xcd * kNumXcd), (unsigned)splits);
+  g.tail_ways = 1;
+  if (workspace && splits == 1) {
+    const TailPlan tp = tail_plan_of(m, n, k);
+    if (tp.ways > 1) {
+      if (workspace_bytes < tp.bytes || (addr(workspace) & 15)) return APS_ERR_WORKSPACE;
+      g.tail_partial = (float*)workspace;
+      g.tail_from = tp.from; g.tail_ways = tp.ways; g.tail_kt = tp.kt;
+      const int64_t tail_items = (total - tp.from) * tp.ways;
+      grid.x = (unsigned)((tp.from / kNumXcd + (tail_items + kNumXcd - 1) / kNumXcd) * kNumXcd);
+    }
+  }
   // more than 64 KiB of dynamic LDS has to be allowed per function (and per device)
   hipError_t e = hipSuccess;
 #define APS_LAUNCH_TILE(B, M_)                                                                                     \
   do {                                                                                                            \
-    e = hipFuncSetAttribute((const void*)gemm_nt_kernel<B, M_>, hipFuncAttributeMaxDynamicSharedMemorySize,       \
-                            TileShape<M_>::kLdsBytes);                                                            \
+    e = allow_dynamic_lds((const void*)gemm_nt_kernel<B, M_>, TileShape<M_>::kLdsBytes, (B ? 4 : 0) + M_ - 1);    \
     if (e == hipSuccess)                                                                                          \
       hipLaunchKernelGGL((gemm_nt_kernel<B, M_>), grid, dim3(kThreads), TileShape<M_>::kLdsBytes, s, g);          \
   } while (0)
@@ -842,6 +955,12 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
 #undef APS_LAUNCH_TILE
   if (e != hipSuccess) return (int)e;
   int st = launch_status();
+  if (st == APS_OK && g.tail_ways > 1) {
+    const dim3 tgrid((unsigned)((total - g.tail_from) * 64));
+    if (dtype == APS_BF16) hipLaunchKernelGGL(tail_reduce_kernel<true>, tgrid, dim3(256), 0, s, g);
+    else hipLaunchKernelGGL(tail_reduce_kernel<false>, tgrid, dim3(256), 0, s, g);
+    return launch_status();
+  }
   if (st != APS_OK || splits <= 1) return st;
   const int64_t quads = (m * n + 3) / 4;
   const dim3 rgrid((unsigned)((quads + 255) / 256));

@@ -390,6 +390,12 @@ def reproject_figures(torch, ops, dev, seed):
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": tf / MFMA_F16_PEAK_TFLOPS,
                          "traffic": PMC_TRAFFIC_BYTES["gemm_T%d" % T] if seed == 0 else None}}
+        # the vendor BLAS on the same product (what the reference's F.linear call runs on this GPU), as a
+        # stated comparison: same operands, same event timing
+        ms_blas = median(event_times(torch, lambda: torch.nn.functional.linear(x, w, bias), 20))
+        out["kv_reproject_T%d" % T]["vendor_blas_F_linear"] = {
+            "ms": ms_blas, "tflops": flops / ms_blas / 1e9, "frac_of_mfma_peak": flops / ms_blas / 1e9 / MFMA_F16_PEAK_TFLOPS,
+            "kernel_over_vendor": ms_blas / ms}
         if T == 16384 and hasattr(ops, "kv_reproject_to_cache"):
             # same product, rows written straight to random slots of [blocks,16,40,128] K and V caches
             nblk = 2 * T // 16

@@ -54,7 +54,18 @@ def test_linear_workspace_planning_is_host_only_and_consistent():
         for m in (1, 2, 3, 5, 16, 17, 48, 49, 64, 128, 129, 192, 256, 300, 700, 1024, 4096, 16384):
             s = lib.aps_linear_nt_splits(m, n, k)
             assert s >= 1
-            assert lib.aps_linear_nt_workspace_bytes(m, n, k) == (s * m * n * 4 if s > 1 else 0)
+            ws = lib.aps_linear_nt_workspace_bytes(m, n, k)
+            if s > 1:
+                assert ws == s * m * n * 4
+            elif ws:
+                # tail split of a large product: fp32 images of the parts of the tiles beyond the last full
+                # round of 256 compute units; the parts fit one round
+                tile_bytes = 256 * 256 * 4
+                tiles = -(-m // 256) * (n // 256)
+                rest = tiles % 256
+                assert tiles > 256 and rest and ws % tile_bytes == 0
+                ways = ws // tile_bytes // rest
+                assert 2 <= ways <= 4 and ways * rest <= 256 and ws == ways * rest * tile_bytes
             if m <= 2:
                 assert s == 1                                  # one launch of the dot-product kernel
             elif m <= 48:
