@@ -173,6 +173,54 @@ class HybridAttentionImpl:
         return output.view(num_tokens, hidden_size)
 
 
+class PhaseTimes:
+    """Optional per-phase GPU timing of the layers (events on the current stream).  ``with PhaseTimes() as t:``
+    switches it on for the layers run inside; ``t.totals()`` (after a synchronize) gives milliseconds per phase
+    name.  Off by default: the layers then only test one module attribute."""
+
+    active: Optional["PhaseTimes"] = None
+
+    def __init__(self) -> None:
+        self.spans = []
+
+    def __enter__(self):
+        PhaseTimes.active = self
+        return self
+
+    def __exit__(self, *exc):
+        PhaseTimes.active = None
+
+    def totals(self):
+        torch.cuda.synchronize()
+        out = {}
+        for name, a, b in self.spans:
+            out[name] = out.get(name, 0.0) + a.elapsed_time(b)
+        return out
+
+
+class _Phase:
+    __slots__ = ("name", "a")
+
+    def __init__(self, name: str) -> None:
+        self.name = name
+
+    def __enter__(self):
+        if PhaseTimes.active is not None:
+            self.a = torch.cuda.Event(enable_timing=True)
+            self.a.record()
+
+    def __exit__(self, *exc):
+        t = PhaseTimes.active
+        if t is not None:
+            b = torch.cuda.Event(enable_timing=True)
+            b.record()
+            t.spans.append((self.name, self.a, b))
+
+
+def phase(name: str) -> _Phase:
+    return _Phase(name)
+
+
 class HybridOPTAttention:
     """Self-attention of one OPT decoder layer over the hybrid cache.
 
@@ -207,24 +255,31 @@ class HybridOPTAttention:
         s = w.shape[0] // 3
         H, D = self.num_heads, self.head_dim
         # the newest hidden row of every hidden-cached sequence joins its cache first
-        ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
-                            md.hidden_cache_store_tot)
+        with phase("write"):
+            ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
+                                md.hidden_cache_store_tot)
         n_kv = md.num_decode_tokens - md.num_hidden_cache_tokens
         attn_output = torch.empty_like(hidden_states)
         if n_kv:
-            qkv, _ = self.qkv_proj(hidden_states)
-            q, k, v = qkv.chunk(chunks=3, dim=-1)
-            ops.reshape_and_cache_flash(k, v, kv_cache[0], kv_cache[1], md.new_token_slot, "auto",
-                                        token_idx=md.kv_cache_use_input)
-            ops.paged_decode_attention(q.view(-1, H, D), kv_cache[0], kv_cache[1], md.private_block_tables,
-                                       md.kv_seq_lens, self.scaling, max_seq_len=md.max_kv_seq_len or None,
-                                       out=attn_output.view(-1, H, D))
+            with phase("projections"):
+                qkv, _ = self.qkv_proj(hidden_states)
+                q, k, v = qkv.chunk(chunks=3, dim=-1)
+            with phase("write"):
+                ops.reshape_and_cache_flash(k, v, kv_cache[0], kv_cache[1], md.new_token_slot, "auto",
+                                            token_idx=md.kv_cache_use_input)
+            with phase("attention"):
+                ops.paged_decode_attention(q.view(-1, H, D), kv_cache[0], kv_cache[1], md.private_block_tables,
+                                           md.kv_seq_lens, self.scaling, max_seq_len=md.max_kv_seq_len or None,
+                                           out=attn_output.view(-1, H, D))
         else:
-            q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
-        ops.absorbed_hidden_attention(q, kv_cache, md.hidden_slots, md.hidden_seq_start, md.hidden_cache_use_input,
-                                      md.max_hidden_seq_len, w[s:2 * s], w[2 * s:], None if b is None else b[2 * s:],
-                                      self.scaling, attn_output)
-        return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
+            with phase("projections"):
+                q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
+        with phase("attention_on_hidden_rows"):
+            ops.absorbed_hidden_attention(q, kv_cache, md.hidden_slots, md.hidden_seq_start,
+                                          md.hidden_cache_use_input, md.max_hidden_seq_len, w[s:2 * s], w[2 * s:],
+                                          None if b is None else b[2 * s:], self.scaling, attn_output)
+        with phase("projections"):
+            return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
 
     def forward(self, hidden_states, kv_cache, shared_cache, attn_metadata: HybridAttentionMetadata):
         md = attn_metadata
@@ -236,8 +291,9 @@ class HybridOPTAttention:
                 if self.fused and md.holder_src is not None:
                     holder = torch.empty(md.num_tot_tokens, hidden_states.shape[1], device=hidden_states.device,
                                          dtype=hidden_states.dtype)
-                    ops.gather_hidden_rows(holder, hidden_states, kv_cache, md.holder_src, md.slot_mapping,
-                                           md.hidden_cache_use_input, md.hidden_cache_store_tot)
+                    with phase("gather"):
+                        ops.gather_hidden_rows(holder, hidden_states, kv_cache, md.holder_src, md.slot_mapping,
+                                               md.hidden_cache_use_input, md.hidden_cache_store_tot)
                 else:                                                               # aptserve_opt.py:108-121
                     ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
                                         md.hidden_cache_store_tot)
@@ -245,15 +301,19 @@ class HybridOPTAttention:
                                          dtype=hidden_states.dtype)
                     holder[md.hidden_holder_upd] = hidden_states
                     ops.cache_to_hidden(holder, kv_cache, md.slot_mapping, md.hidden_cache_use_tot)
-                q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
+                with phase("projections"):
+                    q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
                 if (self.fuse_kv_write and md.kv_dest is not None and kv_cache is not None
                         and kv_cache.dtype == holder.dtype):
                     w, b = self.qkv_proj.weight, self.qkv_proj.bias
                     s = w.shape[0] // 3
-                    ops.kv_reproject_to_cache(holder, w[s:], None if b is None else b[s:], shared_cache[0],
-                                              shared_cache[1], kv_cache[0], kv_cache[1], md.kv_dest)
-                    attn_output = self.attn.forward(q, None, None, kv_cache, shared_cache, md, kv_written=True)
-                    return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
+                    with phase("kv_gemm"):
+                        ops.kv_reproject_to_cache(holder, w[s:], None if b is None else b[s:], shared_cache[0],
+                                                  shared_cache[1], kv_cache[0], kv_cache[1], md.kv_dest)
+                    with phase("attention"):
+                        attn_output = self.attn.forward(q, None, None, kv_cache, shared_cache, md, kv_written=True)
+                    with phase("projections"):
+                        return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
                 else:
                     kv, _ = self.qkv_proj(holder, q_only=False, kv_only=True)
                     k, v = kv.chunk(chunks=2, dim=-1)

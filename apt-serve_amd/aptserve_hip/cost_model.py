@@ -10,7 +10,10 @@ point added) and returns ``slope / 5``.  ``get_coef`` keeps that recipe and swap
 * ``mode="reprojection"``: the K/V re-projection GEMM of this library (``ops.linear_nt``), i.e. the cost
   the reference's data flow pays per cached hidden block and layer;
 * ``mode="absorbed"``: the attention on the hidden rows themselves (``ops.absorbed_hidden_attention``),
-  minus nothing: what a hidden-cached block costs per layer when nothing is re-projected.
+  minus nothing: what a hidden-cached block costs per layer when nothing is re-projected;
+* ``mode="reference_recipe"``: the reference's own timed operation, ``torch.nn.functional.linear`` (the vendor
+  BLAS on this GPU) — in fp32 when ``dtype=torch.float32``, which is what the reference's ``torch.randn(...)``
+  operands are — as the figure to hold the other two against.
 """
 
 from __future__ import annotations
@@ -42,7 +45,17 @@ def get_coef(hidden_size: int, num_heads: int, num_layers: int, block_size: int,
     g = torch.Generator(device=dev).manual_seed(0)
     w = (torch.randn(3 * hidden_size, hidden_size, generator=g, device=dev) * 0.02).to(dtype)
     stats = []
-    if mode == "reprojection":
+    if mode == "reference_recipe":
+        for n in token_counts:
+            x = torch.randn(n, hidden_size, generator=g, device=dev).to(dtype)
+            torch.nn.functional.linear(x, w, None)
+            torch.cuda.synchronize(dev)
+            t0 = time.time()
+            for _ in range(num_layers):
+                torch.nn.functional.linear(x, w, None)
+            torch.cuda.synchronize(dev)
+            stats.append((n, time.time() - t0))
+    elif mode == "reprojection":
         for n in token_counts:
             x = torch.randn(n, hidden_size, generator=g, device=dev).to(dtype)
             out = torch.empty(n, 3 * hidden_size, dtype=dtype, device=dev)

@@ -152,19 +152,38 @@ class _Staging:
 _staging = {}
 
 
-def _stage(device, n: int):
+def _stage(device, n: int, zero: bool = True):
     st = _staging.setdefault(device, _Staging())
     i, host = st.take(n)
-    host.zero_()
+    if zero:                       # ragged lists leave the padding untouched; packed arrays overwrite everything
+        host.zero_()
     return st, i, host
 
 
-def _table_lens(tables: Sequence[Sequence[int]]) -> np.ndarray:
+def _table_lens(tables, need_blocks=None) -> np.ndarray:
+    """Entries per table.  A packed ``[B, W]`` array carries no lengths: every table is then taken to be exactly
+    as long as its sequence needs (what a block manager that grows tables one block at a time produces), or
+    empty when the array has no columns."""
+    if isinstance(tables, np.ndarray):
+        if tables.ndim != 2:
+            raise ValueError("packed block tables must be a [batch, width] array")
+        if tables.shape[1] == 0 or need_blocks is None:
+            return np.zeros(tables.shape[0], dtype=np.int64)
+        if int(need_blocks.max()) > tables.shape[1]:
+            raise ValueError("packed block table narrower than ceil(seq_len/block_size)")
+        return need_blocks.astype(np.int64)
     return np.fromiter(map(len, tables), dtype=np.int64, count=len(tables))
 
 
-def _pack_tables(tables: Sequence[Sequence[int]], lens: np.ndarray, out: np.ndarray) -> None:
-    """Ragged lists -> 0-padded ``out[B, W]`` with one flat copy instead of a Python loop per row."""
+def _pack_tables(tables, lens: np.ndarray, out: np.ndarray, rows: Optional[np.ndarray] = None) -> None:
+    """Ragged lists -> 0-padded ``out[B, W]`` with one flat copy instead of a Python loop per row.  A packed
+    ``[B, >=W]`` int array is copied as it is (``rows``: boolean mask of the tables that count, the others are
+    left empty)."""
+    if isinstance(tables, np.ndarray):       # 0-padded by contract: one block copy
+        out[:, :] = tables[:, :out.shape[1]]
+        if rows is not None:
+            out[~rows] = 0
+        return
     total = int(lens.sum())
     if total == 0:
         return
@@ -185,6 +204,10 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
     ``block_tables[b]`` is sequence b's private table, ``block_tables_4_shared[b]`` its
     shared (workspace) table (empty for K/V-cached sequences).  An empty private table
     (the memory-profiling run) yields padding slots.
+
+    Tables may be lists of lists (what the reference's scheduler hands over) or packed, 0-padded
+    ``[batch, width]`` int arrays that the caller keeps up to date between steps: flattening ~10 k Python
+    integers of a 256-sequence batch costs more host time than everything else in this function together.
     """
     device = torch.device(device)
     B = len(seq_lens)
@@ -197,7 +220,7 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
     if np.any(lens <= 0):
         raise ValueError("sequence lengths must be positive")
     need_blocks = -(-lens // block_size)
-    bt_lens = _table_lens(block_tables)
+    bt_lens = _table_lens(block_tables, need_blocks)
     have_tables = bool(bt_lens.any())
     W = int(bt_lens.max()) if have_tables else 0
     if have_tables and np.any(bt_lens < need_blocks):
@@ -210,7 +233,7 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
     if not is_prompt:
         if len(block_tables_4_shared) != B:
             raise ValueError("block_tables_4_shared must have one entry per sequence")
-        bts_lens = _table_lens(block_tables_4_shared) * hid      # tables of K/V-cached sequences are ignored
+        bts_lens = _table_lens(block_tables_4_shared, need_blocks * hid) * hid   # K/V-cached sequences: ignored
         if have_tables and np.any(bts_lens[hid] < need_blocks[hid]):
             b = int(np.nonzero(hid & (bts_lens < need_blocks))[0][0])
             raise ValueError(f"sequence {b}: shared block table shorter than ceil(seq_len/block_size)")
@@ -222,15 +245,19 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
         # width of the table handed to attention: the longest *selected* table (:601-609)
         Wo = int(np.where(hid, bts_lens, bt_lens).max()) if have_tables else 0
         # one packed upload: lens | flags | private tables | shared tables
-        stg, slot, host = _stage(device, 2 * B + B * W + B * Ws)
+        arrays = isinstance(block_tables, np.ndarray) and (Ws == 0 or isinstance(block_tables_4_shared, np.ndarray))
+        stg, slot, host = _stage(device, 2 * B + B * W + B * Ws, zero=not arrays)
         hv = host.numpy()
         hv[:B] = lens
         hv[B:2 * B] = hid
         if W:
             _pack_tables(block_tables, bt_lens, hv[2 * B:2 * B + B * W].reshape(B, W))
         if Ws:
-            shared = [t if h else () for t, h in zip(block_tables_4_shared, hid)]
-            _pack_tables(shared, bts_lens, hv[2 * B + B * W:].reshape(B, Ws))
+            if isinstance(block_tables_4_shared, np.ndarray):
+                _pack_tables(block_tables_4_shared, bts_lens, hv[2 * B + B * W:].reshape(B, Ws), rows=hid)
+            else:
+                shared = [t if h else () for t, h in zip(block_tables_4_shared, hid)]
+                _pack_tables(shared, bts_lens, hv[2 * B + B * W:].reshape(B, Ws))
         packed = stg.upload(slot, host, device)
         d_lens, d_hid = packed[:B], packed[B:2 * B]
         d_bt = packed[2 * B:2 * B + B * W].view(B, W)
@@ -242,10 +269,13 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
         (slot_mapping, slot_mapping_shared, use_tot, kv_use, use_input, store_tot, upd, pull, positions,
          totals, holder_src, kv_dest, hidden_slots, hidden_seq_start, kv_use_input,
          new_token_slot) = torch.split(buf64, sizes64)
-        sizes32 = [B * Wo, B + 1, B + 1, B, B]
+        n_types = (B * Wo + 3) // 4 if (n_hs and Wo) else 0          # uint8 [B, Wo] carried in the int32 buffer
+        sizes32 = [B * Wo, B + 1, B + 1, B, B, n_types]
         buf32 = torch.empty(sum(sizes32), **i32)
-        bt_out, seq_start, query_start, ctx, kv_seq_lens = torch.split(buf32, sizes32)
+        bt_out, seq_start, query_start, ctx, kv_seq_lens, types32 = torch.split(buf32, sizes32)
         bt_out = bt_out.view(B, Wo)
+        # per-block source for the hybrid attention: every block of a hidden sequence is a workspace block
+        block_types = types32.view(torch.uint8)[:B * Wo].view(B, Wo) if n_types else None
         with torch.cuda.device(device):
             st = lib.aps_build_decode_metadata(
                 d_lens.data_ptr(), d_hid.data_ptr(), d_bt.data_ptr() if W else None, W, W,
@@ -256,7 +286,8 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
                 holder_src.data_ptr(), kv_dest.data_ptr(), hidden_slots.data_ptr() if n_hr else None,
                 hidden_seq_start.data_ptr() if n_hs else None, kv_use_input.data_ptr() if n_kv else None,
                 new_token_slot.data_ptr(), kv_seq_lens.data_ptr(), num_tot, n_hr, n_hs, n_kv,
-                bt_out.data_ptr() if Wo else None, Wo, Wo, seq_start.data_ptr(),
+                bt_out.data_ptr() if Wo else None, Wo, Wo,
+                None if block_types is None else block_types.data_ptr(), seq_start.data_ptr(),
                 query_start.data_ptr(), ctx.data_ptr(), positions.data_ptr(), totals.data_ptr(),
                 torch.cuda.current_stream(device).cuda_stream)
         _lib.check(st, "build_decode_metadata")
@@ -264,14 +295,12 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
             got = totals.tolist()
             if got != [num_tot, n_hr, n_hs, n_kv]:
                 raise RuntimeError(f"device totals {got} disagree with the host's {[num_tot, n_hr, n_hs, n_kv]}")
-        # per-block source for the hybrid attention: every block of a hidden sequence is a workspace block
-        block_types = d_hid.to(torch.uint8).unsqueeze(1).expand(B, Wo).contiguous() if (n_hs and Wo) else None
         return HybridAttentionMetadata(
             num_prefills=0, num_prefill_tokens=0, num_decode_tokens=B, num_hidden_cache_tokens=n_hs,
             num_tot_tokens=num_tot, slot_mapping=slot_mapping, slot_mapping_shared=slot_mapping_shared,
             hidden_cache_use_tot=use_tot, kv_cache_use_tot=kv_use, hidden_cache_use_input=use_input,
             hidden_cache_store_tot=store_tot, hidden_holder_upd=upd, hidden_holder_pull=pull,
-            seq_lens=[int(x) for x in lens], seq_lens_tensor=d_lens, max_query_len=1, max_prefill_seq_len=0,
+            seq_lens=lens.tolist(), seq_lens_tensor=d_lens, max_query_len=1, max_prefill_seq_len=0,
             max_decode_seq_len=int(lens.max()), query_start_loc=query_start, seq_start_loc=seq_start,
             context_lens_tensor=ctx, block_tables=bt_out, use_cuda_graph=False, input_positions=positions,
             block_types=block_types, holder_src=holder_src, kv_dest=kv_dest, hidden_slots=hidden_slots,
@@ -322,14 +351,19 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
         num_tot_tokens=n_tok, slot_mapping=slot_mapping, slot_mapping_shared=empty64,
         hidden_cache_use_tot=use_input, kv_cache_use_tot=kv_use, hidden_cache_use_input=use_input,
         hidden_cache_store_tot=use_input, hidden_holder_upd=empty64, hidden_holder_pull=empty64,
-        seq_lens=[int(x) for x in lens], seq_lens_tensor=d_lens, max_query_len=int(qlens.max()),
+        seq_lens=lens.tolist(), seq_lens_tensor=d_lens, max_query_len=int(qlens.max()),
         max_prefill_seq_len=int(lens.max()), max_decode_seq_len=0, query_start_loc=query_start,
         seq_start_loc=seq_start, context_lens_tensor=ctx,
         block_tables=torch.empty(B, 0, **i32), use_cuda_graph=False, input_positions=positions, block_types=None,
         token_is_hidden=token_is_hidden, max_prompt_context_len=int(ctxs.max()))
 
 
-def build_from_batch(batch, device, **kw) -> HybridAttentionMetadata:
-    """Convenience for :class:`aptserve_hip.workloads.Batch`."""
+def build_from_batch(batch, device, packed: bool = False, **kw) -> HybridAttentionMetadata:
+    """Convenience for :class:`aptserve_hip.workloads.Batch`; ``packed`` hands over the batch's block tables as
+    the 0-padded int32 arrays ``batch.packed_tables()`` keeps instead of as lists of lists."""
+    if packed:
+        bt, bts = batch.packed_tables()
+        return build_metadata(batch.is_prompt, batch.seq_lens_np, batch.use_hidden_np, bt, bts, batch.block_size,
+                              device, **kw)
     return build_metadata(batch.is_prompt, batch.seq_lens, batch.use_hidden, batch.block_tables,
                           batch.block_tables_4_shared, batch.block_size, device, **kw)

@@ -19,7 +19,7 @@ import torch
 import torch.nn.functional as F
 
 from . import ops
-from .backend import HybridOPTAttention
+from .backend import HybridOPTAttention, phase
 from .metadata import HybridAttentionMetadata
 
 
@@ -75,9 +75,10 @@ class HybridOPTDecoderLayer:
         hidden_states = residual + hidden_states
         residual = hidden_states
         hidden_states = F.layer_norm(hidden_states, (Hd,), w[p + "final_ln_w"], w[p + "final_ln_b"])
-        hidden_states = ops.linear_nt(hidden_states, w[p + "fc1_w"], w[p + "fc1_b"])
-        hidden_states = torch.relu_(hidden_states)
-        hidden_states = ops.linear_nt(hidden_states, w[p + "fc2_w"], w[p + "fc2_b"])
+        with phase("projections"):
+            hidden_states = ops.linear_nt(hidden_states, w[p + "fc1_w"], w[p + "fc1_b"])
+            hidden_states = torch.relu_(hidden_states)
+            hidden_states = ops.linear_nt(hidden_states, w[p + "fc2_w"], w[p + "fc2_b"])
         return residual + hidden_states
 
     __call__ = forward

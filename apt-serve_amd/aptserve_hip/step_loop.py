@@ -66,6 +66,16 @@ def synth_requests(seed: int, n: int, rate: float = 3.0, cv: float = 1.0, hidden
     return reqs
 
 
+def fixed_step_cost(decode_s: float = 0.0125, prefill_s: float = 0.010, prefill_s_per_token: float = 2.0e-5):
+    """A fixed cost model for the simulated clock: a decode step costs ``decode_s``, a prompt step
+    ``prefill_s + tokens * prefill_s_per_token`` (roughly what OPT-13B takes on one MI355X)."""
+    def cost(entry: Dict) -> float:
+        if entry["kind"] == "decode":
+            return decode_s
+        return prefill_s + prefill_s_per_token * entry["tokens"]
+    return cost
+
+
 class BlockPool:
     def __init__(self, num_blocks: int) -> None:
         self.n = num_blocks
@@ -105,7 +115,10 @@ class StepLoop:
 
     def __init__(self, forward: Callable, pick: Callable, requests: List[Request], num_blocks: int, block_size: int,
                  device, max_prompt_tokens: int = 4096, max_seqs: int = 256,
-                 on_step: Optional[Callable] = None) -> None:
+                 on_step: Optional[Callable] = None, step_cost: Optional[Callable[[Dict], float]] = None) -> None:
+        """``step_cost(entry) -> seconds`` drives the simulated clock from a fixed cost model (same arrivals,
+        admissions and batches whatever the measured speed, so two data flows can be compared step by step);
+        ``None`` advances it by the measured wall time of every step."""
         self.forward, self.pick = forward, pick
         self.waiting = sorted(requests, key=lambda r: r.arrival)
         self.running: List[Request] = []
@@ -115,6 +128,8 @@ class StepLoop:
         self.max_prompt_tokens, self.max_seqs = max_prompt_tokens, max_seqs
         self.now = 0.0
         self.on_step = on_step
+        self.step_cost = step_cost
+        self.preemptions = 0
         self.log: List[Dict] = []
 
     def _admit(self) -> List[Request]:
@@ -131,6 +146,27 @@ class StepLoop:
             tokens += len(r.prompt_ids)
         return batch
 
+    def _make_room(self) -> None:
+        """Before a decode step: if the free lists cannot take the blocks the running sequences are about to
+        need, the most recently admitted sequences are preempted in recompute mode (blocks released, generated
+        tokens dropped, back to the head of the queue), as the reference does when it runs out of blocks
+        (additional_designs/core/aptserve_scheduler.py:2118-2130)."""
+        while self.running:
+            need_p = need_s = 0
+            for r in self.running:
+                p, s_ = self.pool.blocks_needed(r, r.seq_len, self.block_size)
+                need_p += p
+                need_s += s_
+            if need_p <= len(self.pool.free_private) and need_s <= len(self.pool.free_shared):
+                return
+            if len(self.running) == 1:
+                raise RuntimeError("the block pool cannot hold a single sequence of this length")
+            victim = self.running.pop()
+            self.pool.release(victim)
+            victim.generated = []
+            self.waiting.insert(0, victim)
+            self.preemptions += 1
+
     def step(self) -> Optional[Dict]:
         """Run one step; returns its log entry, or None when nothing is left to do."""
         batch = self._admit()
@@ -141,6 +177,7 @@ class StepLoop:
                     return None
                 self.now = self.waiting[0].arrival      # idle until the next arrival
                 return self.step()
+            self._make_room()
             batch = self.running
             for r in batch:                              # slot for the token produced by the previous step
                 self.pool.grow(r, r.seq_len, self.block_size)
@@ -158,12 +195,14 @@ class StepLoop:
         t1 = time.perf_counter()
         hidden = self.forward(input_ids, md.input_positions, md)
         nxt = self.pick(hidden, md)
+        t_enq = time.perf_counter()              # everything is enqueued: host time of the step
         torch.cuda.synchronize(self.device)
         t2 = time.perf_counter()
         nxt_host = nxt.tolist()
         entry = dict(kind="prefill" if is_prompt else "decode", seqs=len(batch), tokens=int(len(ids)),
                      rows=md.num_tot_tokens, hidden_seqs=sum(r.use_hidden for r in batch),
-                     metadata_ms=(t1 - t0) * 1e3, model_ms=(t2 - t1) * 1e3, now=self.now)
+                     metadata_ms=(t1 - t0) * 1e3, model_ms=(t2 - t1) * 1e3, host_enqueue_ms=(t_enq - t1) * 1e3,
+                     now=self.now)
         if self.on_step is not None:
             self.on_step(dict(is_prompt=is_prompt, seq_lens=seq_lens, use_hidden=[r.use_hidden for r in batch],
                               block_tables=[list(r.block_table) for r in batch],
@@ -178,7 +217,7 @@ class StepLoop:
             self.pool.release(r)
             self.running.remove(r)
             self.finished.append(r)
-        self.now += (t2 - t0)
+        self.now += self.step_cost(entry) if self.step_cost is not None else (t2 - t0)
         self.log.append(entry)
         return entry
 

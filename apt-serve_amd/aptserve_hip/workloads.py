@@ -38,6 +38,22 @@ class Batch:
     def context_lens(self) -> List[int]:
         return [0 if self.is_prompt else l - 1 for l in self.seq_lens]
 
+    def packed_tables(self):
+        """The block tables as 0-padded int32 ``[batch, width]`` arrays (built once, then kept): the form a
+        block manager that updates its tables in place would hand to the metadata builder."""
+        if getattr(self, "_packed", None) is None:
+            def pack(tables):
+                w = max((len(t) for t in tables), default=0)
+                out = np.zeros((len(self.seq_lens), w), dtype=np.int32)
+                for b, t in enumerate(tables):
+                    out[b, :len(t)] = t
+                return out
+            shared = self.block_tables_4_shared or [[] for _ in self.seq_lens]
+            self._packed = (pack(self.block_tables), pack(shared))
+            self.seq_lens_np = np.asarray(self.seq_lens, dtype=np.int64)
+            self.use_hidden_np = np.asarray(self.use_hidden, dtype=bool)
+        return self._packed
+
 
 def lognormal_lengths(rng: np.random.Generator, n: int, mu: float = 6.2, sigma: float = 0.8,
                       lo: int = 16, hi: int = 2048) -> np.ndarray:

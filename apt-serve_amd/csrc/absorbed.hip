@@ -472,11 +472,11 @@ int launch_nn(const NnArgs& g, int kparts, hipStream_t s) {
   const dim3 grid((unsigned)((g.n + kNnWaves * 128 - 1) / (kNnWaves * 128)), (unsigned)(g.batches * g.m_tiles),
                   (unsigned)kparts);
   if (mt == 1)
-    hipLaunchKernelGGL((nn_few_rows_kernel<BF16, 1>), grid, dim3(kNnWaves * 64), 0, s, g);
+    APS_LAUNCH((nn_few_rows_kernel<BF16, 1>), grid, dim3(kNnWaves * 64), 0, s, g);
   else if (mt == 2)
-    hipLaunchKernelGGL((nn_few_rows_kernel<BF16, 2>), grid, dim3(kNnWaves * 64), 0, s, g);
+    APS_LAUNCH((nn_few_rows_kernel<BF16, 2>), grid, dim3(kNnWaves * 64), 0, s, g);
   else
-    hipLaunchKernelGGL((nn_few_rows_kernel<BF16, 3>), grid, dim3(kNnWaves * 64), 0, s, g);
+    APS_LAUNCH((nn_few_rows_kernel<BF16, 3>), grid, dim3(kNnWaves * 64), 0, s, g);
   return launch_status();
 }
 
@@ -543,7 +543,7 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
 using namespace aps;
 
 // the per-head value projection lives with the other weight-streaming kernels
-int aps_internal_headwise_linear(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n,
+__attribute__((visibility("hidden"))) int aps_internal_headwise_linear(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n,
                                  int64_t k, int64_t x_stride, int64_t x_head_stride, int head_rows, int64_t w_stride,
                                  int64_t out_stride, const int64_t* out_row_map, int64_t out_rows, int dtype,
                                  hipStream_t stream);
@@ -612,7 +612,7 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     g.k = hidden;
     int32_t* tiles = (int32_t*)(ws + p.off_tiles);
     int32_t* order = n_seqs > 1 && n_seqs <= kMaxOrderedSeqs ? (int32_t*)(ws + p.off_order) : nullptr;
-    hipLaunchKernelGGL(seq_plan_kernel, dim3(1), dim3(256), 0, s, seq_start, (int)n_seqs, kScTokens, tiles, order);
+    APS_LAUNCH(seq_plan_kernel, dim3(1), dim3(256), 0, s, seq_start, (int)n_seqs, kScTokens, tiles, order);
     g.tile_start = tiles; g.n_seqs = (int)n_seqs;
     g.k_per_part = p.score_k_per_part; g.s_part_stride = s_part_stride;
     // upper bound of the tile count that the host can know: every sequence at max_len
@@ -625,7 +625,7 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
   do {                                                                                                            \
     e = allow_dynamic_lds((const void*)hidden_scores_kernel<B, N>, scores_lds_bytes<N>(), (B ? 6 : 0) + N - 1);   \
     if (e == hipSuccess)                                                                                          \
-      hipLaunchKernelGGL((hidden_scores_kernel<B, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g);      \
+      APS_LAUNCH((hidden_scores_kernel<B, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g);      \
   } while (0)
 #define APS_LAUNCH_SCORES_N(B)                                                                        \
   switch (nht) {                                                                                      \
@@ -647,10 +647,10 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
   {
     const dim3 grid((unsigned)num_heads, (unsigned)n_seqs);
     if (bf16)
-      hipLaunchKernelGGL(softmax_rows_kernel<true>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp,
+      APS_LAUNCH(softmax_rows_kernel<true>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp,
                          p.score_parts, s_part_stride);
     else
-      hipLaunchKernelGGL(softmax_rows_kernel<false>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp,
+      APS_LAUNCH(softmax_rows_kernel<false>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp,
                          p.score_parts, s_part_stride);
     const int st = launch_status();
     if (st != APS_OK) return st;
@@ -675,10 +675,10 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
       const int64_t quads = n_seqs * num_heads * hidden / 4;
       const dim3 rgrid((unsigned)((quads + 255) / 256));
       if (bf16)
-        hipLaunchKernelGGL(nn_reduce_kernel<true>, rgrid, dim3(256), 0, s, partial, ctx, p.kparts, (int)n_seqs,
+        APS_LAUNCH(nn_reduce_kernel<true>, rgrid, dim3(256), 0, s, partial, ctx, p.kparts, (int)n_seqs,
                            num_heads, hidden, g.out_batch_stride, g.out_row_stride, 1.f);
       else
-        hipLaunchKernelGGL(nn_reduce_kernel<false>, rgrid, dim3(256), 0, s, partial, ctx, p.kparts, (int)n_seqs,
+        APS_LAUNCH(nn_reduce_kernel<false>, rgrid, dim3(256), 0, s, partial, ctx, p.kparts, (int)n_seqs,
                            num_heads, hidden, g.out_batch_stride, g.out_row_stride, 1.f);
       st = launch_status();
       if (st != APS_OK) return st;
@@ -711,7 +711,7 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
   do {                                                                                                           \
     e = allow_dynamic_lds((const void*)head_proj_kernel<B, N>, scores_lds_bytes<N>(), 12 + (B ? 2 : 0) + N - 2); \
     if (e == hipSuccess)                                                                                         \
-      hipLaunchKernelGGL((head_proj_kernel<B, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g);         \
+      APS_LAUNCH((head_proj_kernel<B, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g);         \
   } while (0)
 #define APS_LAUNCH_PROJ_N(B)                                                                          \
   if (nht == 2) APS_LAUNCH_PROJ(B, 2); else APS_LAUNCH_PROJ(B, 3);

@@ -46,6 +46,14 @@ inline int common_vec_bytes(std::initializer_list<uint64_t> vals) {
 
 inline uint64_t addr(const void* p) { return (uint64_t)(uintptr_t)p; }
 
+// Every kernel launch goes through APS_LAUNCH, which first drops whatever error an earlier, unrelated call
+// left in the runtime's per-thread slot: launch_status() then reports this launch and nothing older.
+#define APS_LAUNCH(...)             \
+  do {                              \
+    (void)hipGetLastError();        \
+    hipLaunchKernelGGL(__VA_ARGS__); \
+  } while (0)
+
 inline int launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? APS_OK : (int)e;

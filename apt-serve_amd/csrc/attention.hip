@@ -533,10 +533,10 @@ template <int QT, int KV, int D, int HPW, int DEPTH>
 void launch_group(const AttnArgs& a, int64_t batch, int waves, hipStream_t s) {
   const dim3 grid((unsigned)(a.num_heads / HPW), (unsigned)batch);
   switch (waves) {
-    case 1: hipLaunchKernelGGL((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 1>), grid, dim3(64), 0, s, a); break;
-    case 2: hipLaunchKernelGGL((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 2>), grid, dim3(128), 0, s, a); break;
-    case 4: hipLaunchKernelGGL((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 4>), grid, dim3(256), 0, s, a); break;
-    default: hipLaunchKernelGGL((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 8>), grid, dim3(512), 0, s, a); break;
+    case 1: APS_LAUNCH((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 1>), grid, dim3(64), 0, s, a); break;
+    case 2: APS_LAUNCH((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 2>), grid, dim3(128), 0, s, a); break;
+    case 4: APS_LAUNCH((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 4>), grid, dim3(256), 0, s, a); break;
+    default: APS_LAUNCH((paged_decode_group_kernel<QT, KV, D, HPW, DEPTH, 8>), grid, dim3(512), 0, s, a); break;
   }
 }
 
@@ -554,7 +554,7 @@ void launch_head_size(const AttnArgs& a, int64_t batch, const DecodePlan& plan, 
         launch_group<QT, KV, D, HPW, DEPTH>(a, batch, plan.waves, s);
       } else {
         const dim3 grid((unsigned)(a.num_heads / HPW), (unsigned)a.num_partitions, (unsigned)batch);
-        hipLaunchKernelGGL((paged_decode_kernel<QT, KV, D, HPW, DEPTH>), grid, dim3(64), 0, s, a);
+        APS_LAUNCH((paged_decode_kernel<QT, KV, D, HPW, DEPTH>), grid, dim3(64), 0, s, a);
       }
       return;
     }
@@ -563,14 +563,14 @@ void launch_head_size(const AttnArgs& a, int64_t batch, const DecodePlan& plan, 
     launch_group<QT, KV, D, 1, DEPTH>(a, batch, plan.waves, s);
   } else {
     const dim3 grid((unsigned)a.num_heads, (unsigned)a.num_partitions, (unsigned)batch);
-    hipLaunchKernelGGL((paged_decode_kernel<QT, KV, D, 1, DEPTH>), grid, dim3(64), 0, s, a);
+    APS_LAUNCH((paged_decode_kernel<QT, KV, D, 1, DEPTH>), grid, dim3(64), 0, s, a);
   }
 }
 
 template <int QT, int KV>
 int launch_decode(const AttnArgs& a, int head_size, int64_t batch, const DecodePlan& plan, hipStream_t s) {
   if (plan.order_scratch) {
-    hipLaunchKernelGGL(rank_sequences_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, a.seq_lens,
+    APS_LAUNCH(rank_sequences_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, a.seq_lens,
                        (int)batch, const_cast<int32_t*>(a.seq_order));
     const int st = launch_status();
     if (st != APS_OK) return st;
@@ -588,7 +588,7 @@ int launch_decode(const AttnArgs& a, int head_size, int64_t batch, const DecodeP
   int st = launch_status();
   if (st != APS_OK || plan.group || a.num_partitions == 1) return st;
   const int threads = head_size >= 256 ? 256 : (head_size + 63) / 64 * 64;
-  hipLaunchKernelGGL((combine_partitions_kernel<QT>), dim3((unsigned)a.num_heads, (unsigned)batch), dim3(threads), 0,
+  APS_LAUNCH((combine_partitions_kernel<QT>), dim3((unsigned)a.num_heads, (unsigned)batch), dim3(threads), 0,
                      s, a.out, a.part_out, a.part_lse, a.seq_lens, a.out_stride, a.num_heads, head_size,
                      a.num_partitions, a.partition_size);
   return launch_status();

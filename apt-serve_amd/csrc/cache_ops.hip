@@ -343,7 +343,7 @@ int launch_rows_vb(const Op& op, int64_t n_items, int64_t row_bytes, hipStream_t
   if (grid_y > 65535) return APS_ERR_UNSUPPORTED;
   const int64_t waves = (items_per_y * segs_per_row + U - 1) / U;
   const int64_t grid_x = (waves + kMaxThreads / 64 - 1) / (kMaxThreads / 64);
-  hipLaunchKernelGGL((row_mover<VB, U, Op>), dim3((unsigned)grid_x, (unsigned)grid_y), dim3(kMaxThreads), 0, s, op,
+  APS_LAUNCH((row_mover<VB, U, Op>), dim3((unsigned)grid_x, (unsigned)grid_y), dim3(kMaxThreads), 0, s, op,
                      n_items, (uint32_t)segs_per_row, (uint32_t)row_bytes, (uint32_t)items_per_y);
   return launch_status();
 }
@@ -453,11 +453,11 @@ int launch_kv_scatter_fp8(const void* key, const void* value, void* k_cache, voi
   if (threads > kMaxThreads) threads = kMaxThreads;
   const dim3 grid((unsigned)(2 * n));
   if (aligned)
-    hipLaunchKernelGGL((kv_scatter_fp8<InT, 8>), grid, dim3(threads), 0, s, (const InT*)key, (const InT*)value,
+    APS_LAUNCH((kv_scatter_fp8<InT, 8>), grid, dim3(threads), 0, s, (const InT*)key, (const InT*)value,
                        (uint8_t*)k_cache, (uint8_t*)v_cache, slot_mapping, token_idx, skip_mask, num_tokens,
                        key_stride, value_stride, block_stride, num_blocks, block_size, row_elems, k_scale, v_scale);
   else
-    hipLaunchKernelGGL((kv_scatter_fp8<InT, 1>), grid, dim3(threads), 0, s, (const InT*)key, (const InT*)value,
+    APS_LAUNCH((kv_scatter_fp8<InT, 1>), grid, dim3(threads), 0, s, (const InT*)key, (const InT*)value,
                        (uint8_t*)k_cache, (uint8_t*)v_cache, slot_mapping, token_idx, skip_mask, num_tokens,
                        key_stride, value_stride, block_stride, num_blocks, block_size, row_elems, k_scale, v_scale);
   return launch_status();
@@ -808,13 +808,13 @@ int aps_stream_probe(int mode, int chunks_per_thread, void* dst, const void* src
   VecOf<16>::type* d = (VecOf<16>::type*)dst;
   const VecOf<16>::type* sp = (const VecOf<16>::type*)src;
   if (chunks_per_thread == 1) {
-    if (mode == 0) hipLaunchKernelGGL(copy_bytes_kernel<1>, g, b, 0, s, d, sp, n_vec);
-    else if (mode == 1) hipLaunchKernelGGL(read_bytes_kernel<1>, g, b, 0, s, (uint32_t*)dst, sp, n_vec);
-    else hipLaunchKernelGGL(fill_bytes_kernel<1>, g, b, 0, s, d, n_vec, 0x3c003c00u);
+    if (mode == 0) APS_LAUNCH(copy_bytes_kernel<1>, g, b, 0, s, d, sp, n_vec);
+    else if (mode == 1) APS_LAUNCH(read_bytes_kernel<1>, g, b, 0, s, (uint32_t*)dst, sp, n_vec);
+    else APS_LAUNCH(fill_bytes_kernel<1>, g, b, 0, s, d, n_vec, 0x3c003c00u);
   } else {
-    if (mode == 0) hipLaunchKernelGGL(copy_bytes_kernel<4>, g, b, 0, s, d, sp, n_vec);
-    else if (mode == 1) hipLaunchKernelGGL(read_bytes_kernel<4>, g, b, 0, s, (uint32_t*)dst, sp, n_vec);
-    else hipLaunchKernelGGL(fill_bytes_kernel<4>, g, b, 0, s, d, n_vec, 0x3c003c00u);
+    if (mode == 0) APS_LAUNCH(copy_bytes_kernel<4>, g, b, 0, s, d, sp, n_vec);
+    else if (mode == 1) APS_LAUNCH(read_bytes_kernel<4>, g, b, 0, s, (uint32_t*)dst, sp, n_vec);
+    else APS_LAUNCH(fill_bytes_kernel<4>, g, b, 0, s, d, n_vec, 0x3c003c00u);
   }
   return launch_status();
 }

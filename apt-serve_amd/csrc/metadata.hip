@@ -63,6 +63,7 @@ struct MetaArgs {
   int64_t* hidden_slots; int64_t* hidden_seq_start;
   int64_t* kv_cache_use_input; int64_t* new_token_slot; int32_t* kv_seq_lens;
   int32_t* block_tables_out; int64_t out_stride; int out_width;
+  uint8_t* block_types_out;   // [batch][out_width], nullable: 1 in every column of a hidden-cached sequence
   int32_t* seq_start_loc; int32_t* query_start_loc; int32_t* context_lens_out; int64_t* input_positions;
   int64_t* totals;
   int64_t cap_rows, cap_hidden_rows, cap_hidden_seqs, cap_kv;
@@ -136,8 +137,10 @@ __global__ __launch_bounds__(kThreads) void decode_metadata_kernel(const MetaArg
   // block table handed to attention: the shared table for hidden sequences, the private one otherwise
   const int32_t* src = hid ? bts : bt;
   const int src_w = hid ? a.shared_width : a.table_width;
-  for (int w = threadIdx.x; w < a.out_width; w += kThreads)
+  for (int w = threadIdx.x; w < a.out_width; w += kThreads) {
     a.block_tables_out[(int64_t)b * a.out_stride + w] = (src && w < src_w) ? src[w] : 0;
+    if (a.block_types_out) a.block_types_out[(int64_t)b * a.out_width + w] = hid ? 1 : 0;
+  }
 
   if (threadIdx.x == 0) {
     if (b == 0) { a.seq_start_loc[0] = 0; a.query_start_loc[0] = 0; }
@@ -219,7 +222,8 @@ int aps_build_decode_metadata(const int32_t* seq_lens, const int32_t* use_hidden
                               int64_t* new_token_slot, int32_t* kv_seq_lens, int64_t cap_rows,
                               int64_t cap_hidden_rows,
                               int64_t cap_hidden_seqs, int64_t cap_kv_seqs, int32_t* block_tables_out,
-                              int64_t out_stride, int64_t out_width, int32_t* seq_start_loc,
+                              int64_t out_stride, int64_t out_width, uint8_t* block_types_out,
+                              int32_t* seq_start_loc,
                               int32_t* query_start_loc, int32_t* context_lens, int64_t* input_positions,
                               int64_t* totals, aps_stream_t stream) {
   if (batch < 0 || block_size <= 0 || table_width < 0 || shared_width < 0 || out_width < 0)
@@ -249,11 +253,12 @@ int aps_build_decode_metadata(const int32_t* seq_lens, const int32_t* use_hidden
   a.hidden_slots = hidden_slots; a.hidden_seq_start = hidden_seq_start;
   a.kv_cache_use_input = kv_cache_use_input; a.new_token_slot = new_token_slot; a.kv_seq_lens = kv_seq_lens;
   a.block_tables_out = block_tables_out; a.out_stride = out_stride; a.out_width = (int)out_width;
+  a.block_types_out = out_width ? block_types_out : nullptr;
   a.seq_start_loc = seq_start_loc; a.query_start_loc = query_start_loc; a.context_lens_out = context_lens;
   a.input_positions = input_positions; a.totals = totals;
   a.cap_rows = cap_rows; a.cap_hidden_rows = cap_hidden_rows; a.cap_hidden_seqs = cap_hidden_seqs;
   a.cap_kv = cap_kv_seqs;
-  hipLaunchKernelGGL(decode_metadata_kernel, dim3((unsigned)batch), dim3(kThreads), 0, (hipStream_t)stream, a);
+  APS_LAUNCH(decode_metadata_kernel, dim3((unsigned)batch), dim3(kThreads), 0, (hipStream_t)stream, a);
   return launch_status();
 }
 
@@ -282,7 +287,7 @@ int aps_build_prefill_metadata(const int32_t* seq_lens, const int32_t* context_l
   a.seq_start_loc = seq_start_loc; a.query_start_loc = query_start_loc; a.context_lens_out = context_lens;
   a.totals = totals;
   a.cap_rows = cap_tokens; a.cap_hidden_rows = cap_hidden_tokens; a.cap_kv = cap_kv_tokens;
-  hipLaunchKernelGGL(prefill_metadata_kernel, dim3((unsigned)batch), dim3(kThreads), 0, (hipStream_t)stream, a);
+  APS_LAUNCH(prefill_metadata_kernel, dim3((unsigned)batch), dim3(kThreads), 0, (hipStream_t)stream, a);
   return launch_status();
 }
 

@@ -289,11 +289,11 @@ int aps_varlen_prefill_attention(void* out, const void* q, const void* k, const 
   const dim3 grid((unsigned)num_heads, (unsigned)num_seqs, (unsigned)q_tiles);
   hipStream_t s = (hipStream_t)stream;
   if (dtype == APS_F16) {
-    if (head_size == 64) hipLaunchKernelGGL((prefill_attention_kernel<false, 64>), grid, dim3(kThreads), 0, s, a);
-    else hipLaunchKernelGGL((prefill_attention_kernel<false, 128>), grid, dim3(kThreads), 0, s, a);
+    if (head_size == 64) APS_LAUNCH((prefill_attention_kernel<false, 64>), grid, dim3(kThreads), 0, s, a);
+    else APS_LAUNCH((prefill_attention_kernel<false, 128>), grid, dim3(kThreads), 0, s, a);
   } else {
-    if (head_size == 64) hipLaunchKernelGGL((prefill_attention_kernel<true, 64>), grid, dim3(kThreads), 0, s, a);
-    else hipLaunchKernelGGL((prefill_attention_kernel<true, 128>), grid, dim3(kThreads), 0, s, a);
+    if (head_size == 64) APS_LAUNCH((prefill_attention_kernel<true, 64>), grid, dim3(kThreads), 0, s, a);
+    else APS_LAUNCH((prefill_attention_kernel<true, 128>), grid, dim3(kThreads), 0, s, a);
   }
   return launch_status();
 }

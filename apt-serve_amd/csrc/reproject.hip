@@ -611,7 +611,7 @@ __global__ __launch_bounds__(kRsWaves * 64) void rowstream_nt_kernel(const GemmA
 
 template <bool BF16, int MT>
 int launch_rowstream(const GemmArgs& g, hipStream_t s) {
-  hipLaunchKernelGGL((rowstream_nt_kernel<BF16, MT>), dim3((unsigned)(g.n / (kRsWaves * kRsRows))),
+  APS_LAUNCH((rowstream_nt_kernel<BF16, MT>), dim3((unsigned)(g.n / (kRsWaves * kRsRows))),
                      dim3(kRsWaves * 64), 0, s, g);
   return launch_status();
 }
@@ -711,7 +711,7 @@ int launch_weight_stream(const GemmArgs& g, int parts, int64_t k_per_part, hipSt
   do {                                                                                                            \
     e = allow_dynamic_lds((const void*)weight_stream_kernel<BF16, N>, scores_lds_bytes<N>(), 8 + (BF16 ? 3 : 0) + N - 1); \
     if (e == hipSuccess)                                                                                          \
-      hipLaunchKernelGGL((weight_stream_kernel<BF16, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g,    \
+      APS_LAUNCH((weight_stream_kernel<BF16, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g,    \
                          k_per_part);                                                                             \
   } while (0)
   if (nht == 1) APS_LAUNCH_WS(1); else if (nht == 2) APS_LAUNCH_WS(2); else APS_LAUNCH_WS(3);
@@ -893,10 +893,10 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
       const int64_t quads = m * n / 4;
       const dim3 rgrid((unsigned)((quads + 255) / 256));
       if (dtype == APS_BF16)
-        hipLaunchKernelGGL(splitk_reduce_kernel<true>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m, n,
+        APS_LAUNCH(splitk_reduce_kernel<true>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m, n,
                            parts);
       else
-        hipLaunchKernelGGL(splitk_reduce_kernel<false>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m,
+        APS_LAUNCH(splitk_reduce_kernel<false>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m,
                            n, parts);
       return launch_status();
     }
@@ -910,9 +910,9 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
     const int per_wave = (pairs + kSkWaves - 1) / kSkWaves;
     const dim3 grid((unsigned)(n / 16));
     if (dtype == APS_BF16)
-      hipLaunchKernelGGL(skinny_nt_kernel<true>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
+      APS_LAUNCH(skinny_nt_kernel<true>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
     else
-      hipLaunchKernelGGL(skinny_nt_kernel<false>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
+      APS_LAUNCH(skinny_nt_kernel<false>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
     return launch_status();
   }
   const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
@@ -945,7 +945,7 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   do {                                                                                                            \
     e = allow_dynamic_lds((const void*)gemm_nt_kernel<B, M_>, TileShape<M_>::kLdsBytes, (B ? 4 : 0) + M_ - 1);    \
     if (e == hipSuccess)                                                                                          \
-      hipLaunchKernelGGL((gemm_nt_kernel<B, M_>), grid, dim3(kThreads), TileShape<M_>::kLdsBytes, s, g);          \
+      APS_LAUNCH((gemm_nt_kernel<B, M_>), grid, dim3(kThreads), TileShape<M_>::kLdsBytes, s, g);          \
   } while (0)
 #define APS_LAUNCH_TILE_MI(B)                                                                        \
   if (mi == 1) APS_LAUNCH_TILE(B, 1); else if (mi == 2) APS_LAUNCH_TILE(B, 2);                        \
@@ -957,18 +957,18 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   int st = launch_status();
   if (st == APS_OK && g.tail_ways > 1) {
     const dim3 tgrid((unsigned)((total - g.tail_from) * 64));
-    if (dtype == APS_BF16) hipLaunchKernelGGL(tail_reduce_kernel<true>, tgrid, dim3(256), 0, s, g);
-    else hipLaunchKernelGGL(tail_reduce_kernel<false>, tgrid, dim3(256), 0, s, g);
+    if (dtype == APS_BF16) APS_LAUNCH(tail_reduce_kernel<true>, tgrid, dim3(256), 0, s, g);
+    else APS_LAUNCH(tail_reduce_kernel<false>, tgrid, dim3(256), 0, s, g);
     return launch_status();
   }
   if (st != APS_OK || splits <= 1) return st;
   const int64_t quads = (m * n + 3) / 4;
   const dim3 rgrid((unsigned)((quads + 255) / 256));
   if (dtype == APS_BF16)
-    hipLaunchKernelGGL(splitk_reduce_kernel<true>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m, n,
+    APS_LAUNCH(splitk_reduce_kernel<true>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m, n,
                        splits);
   else
-    hipLaunchKernelGGL(splitk_reduce_kernel<false>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m, n,
+    APS_LAUNCH(splitk_reduce_kernel<false>, rgrid, dim3(256), 0, s, (const float*)workspace, bias, om, m, n,
                        splits);
   return launch_status();
 }
@@ -978,7 +978,7 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
 // out[map[m]][n] = <weight[n], x[m] + (n / head_rows) * x_head_stride> + bias[n]: the value projection of the
 // absorbed attention, where the rows of head h multiply that head's context vector.  Any m: at most 8 rows
 // stream the weights through the dot kernel, more go through the MFMA kernel in tiles of 16 rows.
-int aps_internal_headwise_linear(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n,
+__attribute__((visibility("hidden"))) int aps_internal_headwise_linear(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n,
                                  int64_t k, int64_t x_stride, int64_t x_head_stride, int head_rows, int64_t w_stride,
                                  int64_t out_stride, const int64_t* out_row_map, int64_t out_rows, int dtype,
                                  hipStream_t s) {
@@ -999,9 +999,9 @@ int aps_internal_headwise_linear(const void* x, const void* weight, const void* 
   const int per_wave = (pairs + kSkWaves - 1) / kSkWaves;
   const dim3 grid((unsigned)(n / 16), (unsigned)((m + 15) / 16));
   if (dtype == APS_BF16)
-    hipLaunchKernelGGL(skinny_nt_kernel<true>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
+    APS_LAUNCH(skinny_nt_kernel<true>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
   else
-    hipLaunchKernelGGL(skinny_nt_kernel<false>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
+    APS_LAUNCH(skinny_nt_kernel<false>, grid, dim3(kSkWaves * 64), 0, s, g, per_wave);
   return launch_status();
 }
 

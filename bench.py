@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip attention / re-projection figures")
-    ap.add_argument("--extras", default="attention,prefill,metadata,write,reproject,layer,step_loop",
+    ap.add_argument("--extras", default="attention,prefill,metadata,write,reproject,layer,step_loop,cost,cpu",
                     help="comma-separated subset of the extra figures to run")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="first run the plain copy kernel on 1 GiB three times (known traffic for counter scaling)")
@@ -210,15 +210,19 @@ def main():
             extras["decode_attention_fp8" if fp8 else "decode_attention_f16"] = attention_figures(
                 torch, ops, workloads, np, dev, args.seed, fp8)
         # metadata build, GPU vs the list-based host algorithm
-        t = []
-        for _ in range(10 if "metadata" in want else 0):
-            torch.cuda.synchronize()
-            a = time.perf_counter()
-            metadata.build_from_batch(batch, dev)
-            torch.cuda.synchronize()
-            t.append((time.perf_counter() - a) * 1e6)
-        if t:
-            extras["metadata_build_us"] = median(t)
+        # from packed 0-padded int32 tables (kept up to date by the caller) and from the lists of lists the
+        # reference's scheduler hands over; both include the kernel and a final synchronize
+        for md_key, packed in (("metadata_build_us", True), ("metadata_build_us_from_lists", False)):
+            t = []
+            batch.packed_tables()
+            for _ in range(20 if "metadata" in want else 0):
+                torch.cuda.synchronize()
+                a = time.perf_counter()
+                metadata.build_from_batch(batch, dev, packed=packed)
+                torch.cuda.synchronize()
+                t.append((time.perf_counter() - a) * 1e6)
+            if t:
+                extras[md_key] = median(t)
         if not args.no_cpu and "metadata" in want:
             # the reference's approach to the same metadata: Python lists per cached token, then tensors
             from oracle.metadata import SeqRecord, build_metadata as list_build
@@ -247,6 +251,15 @@ def main():
             torch.cuda.empty_cache()
             extras["opt13b_step_loop_absorbed"] = step_loop_figures(torch, dev, args.seed, absorbed=True, weights=w13)
             del w13
+            # both flows ran the same schedule (fixed-cost clock): keep one copy, as a compact string
+            a_, b_ = extras["opt13b_step_loop"].pop("schedule"), extras["opt13b_step_loop_absorbed"].pop("schedule")
+            extras["opt13b_step_loop_same_schedule"] = a_ == b_
+        if "cost" in want:
+            extras["cost_coef"] = cost_coef_figures(torch, dev)
+        if not args.no_cpu and "cpu" in want:
+            extras["cpu_baselines"] = {
+                "config3_kv_reproject_T4096": cpu_baseline_reproject(torch),
+                "config4_decode_attention": cpu_baseline_attention(torch, np, workloads, args.seed)}
         result["extras"] = extras
 
     if not args.no_cpu:
@@ -294,36 +307,100 @@ def write_figures(torch, ops, dev, seed):
                          "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
 
 
-def step_loop_figures(torch, dev, seed, max_steps=48, absorbed=False, weights=None):
+def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile_steps=12, absorbed=False,
+                      weights=None):
     """BASELINE configs[4]: OPT-13B (random-init fp16, 40 layers) serving steps on the hybrid cache with
-    synthetic arrivals (3 req/s, CV 1) and lognormal prompt/output lengths; half of the requests hidden-cached."""
+    synthetic arrivals (3 req/s, CV 1) and lognormal prompt/output lengths; half of the requests hidden-cached.
+    The simulated clock runs on a fixed cost per step, so every data flow sees the same arrivals, admissions and
+    batches; the first `warm_steps` steps (the start-up transient: ~3 s of simulated time) are not counted.
+    Afterwards `profile_steps` decode steps run with per-phase GPU timers for the split of a step."""
     from aptserve_hip import backend, opt_model, step_loop
     cfg = opt_model.OPTConfig.opt_13b()
     N, BS = 6144, 16
+    Hd, L = cfg.hidden_size, cfg.num_hidden_layers
     w = weights if weights is not None else opt_model.random_weights(cfg, seed, dev)
     model = opt_model.HybridOPTModel(cfg, w, absorbed=absorbed)
     kv, shared = backend.allocate_caches(cfg.num_hidden_layers, N, BS, cfg.num_attention_heads,
                                          cfg.hidden_size // cfg.num_attention_heads, torch.float16, dev)
-    reqs = step_loop.synth_requests(seed, 64, rate=3.0, cv=1.0, hidden_fraction=0.5)
-    loop = step_loop.StepLoop(lambda ids, pos, md: model(ids, pos, kv, shared, md), model.next_tokens, reqs, N, BS, dev)
-    loop.run(4)                      # warm-up steps (allocator, kernels)
-    log = loop.run(max_steps)[4:]
+    reqs = step_loop.synth_requests(seed, 96, rate=3.0, cv=1.0, hidden_fraction=0.5)
+    seq_len_sum = []
+
+    def on_step(info):
+        seq_len_sum.append((sum(info["seq_lens"]), sum(l for l, h in zip(info["seq_lens"], info["use_hidden"]) if h)))
+    loop = step_loop.StepLoop(lambda ids, pos, md: model(ids, pos, kv, shared, md), model.next_tokens, reqs, N, BS, dev,
+                              step_cost=step_loop.fixed_step_cost(), on_step=on_step)
+    loop.run(warm_steps)
+    log = loop.run(warm_steps + timed_steps)[warm_steps:]
     dec = [e for e in log if e["kind"] == "decode"]
     pre = [e for e in log if e["kind"] == "prefill"]
     mean = lambda xs: sum(xs) / len(xs) if xs else None
+    # ---- split of a decode step: per-phase GPU time and what each phase achieves
+    phases, host = {}, {"metadata_ms": 0.0, "model_ms": 0.0}
+    work = {"gather_bytes": 0.0, "gemm_flops": 0.0, "attention_bytes": 0.0, "hidden_attention_bytes": 0.0}
+    n_prof = 0
+    while n_prof < profile_steps:
+        n_before = len(seq_len_sum)
+        with backend.PhaseTimes() as pt:
+            e = loop.step()
+        if e is None:
+            break
+        if e["kind"] != "decode":
+            continue
+        tot = pt.totals()
+        for k_, v_ in tot.items():
+            phases[k_] = phases.get(k_, 0.0) + v_
+        host["metadata_ms"] += e["metadata_ms"]
+        host["model_ms"] += e["model_ms"]
+        all_len, hidden_len = seq_len_sum[n_before]
+        kv_len = all_len - hidden_len
+        if absorbed:
+            work["attention_bytes"] += L * kv_len * 2 * Hd * 2
+            work["hidden_attention_bytes"] += L * 2 * hidden_len * Hd * 2
+        else:
+            work["gather_bytes"] += L * hidden_len * 2 * Hd * 2
+            work["gemm_flops"] += L * 2.0 * e["rows"] * Hd * 2 * Hd
+            work["attention_bytes"] += L * all_len * 2 * Hd * 2
+        n_prof += 1
+    split = None
+    if n_prof:
+        per = {k_: v_ / n_prof for k_, v_ in phases.items()}
+        model_ms = host["model_ms"] / n_prof
+        split = {"steps_profiled": n_prof, "metadata_ms": host["metadata_ms"] / n_prof, "model_ms": model_ms,
+                 "gpu_ms": per, "rest_ms": model_ms - sum(per.values()),
+                 "note": "projections = q / out / MLP products (weight streaming); rest = layer norms, residual "
+                         "adds, embedding, logits, launch gaps"}
+        frac = {}
+        if per.get("gather"):
+            frac["gather_hbm"] = work["gather_bytes"] / n_prof / per["gather"] / 1e6 / HBM_PEAK_GBS
+        if per.get("kv_gemm"):
+            frac["kv_gemm_mfma"] = work["gemm_flops"] / n_prof / per["kv_gemm"] / 1e9 / MFMA_F16_PEAK_TFLOPS
+        if per.get("attention"):
+            frac["attention_hbm"] = work["attention_bytes"] / n_prof / per["attention"] / 1e6 / HBM_PEAK_GBS
+        if per.get("attention_on_hidden_rows"):
+            frac["attention_on_hidden_rows_hbm"] = (work["hidden_attention_bytes"] / n_prof /
+                                                    per["attention_on_hidden_rows"] / 1e6 / HBM_PEAK_GBS)
+        if per.get("projections"):
+            stream = L * (10 if not absorbed else 12) * Hd * Hd * 2      # q, out, fc1, fc2 (and k, v when projected whole)
+            frac["projections_hbm"] = stream / per["projections"] / 1e6 / HBM_PEAK_GBS
+        split["achieved_fraction_of_peak"] = frac
     return {"workload": "OPT-13B 40 layers fp16 random-init, eager; gamma arrivals 3 req/s cv 1; prompts "
                         "lognormal(5.5,1.0) in [4,2048]; outputs lognormal(5.0,0.9) in [4,1024]; 50% hidden-cached; "
+                        "simulated clock on a fixed cost per step (12.5 ms decode, 10 ms + 20 us/token prompt); "
                         + ("hidden-cached sequences attend on their hidden rows (absorbed projections)" if absorbed
                            else "hidden-cached sequences are re-projected every layer (the reference's data flow)"),
-            "steps": len(log), "decode_steps": len(dec), "prefill_steps": len(pre),
+            "warm_steps": warm_steps, "steps": len(log), "decode_steps": len(dec), "prefill_steps": len(pre),
+            "schedule": [(e["kind"][0], e["seqs"], e["rows"]) for e in log],
+            "preemptions": loop.preemptions,
             "decode_ms_per_step": mean([e["model_ms"] for e in dec]),
             "decode_seqs_per_step": mean([e["seqs"] for e in dec]),
             "decode_rows_per_step": mean([e["rows"] for e in dec]),
             "prefill_ms_per_step": mean([e["model_ms"] for e in pre]),
             "prefill_tokens_per_step": mean([e["tokens"] for e in pre]),
             "metadata_ms_per_step": mean([e["metadata_ms"] for e in log]),
+            "decode_host_enqueue_ms_per_step": mean([e["host_enqueue_ms"] for e in dec]),
             "decode_tokens_per_s": (sum(e["seqs"] for e in dec) / (sum(e["model_ms"] + e["metadata_ms"] for e in dec) * 1e-3)
-                                    if dec else None)}
+                                    if dec else None),
+            "decode_step_split": split}
 
 
 def decode_layer_figures(torch, ops, workloads, metadata, dev, seed):
@@ -410,6 +487,82 @@ def reproject_figures(torch, ops, dev, seed):
                              "unit": "TFLOP/s", "frac": flops / ms2 / 1e9 / MFMA_F16_PEAK_TFLOPS, "traffic": None}}
             del caches
     return out
+
+
+def cost_coef_figures(torch, dev):
+    """The scheduler's profit coefficient (additional_designs/engine/aptserve_llm_engine.py:316-354: 40 layers of
+    the QKV product timed over growing token counts, slope over 16-token blocks / 5) at OPT-13B shape, measured
+    on this library's two data flows and with the reference's own recipe (F.linear, whose operands the reference
+    creates in fp32; fp16 beside it).  Every fourth point of the reference's range(1, 4101, 100)."""
+    from aptserve_hip import cost_model
+    counts = tuple(range(1, 4101, 400))
+    out = {"token_counts": list(counts), "layers": 40, "block_size": 16, "unit": "seconds per block / 5"}
+    for name, kw in (("reprojection", dict(mode="reprojection")), ("absorbed", dict(mode="absorbed")),
+                     ("reference_recipe_F_linear_fp16", dict(mode="reference_recipe")),
+                     ("reference_recipe_F_linear_fp32", dict(mode="reference_recipe", dtype=torch.float32))):
+        c, st = cost_model.get_coef(5120, 40, 40, 16, dev, token_counts=counts, **kw)
+        out[name] = c
+        out[name + "_seconds_at_%d_tokens" % counts[-1]] = st[-1][1]
+    out["reprojection_over_recipe_fp16"] = out["reprojection"] / out["reference_recipe_F_linear_fp16"]
+    out["reprojection_over_recipe_fp32"] = out["reprojection"] / out["reference_recipe_F_linear_fp32"]
+    return out
+
+
+def cpu_baseline_reproject(torch):
+    """BASELINE configs[2] on the host cores: F.linear in fp32 on fp16-rounded operands, T = 4096."""
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    Hd, T = 5120, 4096
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(T, Hd, generator=g).half().float()
+    w = (torch.randn(2 * Hd, Hd, generator=g) * 0.02).half().float()
+    b = torch.randn(2 * Hd, generator=g).half().float()
+    ts = []
+    for i in range(4):
+        a = time.perf_counter()
+        torch.nn.functional.linear(x, w, b)
+        if i >= 1:
+            ts.append(time.perf_counter() - a)
+    s = median(ts)
+    return {"value": 2.0 * T * Hd * 2 * Hd / s / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port", "host_cpus": threads,
+            "sample": "the whole T=4096 product in fp32 (torch CPU F.linear), 1 warm-up, median of 3, %.3f s" % s}
+
+
+def cpu_baseline_attention(torch, np, workloads, seed, n_seqs=16):
+    """BASELINE configs[3] on the host cores with the oracle (per-sequence fp32 softmax over K/V materialised
+    through the block table), on the first `n_seqs` sequences of the batch and a pool that holds only their
+    blocks."""
+    from oracle import attention as OA
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    H, D, BS, B = 40, 128, 16, 128
+    rng = np.random.default_rng(seed)
+    lens = workloads.lognormal_lengths(rng, B)[:n_seqs]
+    nblk = [-(-int(l) // BS) for l in lens]
+    W, total = max(nblk), sum(nblk)
+    bt = np.zeros((n_seqs, W), dtype=np.int32)
+    p = 0
+    for b_, n in enumerate(nblk):
+        bt[b_, :n] = np.arange(p, p + n)
+        p += n
+    types = (rng.random((n_seqs, W)) < 0.5).astype(np.uint8)
+    g = torch.Generator().manual_seed(seed)
+    kc, vc, wk, wv = (torch.randn(total, BS, H, D, generator=g).half() for _ in range(4))
+    q = torch.randn(n_seqs, H, D, generator=g).half()
+    sl = torch.from_numpy(lens.astype(np.int32))
+    ts = []
+    for i in range(3):
+        a = time.perf_counter()
+        OA.paged_decode_attention(q, kc, vc, torch.from_numpy(bt), sl, D ** -0.5, block_types=torch.from_numpy(types),
+                                  ws_k_cache=wk, ws_v_cache=wv)
+        if i >= 1:
+            ts.append(time.perf_counter() - a)
+    s = median(ts)
+    return {"value": n_seqs / s, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "host_cpus": threads,
+            "sample": "first %d of the 128 sequences (sum of lengths %d), fp16 cache, hybrid block types, 1 warm-up, "
+                      "median of 2, %.3f s" % (n_seqs, int(lens.sum()), s)}
 
 
 def cpu_baseline(torch, np, batch, md, cache, hs, key, value, kv_seq_idx, new_slots, step_bytes, T, Hd):

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define APS_ABI_VERSION 4
+#define APS_ABI_VERSION 5
 
 typedef void* aps_stream_t; /* a hipStream_t; NULL = the null stream */
 
@@ -316,7 +316,10 @@ int aps_varlen_prefill_attention(void* out, const void* q, const void* k,
  *   kv_dest[row]             (nullable, not in the reference) where the row's re-projected K/V go, for
  *                            aps_kv_reproject_to_cache: shared slot (hidden rows), -(private slot + 2)
  *                            (the new token of a K/V sequence), -1 for padding
- *   block_tables_out[b,:]    shared table for hidden sequences, private otherwise (:415-418)
+ *   block_tables_out[b,:]    shared table for hidden sequences, private otherwise (:415-418);
+ *   block_types_out[b,:]     (nullable, uint8 [batch, out_width] contiguous, not in the reference) 1 in every
+ *                            column of a hidden-cached sequence: the per-block source mask of
+ *                            aps_paged_decode_attention
  *   seq_start_loc / query_start_loc int32 cumulative sums with leading 0;
  *   context_lens = seq_len-1; input_positions = seq_len-1. */
 int aps_build_decode_metadata(
@@ -332,7 +335,8 @@ int aps_build_decode_metadata(
     int64_t* kv_cache_use_input, int64_t* new_token_slot, int32_t* kv_seq_lens,
     int64_t cap_rows, int64_t cap_hidden_rows,
     int64_t cap_hidden_seqs, int64_t cap_kv_seqs, int32_t* block_tables_out,
-    int64_t out_stride, int64_t out_width, int32_t* seq_start_loc,
+    int64_t out_stride, int64_t out_width, uint8_t* block_types_out,
+    int32_t* seq_start_loc,
     int32_t* query_start_loc, int32_t* context_lens, int64_t* input_positions,
     int64_t* totals, aps_stream_t stream);
 

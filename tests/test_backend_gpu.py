@@ -67,6 +67,34 @@ def test_decode_layer_matches_oracle(dev, frac, fused):
     assert torch.equal(d_sh[:, :N].cpu(), sh[:, :N])
 
 
+@pytest.mark.parametrize("fused", [True, False, "absorbed"])
+def test_decode_layer_matches_oracle_at_opt13b_width(dev, fused):
+    """The same check at 40 heads x 128 (hidden 5120): the fused flow, the reference's operator sequence and the
+    attention on hidden rows against the layer oracle, on a small mixed batch."""
+    h, d, n = 40, 128, 40
+    hd = h * d
+    sc = 0.03 * (768 / hd) ** 0.5
+    W = ((randn((3 * hd, hd), 20) * sc).half(), (randn((3 * hd,), 21) * 0.1).half(),
+         (randn((hd, hd), 22) * sc).half(), (randn((hd,), 23) * 0.1).half())
+    batch = workloads.small_decode_batch(11, 6, 90, 0.5, n)
+    ref_md = oracle_metadata(batch)
+    B = len(batch.seq_lens)
+    hs = randn((B, hd), 24)
+    kv = randn((2, n, BS, h, d), 25)
+    sh = randn((2, 2 * n, BS, h, d), 26)
+    ref_kv, ref_sh = kv.clone(), sh.clone()
+    ref = OL.opt_attention(hs, ref_kv, ref_sh, ref_md, *W, h)
+    layer = backend.HybridOPTAttention(hd, h, *(w.to(dev) for w in W), fused=bool(fused),
+                                       fuse_kv_write=fused is True, absorbed=fused == "absorbed")
+    md = metadata.build_from_batch(batch, dev)
+    d_kv, d_sh = kv.to(dev), sh.to(dev)
+    out = layer(hs.to(dev), d_kv, d_sh, md)
+    close(out, ref)
+    close(d_kv, ref_kv)
+    if fused != "absorbed":
+        close(d_sh[:, n:], ref_sh[:, n:])
+
+
 @pytest.mark.parametrize("frac", [0.4, 1.0])
 def test_fused_kv_write_is_bit_identical_to_the_operator_sequence(dev, frac):
     """Projection with the cache write in its epilogue == projection, chunk, mixed_kv_to_cache."""

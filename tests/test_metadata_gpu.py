@@ -55,6 +55,16 @@ def test_decode_metadata_small(dev, seed, frac, bs):
     assert_same(md, oracle_metadata(batch))
 
 
+@pytest.mark.parametrize("frac", [0.0, 0.5, 1.0])
+@pytest.mark.parametrize("prompt", [False, True])
+def test_packed_tables_give_the_same_metadata_as_lists(dev, frac, prompt):
+    """Block tables handed over as 0-padded int32 arrays: every field equals the oracle's, as with lists."""
+    batch = (workloads.small_prefill_batch(3, 9, 200, frac, 300) if prompt
+             else workloads.small_decode_batch(3, 11, 300, frac, 400))
+    md = metadata.build_from_batch(batch, dev, packed=True, check_totals=True)
+    assert_same(md, oracle_metadata(batch))
+
+
 @pytest.mark.parametrize("seed", range(4))
 @pytest.mark.parametrize("frac", [0.0, 0.4, 1.0])
 def test_prefill_metadata_small(dev, seed, frac):

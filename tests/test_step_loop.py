@@ -30,3 +30,35 @@ def test_cost_coefficient_regression_follows_the_reference_recipe():
     assert abs(fit_coef(tokens, secs, 16) - slope / 5) < 1e-4 * slope
     # an intercept does not change the slope much (ordinary least squares with intercept)
     assert abs(fit_coef(tokens, [s + 1e-3 for s in secs], 16) - slope / 5) < 0.05 * slope / 5
+
+
+def test_decode_growth_preempts_instead_of_running_out_of_blocks():
+    """Before a decode step the loop checks the free lists; when the running sequences need more blocks than are
+    free, the most recently admitted ones go back to the queue in recompute mode."""
+    reqs = [step_loop.Request(i, 0.0, np.zeros(16, dtype=np.int64), 64, bool(i % 2)) for i in range(4)]
+    loop = step_loop.StepLoop(None, None, [], 6, 16, "cpu")
+    for r in reqs:                      # 16 prompt tokens: one private (+ one shared) block each
+        loop.pool.grow(r, 16, 16)
+        r.generated = [1]               # the next step needs token slot 16: a second block for everybody
+        loop.running.append(r)
+    assert len(loop.pool.free_private) == 2
+    loop._make_room()
+    # K/V sequences need a private block each, hidden ones a V-plane slab (no new private block) and a shared block
+    assert [r.rid for r in loop.running] == [0, 1, 2, 3][:len(loop.running)] and loop.preemptions >= 0
+    need = sum(loop.pool.blocks_needed(r, r.seq_len, 16)[0] for r in loop.running)
+    assert need <= len(loop.pool.free_private)
+    small = step_loop.StepLoop(None, None, [], 5, 16, "cpu")
+    kv = [step_loop.Request(i, 0.0, np.zeros(16, dtype=np.int64), 64, False) for i in range(4)]
+    for r in kv:
+        small.pool.grow(r, 16, 16)
+        r.generated = [1]
+        small.running.append(r)
+    small._make_room()                  # 4 sequences want 4 blocks, 1 is free: the newest ones are preempted
+    assert small.preemptions == 2 and [r.rid for r in small.running] == [0, 1]
+    assert [r.rid for r in small.waiting] == [2, 3] and all(not r.generated and not r.block_table for r in small.waiting)
+
+
+def test_virtual_clock_is_independent_of_measured_time():
+    cost = step_loop.fixed_step_cost()
+    assert cost(dict(kind="decode", seqs=5, tokens=5)) == cost(dict(kind="decode", seqs=9, tokens=9))
+    assert cost(dict(kind="prefill", seqs=1, tokens=2000)) > cost(dict(kind="prefill", seqs=1, tokens=20))
