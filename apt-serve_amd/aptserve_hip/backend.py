@@ -232,11 +232,14 @@ class HybridOPTAttention:
     its rows straight into the cache slots (``ops.kv_reproject_to_cache``): no ``[T, 2*Hd]``
     intermediate and no ``mixed_kv_to_cache`` pass.  Results are identical again: the same
     values are rounded once and land in the same slots.
+
+    ``holder_free=True`` (with ``fuse_kv_write``) also drops the holder: the re-projection reads every cached
+    hidden row where it lies (``ops.kv_reproject_gathered``); only the newest hidden rows are stored first.
     """
 
     def __init__(self, embed_dim: int, num_heads: int, qkv_weight, qkv_bias, out_weight, out_bias, *,
                  fused: bool = True, literal: bool = False, prefill_attention: Optional[Callable] = None,
-                 fuse_kv_write: bool = True, absorbed: bool = False) -> None:
+                 fuse_kv_write: bool = True, absorbed: bool = False, holder_free: bool = True) -> None:
         self.embed_dim, self.num_heads = embed_dim, num_heads
         self.head_dim = embed_dim // num_heads
         self.scaling = self.head_dim ** -0.5
@@ -244,6 +247,7 @@ class HybridOPTAttention:
         self.out_weight, self.out_bias = out_weight, out_bias
         self.fused = fused
         self.fuse_kv_write = fuse_kv_write and fused and not literal
+        self.holder_free = holder_free and self.fuse_kv_write
         self.absorbed = absorbed and not literal
         self.attn = HybridAttentionImpl(num_heads, self.head_dim, self.scaling, literal=literal,
                                         prefill_attention=prefill_attention)
@@ -288,6 +292,24 @@ class HybridOPTAttention:
                     and kv_cache.dtype == hidden_states.dtype):
                 return self._forward_absorbed(hidden_states, kv_cache, md)
             if md.num_decode_tokens != 0:
+                if (self.holder_free and md.holder_src is not None and md.kv_dest is not None
+                        and kv_cache is not None and kv_cache.dtype == hidden_states.dtype
+                        and md.num_tot_tokens > 48):   # fewer rows: the weight-streaming kernels on a holder
+                    with phase("write"):
+                        ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
+                                            md.hidden_cache_store_tot)
+                    with phase("projections"):
+                        q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
+                    w, b = self.qkv_proj.weight, self.qkv_proj.bias
+                    s = w.shape[0] // 3
+                    with phase("kv_gemm"):
+                        ops.kv_reproject_gathered(hidden_states, kv_cache, md.holder_src, w[s:],
+                                                  None if b is None else b[s:], shared_cache[0], shared_cache[1],
+                                                  kv_cache[0], kv_cache[1], md.kv_dest)
+                    with phase("attention"):
+                        attn_output = self.attn.forward(q, None, None, kv_cache, shared_cache, md, kv_written=True)
+                    with phase("projections"):
+                        return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
                 if self.fused and md.holder_src is not None:
                     holder = torch.empty(md.num_tot_tokens, hidden_states.shape[1], device=hidden_states.device,
                                          dtype=hidden_states.dtype)

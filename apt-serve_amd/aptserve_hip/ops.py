@@ -570,6 +570,65 @@ def kv_reproject_to_cache(x, w_kv, b_kv, ws_k_cache, ws_v_cache, k_cache, v_cach
     _lib.check(st, "kv_reproject_to_cache")
 
 
+def kv_reproject_gathered(hidden_states, paged_cache, holder_src, w_kv, b_kv, ws_k_cache, ws_v_cache, k_cache,
+                          v_cache, kv_dest, workspace=None, split_k: bool = True) -> None:
+    """``kv_reproject_to_cache`` without the holder: row ``t`` of the product's left operand is read where it is
+    cached (``holder_src[t] >= 0``: that slot of ``paged_cache``; ``-(b+1)``: row ``b`` of ``hidden_states``),
+    so the sequence ``torch.zeros`` / index_put / ``cache_to_hidden`` of
+    additional_designs/model_executor/models/aptserve_opt.py:112-121 and its ``[num_tot, Hd]`` tensor disappear.
+    Rows without a source must have ``kv_dest == -1`` (the metadata builder writes them so).  Cache contents are
+    bit-identical to ``gather_hidden_rows`` + ``kv_reproject_to_cache``."""
+    dev = hidden_states.device
+    for n, t in (("hidden_states", hidden_states), ("paged_cache", paged_cache), ("w_kv", w_kv)):
+        _check_data(n, t, dev)
+    _need(hidden_states.dim() == 2 and w_kv.dim() == 2 and hidden_states.size(1) == w_kv.size(1),
+          "hidden_states [B,K] and w_kv [2*Hd,K] expected")
+    _need(hidden_states.dtype == w_kv.dtype == paged_cache.dtype and hidden_states.dtype in (torch.float16, torch.bfloat16),
+          "f16 or bf16 operands and cache expected")
+    K = hidden_states.size(1)
+    _check_paged(paged_cache, K)
+    _need(w_kv.size(0) % 2 == 0, "w_kv must stack the K and V projections")
+    Hd = w_kv.size(0) // 2
+    if b_kv is not None:
+        _check_data("b_kv", b_kv, dev)
+        _need(b_kv.dim() == 1 and b_kv.numel() == 2 * Hd and b_kv.dtype == w_kv.dtype and b_kv.is_contiguous(),
+              "b_kv must be a contiguous [2*Hd] vector of the operand dtype")
+    _check_index("holder_src", holder_src, dev)
+    _check_index("kv_dest", kv_dest, dev)
+    T = holder_src.numel()
+    _need(kv_dest.numel() == T, "one destination per row expected")
+    slots = [0, 0]
+    stride = None
+    for i, (kc, vc, nm) in enumerate(((ws_k_cache, ws_v_cache, "workspace"), (k_cache, v_cache, "private"))):
+        _need((kc is None) == (vc is None), f"{nm} K and V caches must be given together")
+        if kc is None:
+            continue
+        for c in (kc, vc):
+            _check_data(f"{nm} cache", c, dev)
+            _need(c.dim() == 4 and c.is_contiguous() and c.dtype == w_kv.dtype and c.size(2) * c.size(3) == Hd,
+                  f"{nm} caches must be contiguous [blocks, BS, H, D] of the operand dtype with H*D = Hd")
+        _need(kc.shape == vc.shape, f"{nm} K and V caches differ in shape")
+        slots[i] = kc.size(0) * kc.size(1)
+        stride = Hd
+    _need(stride is not None, "no destination cache given")
+    if T == 0:
+        return
+    lib = _lib.load()
+    need = lib.aps_linear_nt_workspace_bytes(T, 2 * Hd, K) if (split_k and T > 48) else 0
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)     # scratch is host-side plumbing
+    slot_stride = paged_cache.stride(2)
+    with torch.cuda.device(dev):
+        st = lib.aps_kv_reproject_gathered(
+            paged_cache.data_ptr(), slot_stride, paged_cache.numel() // slot_stride, hidden_states.data_ptr(),
+            hidden_states.stride(0), hidden_states.size(0), holder_src.data_ptr(), T, w_kv.data_ptr(),
+            None if b_kv is None else b_kv.data_ptr(), _ptr(ws_k_cache), _ptr(ws_v_cache), _ptr(k_cache),
+            _ptr(v_cache), kv_dest.data_ptr(), Hd, K, w_kv.stride(0), stride, slots[0], slots[1],
+            _DTYPE_CODE[w_kv.dtype], workspace.data_ptr() if need else None,
+            workspace.numel() * workspace.element_size() if need else 0, _stream(hidden_states))
+    _lib.check(st, "kv_reproject_gathered")
+
+
 # ------------------------------------------------------------------ prompt attention
 
 def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=None, max_seqlen_k=None,

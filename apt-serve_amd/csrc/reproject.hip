@@ -113,6 +113,13 @@ struct GemmArgs {
   // part p of tail tile i stores its fp32 result tile at tail_partial[(i * tail_ways + p)][256][256]
   float* tail_partial;
   int tail_from, tail_ways, tail_kt;
+  // gathered A operand (GATHER kernels only): row t of A is not a + t*lda but
+  //   row_src[t] >= 0:     slot row_src[t] of the paged cache, slot_base + row_src[t] * slot_stride_b
+  //   row_src[t] = -(b+1): row b of the step's input, alt_base + b * alt_stride_b  (b < alt_rows)
+  // anything else (and rows >= m) reads row 0 of the input: such rows must not be stored (kv_dest = -1).
+  const int64_t* row_src;
+  const char* slot_base; const char* alt_base;
+  int64_t slot_stride_b, alt_stride_b, num_slots, alt_rows;
 };
 
 // Logical tile number -> tile coordinates: groups of kGroupM tile rows, column-major inside a group, so that
@@ -127,7 +134,7 @@ __host__ __device__ __forceinline__ void tile_coords(int logical, int tiles_m, i
   pid_n = r / gsz;
 }
 
-template <bool BF16, int MI>
+template <bool BF16, int MI, bool GATHER = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_nt_kernel(
     const GemmArgs g) {
   using T = TileShape<MI>;
@@ -178,6 +185,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   const uint32_t voff_a0 = (uint32_t)(lrow * g.lda_b + lchunk0 * 16), voff_a1 = (uint32_t)(lrow * g.lda_b + lchunk1 * 16);
   const uint32_t voff_w0 = (uint32_t)(lrow * g.ldw_b + lchunk0 * 16), voff_w1 = (uint32_t)(lrow * g.ldw_b + lchunk1 * 16);
   const uint32_t grp_a = (uint32_t)(8 * g.lda_b), grp_w = (uint32_t)(8 * g.ldw_b);
+  // gathered A: this lane's row of each of the MI 8-row groups the wavefront loads, swizzled chunk included
+  const char* a_row[GATHER ? MI : 1];
+  if constexpr (GATHER) {
+#pragma unroll
+    for (int j = 0; j < MI; ++j) {
+      const int i = wave * MI + j;
+      const int64_t row = row0 + i * 8 + lrow;
+      const char* p = g.alt_base;
+      if (row < g.m) {
+        const int64_t src = g.row_src[row];
+        if (src >= 0) {
+          if (src < g.num_slots) p = g.slot_base + src * g.slot_stride_b;
+        } else if (-(src + 1) < g.alt_rows) {
+          p = g.alt_base + (-(src + 1)) * g.alt_stride_b;
+        }
+      }
+      a_row[j] = p + (((i & 1) ? lchunk1 : lchunk0) * 16);
+    }
+  }
 
   const int kt_base_ = tail_part >= 0 ? tail_part * g.tail_kt : (g.partial ? (int)blockIdx.y * g.kt_per_split : 0);
   auto issue_loads = [&](int kt) {
@@ -187,8 +213,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
     for (int j = 0; j < MI; ++j) {
       const int i = wave * MI + j;  // 8-row group of the A tile handled by this wave-wide load (8*MI groups)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(sa + i * 1024), 16,
-                                               (i & 1) ? voff_a1 : voff_a0, koff + i * grp_a, 0, 0);
+      if constexpr (GATHER)   // every lane brings the 64-bit address of its own row
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_row[j] + koff),
+                                         (__attribute__((address_space(3))) void*)(sa + i * 1024), 16, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(sa + i * 1024), 16,
+                                                 (i & 1) ? voff_a1 : voff_a0, koff + i * grp_a, 0, 0);
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -709,7 +739,7 @@ int launch_weight_stream(const GemmArgs& g, int parts, int64_t k_per_part, hipSt
   hipError_t e = hipSuccess;
 #define APS_LAUNCH_WS(N)                                                                                          \
   do {                                                                                                            \
-    e = allow_dynamic_lds((const void*)weight_stream_kernel<BF16, N>, scores_lds_bytes<N>(), 8 + (BF16 ? 3 : 0) + N - 1); \
+    e = allow_dynamic_lds((const void*)weight_stream_kernel<BF16, N>, scores_lds_bytes<N>(), 16 + (BF16 ? 3 : 0) + N - 1); \
     if (e == hipSuccess)                                                                                          \
       APS_LAUNCH((weight_stream_kernel<BF16, N>), grid, dim3(kScThreads), scores_lds_bytes<N>(), s, g,    \
                          k_per_part);                                                                             \
@@ -862,13 +892,23 @@ int64_t aps_linear_nt_workspace_bytes(int64_t m, int64_t n, int64_t k) {
   return tail_plan_of(m, n, k).bytes;
 }
 
+// Where the rows of a gathered A operand live (see GemmArgs::row_src).
+struct GatherSrc {
+  const int64_t* row_src;
+  const void* slot_base; int64_t slot_stride, num_slots;
+  const void* alt_base; int64_t alt_stride, alt_rows;
+};
+
 static int launch_gemm(const void* x, const void* weight, const void* bias, const OutMap& om, int64_t m, int64_t n,
                        int64_t k, int64_t x_stride, int64_t w_stride, int dtype, void* workspace,
-                       int64_t workspace_bytes, aps_stream_t stream) {
+                       int64_t workspace_bytes, aps_stream_t stream, const GatherSrc* gs = nullptr) {
   if (dtype != APS_F16 && dtype != APS_BF16) return APS_ERR_UNSUPPORTED;
   if (n % BN != 0 || k % BK != 0) return APS_ERR_UNSUPPORTED;
   if (x_stride < k || w_stride < k) return APS_ERR_INVALID_ARG;
   if (common_vec_bytes({addr(x), addr(weight), (uint64_t)x_stride * 2, (uint64_t)w_stride * 2}) != 16)
+    return APS_ERR_UNSUPPORTED;
+  if (gs && common_vec_bytes({addr(gs->slot_base), addr(gs->alt_base), (uint64_t)gs->slot_stride * 2,
+                              (uint64_t)gs->alt_stride * 2}) != 16)
     return APS_ERR_UNSUPPORTED;
   // one tile's rows must be addressable with 32-bit byte offsets
   if ((int64_t)BM * x_stride * 2 >= ((int64_t)1 << 31) || (int64_t)BN * w_stride * 2 >= ((int64_t)1 << 31))
@@ -881,8 +921,16 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   g.tiles_m = (int)((m + 64 * mi - 1) / (64 * mi)); g.tiles_n = (int)(n / BN);
   g.out = om;
   hipStream_t s = (hipStream_t)stream;
-  if (m <= kRsMaxRows) return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
-  if (m <= kWsMaxRows) {
+  if (gs) {   // only the tile kernel reads its A rows through a row map
+    g.a = nullptr;
+    g.row_src = gs->row_src;
+    g.slot_base = (const char*)gs->slot_base; g.alt_base = (const char*)gs->alt_base;
+    g.slot_stride_b = gs->slot_stride * 2; g.alt_stride_b = gs->alt_stride * 2;
+    g.num_slots = gs->num_slots; g.alt_rows = gs->alt_rows;
+  }
+  if (!gs && m <= kRsMaxRows)
+    return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
+  if (!gs && m <= kWsMaxRows) {
     int64_t k_per_part = 0;
     const int parts = weight_stream_parts(m, n, k, &k_per_part);
     if (parts == 1 || (workspace && workspace_bytes >= (int64_t)parts * m * n * 4 && !(addr(workspace) & 15))) {
@@ -904,7 +952,7 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
     // no workspace: the single-launch kernels below
     if (m <= 8) return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
   }
-  if (m <= kSkinnyMaxRows && n / 16 < ((int64_t)1 << 31) && x_stride * 2 * 16 < ((int64_t)1 << 31) &&
+  if (!gs && m <= kSkinnyMaxRows && n / 16 < ((int64_t)1 << 31) && x_stride * 2 * 16 < ((int64_t)1 << 31) &&
       w_stride * 2 * 16 < ((int64_t)1 << 31)) {
     const int pairs = (int)((k / 32 + 1) / 2);
     const int per_wave = (pairs + kSkWaves - 1) / kSkWaves;
@@ -919,7 +967,7 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   if (total >= ((int64_t)1 << 30)) return APS_ERR_UNSUPPORTED;
   const int64_t per_xcd = (total + kNumXcd - 1) / kNumXcd;
   int splits = 1;
-  if (workspace) {
+  if (workspace && !(gs && m <= kWsMaxRows)) {   // (the split plan of few rows belongs to the streaming kernels)
     splits = aps_linear_nt_splits(m, n, k);
     if (splits > 1 && (workspace_bytes < (int64_t)splits * m * n * 4 || (addr(workspace) & 15))) return APS_ERR_WORKSPACE;
   }
@@ -943,9 +991,16 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   hipError_t e = hipSuccess;
 #define APS_LAUNCH_TILE(B, M_)                                                                                     \
   do {                                                                                                            \
-    e = allow_dynamic_lds((const void*)gemm_nt_kernel<B, M_>, TileShape<M_>::kLdsBytes, (B ? 4 : 0) + M_ - 1);    \
-    if (e == hipSuccess)                                                                                          \
-      APS_LAUNCH((gemm_nt_kernel<B, M_>), grid, dim3(kThreads), TileShape<M_>::kLdsBytes, s, g);          \
+    if (gs) {                                                                                                     \
+      e = allow_dynamic_lds((const void*)gemm_nt_kernel<B, M_, true>, TileShape<M_>::kLdsBytes,                   \
+                            8 + (B ? 4 : 0) + M_ - 1);                                                            \
+      if (e == hipSuccess)                                                                                        \
+        APS_LAUNCH((gemm_nt_kernel<B, M_, true>), grid, dim3(kThreads), TileShape<M_>::kLdsBytes, s, g);          \
+    } else {                                                                                                      \
+      e = allow_dynamic_lds((const void*)gemm_nt_kernel<B, M_>, TileShape<M_>::kLdsBytes, (B ? 4 : 0) + M_ - 1);  \
+      if (e == hipSuccess)                                                                                        \
+        APS_LAUNCH((gemm_nt_kernel<B, M_>), grid, dim3(kThreads), TileShape<M_>::kLdsBytes, s, g);                \
+    }                                                                                                             \
   } while (0)
 #define APS_LAUNCH_TILE_MI(B)                                                                        \
   if (mi == 1) APS_LAUNCH_TILE(B, 1); else if (mi == 2) APS_LAUNCH_TILE(B, 2);                        \
@@ -1043,6 +1098,35 @@ int aps_kv_reproject_to_cache(const void* x, const void* w_kv, const void* b_kv,
   om.limit0 = ws_slots; om.limit1 = cache_slots; om.aligned16 = align == 16;
   return launch_gemm(x, w_kv, b_kv, om, m, 2 * hidden_size, k, x_stride, w_stride, dtype, workspace, workspace_bytes,
                      stream);
+}
+
+int aps_kv_reproject_gathered(const void* paged_cache, int64_t cache_slot_stride, int64_t num_cache_slots,
+                              const void* hidden_states, int64_t hidden_stride, int64_t num_inputs,
+                              const int64_t* holder_src, int64_t m, const void* w_kv, const void* b_kv,
+                              void* ws_k_cache, void* ws_v_cache, void* k_cache, void* v_cache,
+                              const int64_t* kv_dest, int64_t hidden_size, int64_t k, int64_t w_stride,
+                              int64_t slot_stride, int64_t ws_slots, int64_t cache_slots, int dtype, void* workspace,
+                              int64_t workspace_bytes, aps_stream_t stream) {
+  if (m < 0 || hidden_size <= 0 || k <= 0 || ws_slots < 0 || cache_slots < 0 || num_cache_slots < 0 || num_inputs <= 0)
+    return APS_ERR_INVALID_ARG;
+  if (m == 0) return APS_OK;
+  if (!paged_cache || !hidden_states || !holder_src || !w_kv || !kv_dest) return APS_ERR_INVALID_ARG;
+  if ((ws_slots && (!ws_k_cache || !ws_v_cache)) || (cache_slots && (!k_cache || !v_cache))) return APS_ERR_INVALID_ARG;
+  if (slot_stride < hidden_size || cache_slot_stride < k || hidden_stride < k) return APS_ERR_INVALID_ARG;
+  if (hidden_size % BN != 0) return APS_ERR_UNSUPPORTED;
+  const int align = common_vec_bytes({addr(ws_k_cache), addr(ws_v_cache), addr(k_cache), addr(v_cache),
+                                      (uint64_t)slot_stride * 2});
+  if (align < 4) return APS_ERR_UNSUPPORTED;
+  OutMap om{};
+  om.base[0] = (char*)ws_k_cache; om.base[1] = (char*)ws_v_cache;
+  om.base[2] = (char*)k_cache; om.base[3] = (char*)v_cache;
+  om.ld = slot_stride; om.n_split = hidden_size; om.map = kv_dest;
+  om.limit0 = ws_slots; om.limit1 = cache_slots; om.aligned16 = align == 16;
+  const GatherSrc gs{holder_src, paged_cache, cache_slot_stride, num_cache_slots, hidden_states, hidden_stride,
+                     num_inputs};
+  // the row pitch checks of the plain path are made on the two sources instead
+  return launch_gemm(hidden_states, w_kv, b_kv, om, m, 2 * hidden_size, k, hidden_stride, w_stride, dtype, workspace,
+                     workspace_bytes, stream, &gs);
 }
 
 }  // extern "C"

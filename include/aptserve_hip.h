@@ -410,6 +410,31 @@ int aps_kv_reproject_to_cache(
     int64_t cache_slots, int dtype, void* workspace, int64_t workspace_bytes,
     aps_stream_t stream);
 
+/* aps_kv_reproject_to_cache without the holder: the rows of the product's left
+ * operand are fetched where they are cached instead of being gathered into a
+ * contiguous [m, k] matrix first (replaces, in addition, the holder assembly
+ * model_executor/models/aptserve_opt.py:112-121: zero fill, index_put and
+ * cache_to_hidden).  Row t of the operand is
+ *   holder_src[t] >= 0       slot holder_src[t] of paged_cache (rows of
+ *                            cache_slot_stride elements, < num_cache_slots)
+ *   holder_src[t] = -(b+1)   row b of hidden_states (the step's input, rows of
+ *                            hidden_stride elements, b < num_inputs)
+ * as aps_build_decode_metadata writes it.  Any other value marks a row without
+ * a source: it is multiplied with unspecified (valid) data and must not be
+ * stored, i.e. its kv_dest must be -1 (the metadata builder guarantees that).
+ * The newest hidden rows still have to be stored into the cache by the caller
+ * (aps_hidden_to_cache); this call does not depend on that store.  Results are
+ * bit-identical to aps_gather_hidden_rows followed by aps_kv_reproject_to_cache.
+ * Everything else as for aps_kv_reproject_to_cache. */
+int aps_kv_reproject_gathered(
+    const void* paged_cache, int64_t cache_slot_stride, int64_t num_cache_slots,
+    const void* hidden_states, int64_t hidden_stride, int64_t num_inputs,
+    const int64_t* holder_src, int64_t m, const void* w_kv, const void* b_kv,
+    void* ws_k_cache, void* ws_v_cache, void* k_cache, void* v_cache,
+    const int64_t* kv_dest, int64_t hidden_size, int64_t k, int64_t w_stride,
+    int64_t slot_stride, int64_t ws_slots, int64_t cache_slots, int dtype,
+    void* workspace, int64_t workspace_bytes, aps_stream_t stream);
+
 /* Decode attention of hidden-cached sequences on their cached hidden rows, the
  * projections absorbed into the query and the output ("next" item 2 of the
  * hybrid path; replaces, for those sequences, the holder gather

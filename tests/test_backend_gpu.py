@@ -106,7 +106,33 @@ def test_fused_kv_write_is_bit_identical_to_the_operator_sequence(dev, frac):
     md = metadata.build_from_batch(batch, dev)
     res = []
     for fuse in (True, False):
-        layer = backend.HybridOPTAttention(Hd, H, *(w.to(dev) for w in W), fuse_kv_write=fuse)
+        layer = backend.HybridOPTAttention(Hd, H, *(w.to(dev) for w in W), fuse_kv_write=fuse, holder_free=False)
+        d_kv, d_sh = kv.to(dev), sh.to(dev)
+        res.append((layer(hs.to(dev), d_kv, d_sh, md).cpu(), d_kv.cpu(), d_sh.cpu()))
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("frac", [0.4, 1.0])
+@pytest.mark.parametrize("shape", [(12, 64, 150), (40, 128, 700)])
+def test_holder_free_reprojection_is_bit_identical_to_the_gathered_holder(dev, frac, shape):
+    """The re-projection that fetches cached hidden rows in place (no holder) against the flow that gathers them
+    into a holder first: same output, same cache contents, bit for bit.  The second shape (40 x 128, ~3000 rows)
+    runs the full-size tiles."""
+    h, d, max_len = shape
+    hd, n = h * d, 12 * max_len // 16
+    sc = 0.03 * (768 / hd) ** 0.5
+    W = ((randn((3 * hd, hd), 30) * sc).half(), (randn((3 * hd,), 31) * 0.1).half(),
+         (randn((hd, hd), 32) * sc).half(), (randn((hd,), 33) * 0.1).half())
+    batch = workloads.small_decode_batch(4, 10, max_len, frac, n)
+    hs = randn((len(batch.seq_lens), hd), 34)
+    kv = randn((2, n, BS, h, d), 35)
+    sh = randn((2, 2 * n, BS, h, d), 36)
+    md = metadata.build_from_batch(batch, dev)
+    assert md.num_tot_tokens > 48
+    res = []
+    for holder_free in (True, False):
+        layer = backend.HybridOPTAttention(hd, h, *(w.to(dev) for w in W), holder_free=holder_free)
         d_kv, d_sh = kv.to(dev), sh.to(dev)
         res.append((layer(hs.to(dev), d_kv, d_sh, md).cpu(), d_kv.cpu(), d_sh.cpu()))
     for a, b in zip(*res):
