@@ -72,7 +72,7 @@ def allocate_caches(num_layers: int, num_blocks: int, block_size: int, num_kv_he
 class HybridAttentionImpl:
     def __init__(self, num_heads: int, head_size: int, scale: float, num_kv_heads: Optional[int] = None,
                  alibi_slopes=None, sliding_window=None, kv_cache_dtype: str = "auto", *, literal: bool = False,
-                 prefill_attention: Optional[Callable] = None) -> None:
+                 prefill_attention: Optional[Callable] = None, k_scale: float = 1.0, v_scale: float = 1.0) -> None:
         if alibi_slopes is not None:
             raise ValueError("alibi_slopes is not supported (OPT has none)")
         if sliding_window is not None:
@@ -84,7 +84,15 @@ class HybridAttentionImpl:
                              f"Supported head sizes are: {HybridCacheBackend.get_supported_head_sizes()}.")
         self.num_heads, self.head_size, self.scale = num_heads, head_size, float(scale)
         self.num_kv_heads = num_heads
+        if kv_cache_dtype not in ("auto", "fp8", "fp8_e4m3"):
+            raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
         self.kv_cache_dtype = kv_cache_dtype
+        self.fp8 = kv_cache_dtype != "auto"
+        if self.fp8 and literal:
+            raise ValueError("the literal (mirror-writing) flow is a byte move: it has no fp8 form")
+        # per-tensor scales of an fp8-e4m3 K/V cache (K = code * k_scale); the reference has none
+        # (aptserve_flash_attn.py:311-312 asserts kv_scale == 1.0)
+        self.k_scale, self.v_scale = float(k_scale), float(v_scale)
         self.literal = literal
         self.prefill_attention = prefill_attention
 
@@ -96,7 +104,8 @@ class HybridAttentionImpl:
         ``kv_written``: the caller has already put this step's K/V into the caches
         (``ops.kv_reproject_to_cache`` in a decode step, where ``key = value = None`` is then
         allowed; ``ops.mixed_reshape_and_cache`` in a prompt step), only the attention runs."""
-        assert kv_scale == 1.0, "kv_scale is not supported"            # :312
+        assert self.fp8 or kv_scale == 1.0, "kv_scale needs an fp8 K/V cache"            # :312
+        ks, vs = self.k_scale * kv_scale, self.v_scale * kv_scale
         md = attn_metadata
         if md.num_prefills and md.max_prompt_context_len > 0:
             # the reference's prefix branch (aptserve_flash_attn.py:431-447) attends over the cache through the
@@ -127,14 +136,22 @@ class HybridAttentionImpl:
             key_cache, value_cache = kv_cache[0], kv_cache[1]
             if n_hidden == 0:                                                       # :334-345
                 ops.reshape_and_cache_flash(key, value, key_cache, value_cache, md.slot_mapping,
-                                            self.kv_cache_dtype)
+                                            self.kv_cache_dtype, ks, vs)
             elif n_prefill != 0:                                                    # :347-355, without the gather copies
                 ops.reshape_and_cache_flash(key, value, key_cache, value_cache, md.slot_mapping,
-                                            self.kv_cache_dtype, token_idx=md.kv_cache_use_tot)
+                                            self.kv_cache_dtype, ks, vs, token_idx=md.kv_cache_use_tot)
             else:
                 shared_k, shared_v = shared_cache[0], shared_cache[1]
                 mixed = md.num_tot_tokens != md.slot_mapping_shared.numel()         # :359
-                if mixed:
+                if self.fp8:
+                    # mixed_kv_to_cache is a byte move; the quantising write goes through two scatters whose
+                    # slot vectors are indexed like the rows (from kv_dest: workspace slot, or -(private slot + 2))
+                    ws_slots, private_slots = md.row_slots_by_destination()
+                    ops.reshape_and_cache_flash(key, value, shared_k, shared_v, ws_slots, self.kv_cache_dtype, ks, vs)
+                    if mixed:
+                        ops.reshape_and_cache_flash(key, value, key_cache, value_cache, private_slots,
+                                                    self.kv_cache_dtype, ks, vs)
+                elif mixed:
                     ops.mixed_kv_to_cache(key, value, key_cache, value_cache, shared_k, shared_v, md.slot_mapping,
                                           md.slot_mapping_shared, md.kv_cache_use_tot, md.hidden_cache_use_tot,
                                           skip_mirror=not self.literal)
@@ -161,15 +178,16 @@ class HybridAttentionImpl:
             if n_hidden == 0:                                                       # :451-461
                 ops.paged_decode_attention(decode_query, key_cache, value_cache, dm.block_tables,
                                            dm.seq_lens_tensor, self.scale, max_seq_len=max_len,
-                                           out=output[n_prefill:])
+                                           out=output[n_prefill:], k_scale=ks, v_scale=vs)
             elif self.literal or not mixed:                                         # :464-473
                 ops.paged_decode_attention(decode_query, shared_k, shared_v, dm.block_tables, dm.seq_lens_tensor,
-                                           self.scale, max_seq_len=max_len, out=output[n_prefill:])
+                                           self.scale, max_seq_len=max_len, out=output[n_prefill:], k_scale=ks,
+                                           v_scale=vs)
             else:
                 ops.paged_decode_attention(decode_query, key_cache, value_cache, dm.block_tables,
                                            dm.seq_lens_tensor, self.scale, block_types=dm.block_types,
                                            ws_k_cache=shared_k, ws_v_cache=shared_v, max_seq_len=max_len,
-                                           out=output[n_prefill:])
+                                           out=output[n_prefill:], k_scale=ks, v_scale=vs)
         return output.view(num_tokens, hidden_size)
 
 
@@ -239,7 +257,8 @@ class HybridOPTAttention:
 
     def __init__(self, embed_dim: int, num_heads: int, qkv_weight, qkv_bias, out_weight, out_bias, *,
                  fused: bool = True, literal: bool = False, prefill_attention: Optional[Callable] = None,
-                 fuse_kv_write: bool = True, absorbed: bool = False, holder_free: bool = True) -> None:
+                 fuse_kv_write: bool = True, absorbed: bool = False, holder_free: bool = True,
+                 kv_cache_dtype: str = "auto", k_scale: float = 1.0, v_scale: float = 1.0) -> None:
         self.embed_dim, self.num_heads = embed_dim, num_heads
         self.head_dim = embed_dim // num_heads
         self.scaling = self.head_dim ** -0.5
@@ -249,18 +268,20 @@ class HybridOPTAttention:
         self.fuse_kv_write = fuse_kv_write and fused and not literal
         self.holder_free = holder_free and self.fuse_kv_write
         self.absorbed = absorbed and not literal
-        self.attn = HybridAttentionImpl(num_heads, self.head_dim, self.scaling, literal=literal,
-                                        prefill_attention=prefill_attention)
+        self.attn = HybridAttentionImpl(num_heads, self.head_dim, self.scaling, kv_cache_dtype=kv_cache_dtype,
+                                        literal=literal, prefill_attention=prefill_attention, k_scale=k_scale,
+                                        v_scale=v_scale)
 
-    def _forward_absorbed(self, hidden_states, kv_cache, md: HybridAttentionMetadata):
+    def _forward_absorbed(self, hidden_states, kv_cache, hidden_cache, md: HybridAttentionMetadata):
         """Decode step without re-projection: hidden-cached sequences attend on their cached hidden rows
         (projection weights absorbed), K/V-cached sequences on their private cache."""
         w, b = self.qkv_proj.weight, self.qkv_proj.bias
         s = w.shape[0] // 3
         H, D = self.num_heads, self.head_dim
         # the newest hidden row of every hidden-cached sequence joins its cache first
+        a = self.attn
         with phase("write"):
-            ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
+            ops.hidden_to_cache(hidden_states, hidden_cache, md.slot_mapping, md.hidden_cache_use_input,
                                 md.hidden_cache_store_tot)
         n_kv = md.num_decode_tokens - md.num_hidden_cache_tokens
         attn_output = torch.empty_like(hidden_states)
@@ -269,41 +290,49 @@ class HybridOPTAttention:
                 qkv, _ = self.qkv_proj(hidden_states)
                 q, k, v = qkv.chunk(chunks=3, dim=-1)
             with phase("write"):
-                ops.reshape_and_cache_flash(k, v, kv_cache[0], kv_cache[1], md.new_token_slot, "auto",
-                                            token_idx=md.kv_cache_use_input)
+                ops.reshape_and_cache_flash(k, v, kv_cache[0], kv_cache[1], md.new_token_slot, a.kv_cache_dtype,
+                                            a.k_scale, a.v_scale, token_idx=md.kv_cache_use_input)
             with phase("attention"):
                 ops.paged_decode_attention(q.view(-1, H, D), kv_cache[0], kv_cache[1], md.private_block_tables,
                                            md.kv_seq_lens, self.scaling, max_seq_len=md.max_kv_seq_len or None,
-                                           out=attn_output.view(-1, H, D))
+                                           out=attn_output.view(-1, H, D), k_scale=a.k_scale, v_scale=a.v_scale)
         else:
             with phase("projections"):
                 q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
         with phase("attention_on_hidden_rows"):
-            ops.absorbed_hidden_attention(q, kv_cache, md.hidden_slots, md.hidden_seq_start,
+            ops.absorbed_hidden_attention(q, hidden_cache, md.hidden_slots, md.hidden_seq_start,
                                           md.hidden_cache_use_input, md.max_hidden_seq_len, w[s:2 * s], w[2 * s:],
                                           None if b is None else b[2 * s:], self.scaling, attn_output)
         with phase("projections"):
             return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
 
-    def forward(self, hidden_states, kv_cache, shared_cache, attn_metadata: HybridAttentionMetadata):
+    def forward(self, hidden_states, kv_cache, shared_cache, attn_metadata: HybridAttentionMetadata,
+                hidden_cache=None):
+        """``hidden_cache``: where hidden rows are cached when it is not ``kv_cache`` itself — a separate
+        ``(2, N, BS, H, D)`` tensor in the activation dtype, needed with an fp8 K/V cache (whose bytes cannot hold
+        16-bit hidden rows)."""
         md = attn_metadata
+        hc = kv_cache if hidden_cache is None else hidden_cache
+        same = kv_cache is not None and kv_cache.dtype == hidden_states.dtype      # K/V cached in the activation dtype
+        fp8 = self.attn.fp8
+        if fp8 and md.num_hidden_cache_tokens != 0 and (hidden_cache is None or hidden_cache.dtype != hidden_states.dtype):
+            raise ValueError("an fp8 K/V cache cannot hold hidden rows: pass hidden_cache in the activation dtype")
         if md.num_hidden_cache_tokens != 0:
             if (self.absorbed and md.num_decode_tokens != 0 and md.hidden_slots is not None and kv_cache is not None
-                    and kv_cache.dtype == hidden_states.dtype):
-                return self._forward_absorbed(hidden_states, kv_cache, md)
+                    and hc.dtype == hidden_states.dtype):
+                return self._forward_absorbed(hidden_states, kv_cache, hc, md)
             if md.num_decode_tokens != 0:
-                if (self.holder_free and md.holder_src is not None and md.kv_dest is not None
-                        and kv_cache is not None and kv_cache.dtype == hidden_states.dtype
+                if (self.holder_free and md.holder_src is not None and md.kv_dest is not None and same
                         and md.num_tot_tokens > 48):   # fewer rows: the weight-streaming kernels on a holder
                     with phase("write"):
-                        ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
+                        ops.hidden_to_cache(hidden_states, hc, md.slot_mapping, md.hidden_cache_use_input,
                                             md.hidden_cache_store_tot)
                     with phase("projections"):
                         q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
                     w, b = self.qkv_proj.weight, self.qkv_proj.bias
                     s = w.shape[0] // 3
                     with phase("kv_gemm"):
-                        ops.kv_reproject_gathered(hidden_states, kv_cache, md.holder_src, w[s:],
+                        ops.kv_reproject_gathered(hidden_states, hc, md.holder_src, w[s:],
                                                   None if b is None else b[s:], shared_cache[0], shared_cache[1],
                                                   kv_cache[0], kv_cache[1], md.kv_dest)
                     with phase("attention"):
@@ -314,19 +343,18 @@ class HybridOPTAttention:
                     holder = torch.empty(md.num_tot_tokens, hidden_states.shape[1], device=hidden_states.device,
                                          dtype=hidden_states.dtype)
                     with phase("gather"):
-                        ops.gather_hidden_rows(holder, hidden_states, kv_cache, md.holder_src, md.slot_mapping,
+                        ops.gather_hidden_rows(holder, hidden_states, hc, md.holder_src, md.slot_mapping,
                                                md.hidden_cache_use_input, md.hidden_cache_store_tot)
                 else:                                                               # aptserve_opt.py:108-121
-                    ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
+                    ops.hidden_to_cache(hidden_states, hc, md.slot_mapping, md.hidden_cache_use_input,
                                         md.hidden_cache_store_tot)
                     holder = torch.zeros(md.num_tot_tokens, hidden_states.shape[1], device=hidden_states.device,
                                          dtype=hidden_states.dtype)
                     holder[md.hidden_holder_upd] = hidden_states
-                    ops.cache_to_hidden(holder, kv_cache, md.slot_mapping, md.hidden_cache_use_tot)
+                    ops.cache_to_hidden(holder, hc, md.slot_mapping, md.hidden_cache_use_tot)
                 with phase("projections"):
                     q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
-                if (self.fuse_kv_write and md.kv_dest is not None and kv_cache is not None
-                        and kv_cache.dtype == holder.dtype):
+                if self.fuse_kv_write and md.kv_dest is not None and same:
                     w, b = self.qkv_proj.weight, self.qkv_proj.bias
                     s = w.shape[0] // 3
                     with phase("kv_gemm"):
@@ -339,16 +367,18 @@ class HybridOPTAttention:
                 else:
                     kv, _ = self.qkv_proj(holder, q_only=False, kv_only=True)
                     k, v = kv.chunk(chunks=2, dim=-1)
-            elif (self.fuse_kv_write and md.token_is_hidden is not None and kv_cache is not None
-                  and kv_cache.dtype == hidden_states.dtype):
+            elif self.fuse_kv_write and md.token_is_hidden is not None and kv_cache is not None and (same or fp8):
                 qkv, _ = self.qkv_proj(hidden_states)
                 q, k, v = qkv.chunk(chunks=3, dim=-1)
-                # hidden rows of hidden-cached prompts and K/V rows of the others, one launch
-                ops.mixed_reshape_and_cache(k, v, hidden_states, kv_cache, md.slot_mapping, md.token_is_hidden)
+                # hidden rows of hidden-cached prompts and K/V rows of the others, one launch (two with fp8:
+                # the byte move of the hidden rows and the quantising write of the K/V rows)
+                ops.mixed_reshape_and_cache(k, v, hidden_states, kv_cache, md.slot_mapping, md.token_is_hidden,
+                                            self.attn.kv_cache_dtype, self.attn.k_scale, self.attn.v_scale,
+                                            hidden_cache=hidden_cache)
                 attn_output = self.attn.forward(q, k, v, kv_cache, shared_cache, md, kv_written=True)
                 return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
             else:                                                                   # :125-127
-                ops.hidden_to_cache(hidden_states, kv_cache, md.slot_mapping, md.hidden_cache_use_input,
+                ops.hidden_to_cache(hidden_states, hc, md.slot_mapping, md.hidden_cache_use_input,
                                     md.hidden_cache_store_tot)
                 qkv, _ = self.qkv_proj(hidden_states)
                 q, k, v = qkv.chunk(chunks=3, dim=-1)

@@ -68,8 +68,19 @@ class HybridAttentionMetadata:
     max_kv_seq_len: int = 0
     private_block_tables: Optional[torch.Tensor] = None  # int32 [batch, W]: every sequence's private table
     max_prompt_context_len: int = 0   # longest already-cached prefix of a prompt step (0: plain prompts)
+    _row_slots: Optional[tuple] = None
     _cached_prefill_metadata: Optional["HybridAttentionMetadata"] = None
     _cached_decode_metadata: Optional["HybridAttentionMetadata"] = None
+
+    def row_slots_by_destination(self):
+        """Two slot vectors indexed like the rows of a decode step, derived from ``kv_dest`` (cached): the
+        workspace slot of every row of a hidden-cached sequence (-1 elsewhere) and the private slot of the
+        newest token of every K/V-cached sequence (-1 elsewhere) — what ``reshape_and_cache_flash`` needs to
+        send each kind of row to its cache."""
+        if self._row_slots is None:
+            d = self.kv_dest
+            self._row_slots = (torch.where(d >= 0, d, -1), torch.where(d <= -2, -(d + 2), -1))
+        return self._row_slots
 
     @property
     def prefill_metadata(self) -> Optional["HybridAttentionMetadata"]:

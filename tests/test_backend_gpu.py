@@ -188,6 +188,66 @@ def test_prefill_layer_cache_writes_and_output(dev, frac):
     assert torch.equal(d_kv2, d_kv)
 
 
+def _fp8_codes(x, scale):
+    return torch.clamp(x.float() / scale, -448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+
+
+@pytest.mark.parametrize("frac", [0.0, 0.4, 1.0])
+@pytest.mark.parametrize("absorbed", [False, True])
+def test_decode_layer_with_fp8_kv_cache_matches_oracle(dev, frac, absorbed):
+    """K/V cached as e4m3 codes with per-tensor scales, hidden rows in a separate 16-bit cache: written codes
+    are bit-exact, the output is within tolerance of the oracle (which quantises the same way)."""
+    W = weights(3)
+    ks, vs = 0.02, 0.015
+    batch = workloads.small_decode_batch(6, 9, 140, frac, N)
+    ref_md = oracle_metadata(batch)
+    hs = randn((len(batch.seq_lens), Hd), 40)
+    kv8 = _fp8_codes(randn((2, N, BS, H, D), 41), 1.0 / 60)             # codes of values around +-1/60 * 448
+    sh8 = _fp8_codes(randn((2, 2 * N, BS, H, D), 42), 1.0 / 60)
+    hcache = randn((2, N, BS, H, D), 43)
+    ref_kv, ref_sh, ref_hc = kv8.clone(), sh8.clone(), hcache.clone()
+    ref = OL.opt_attention(hs, ref_kv, ref_sh, ref_md, *W, H, kv_cache_dtype="fp8", k_scale=ks, v_scale=vs,
+                           hidden_cache=ref_hc)
+    layer = backend.HybridOPTAttention(Hd, H, *(w.to(dev) for w in W), absorbed=absorbed, kv_cache_dtype="fp8",
+                                       k_scale=ks, v_scale=vs)
+    md = metadata.build_from_batch(batch, dev)
+    d_kv, d_sh, d_hc = kv8.to(dev), sh8.to(dev), hcache.to(dev)
+    out = layer(hs.to(dev), d_kv, d_sh, md, hidden_cache=d_hc)
+    close(out, ref, tol=1.5e-2)
+    assert torch.equal(d_hc.cpu(), ref_hc)                       # hidden rows: pure copies
+    # codes written this step: the GEMM's rounding may differ by an ulp of fp16 before quantisation, which can
+    # move a code by one step; everything else must be identical
+    diff = (d_kv.cpu() != ref_kv)
+    assert diff.float().mean().item() < 1e-3
+    if absorbed:
+        assert torch.equal(d_sh.cpu(), sh8)                      # nothing is re-projected
+    else:
+        assert (d_sh.cpu() != ref_sh).float().mean().item() < 1e-3
+    if frac > 0:
+        with pytest.raises(ValueError, match="hidden_cache"):
+            layer(hs.to(dev), d_kv, d_sh, md)
+
+
+def test_prefill_layer_with_fp8_kv_cache(dev):
+    W = weights(4)
+    ks, vs = 0.03, 0.02
+    batch = workloads.small_prefill_batch(7, 5, 90, 0.5, N)
+    ref_md = oracle_metadata(batch)
+    hs = randn((ref_md["num_prefill_tokens"], Hd), 44)
+    kv8 = torch.zeros(2, N, BS, H, D, dtype=torch.uint8)
+    sh8 = torch.zeros(2, 2 * N, BS, H, D, dtype=torch.uint8)
+    hcache = randn((2, N, BS, H, D), 45)
+    ref_kv, ref_hc = kv8.clone(), hcache.clone()
+    ref = OL.opt_attention(hs, ref_kv, sh8.clone(), ref_md, *W, H, kv_cache_dtype="fp8", k_scale=ks, v_scale=vs,
+                           hidden_cache=ref_hc)
+    layer = backend.HybridOPTAttention(Hd, H, *(w.to(dev) for w in W), kv_cache_dtype="fp8", k_scale=ks, v_scale=vs)
+    d_kv, d_hc = kv8.to(dev), hcache.to(dev)
+    out = layer(hs.to(dev), d_kv, sh8.to(dev), metadata.build_from_batch(batch, dev), hidden_cache=d_hc)
+    close(out, ref)
+    assert torch.equal(d_hc.cpu(), ref_hc)
+    assert (d_kv.cpu() != ref_kv).float().mean().item() < 1e-3
+
+
 def test_decode_follows_prefill_through_the_hip_path(dev):
     """Prefill L tokens then decode token L+1 == last row of a prefill of L+1 tokens, for a
     batch mixing both cache types — the whole chain on the GPU."""
