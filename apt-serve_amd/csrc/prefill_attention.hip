@@ -188,39 +188,49 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     // ---- online softmax for this lane's query (its 32 keys here, the other 32 in lane^32)
     // Only a tile that reaches past the wavefront's first query or past the sequence needs the mask.
+    // The maximum is taken on the raw scores (the scale is positive) and the scale goes into the exponent's
+    // fused multiply-add: max, fma, exp2 and add per score, nothing else.
     const bool masked = kv0 + BKV - 1 > wave_q0 || kv0 + BKV > len;
-    float mx = m_run;
+    float mx = m_run;   // raw-score domain
+    if (masked) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int key = kv0 + t * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+          if (!(key <= my_q && key < len)) st[t][e] = -INFINITY;
+        }
+    }
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        float sc = st[t][e] * a.scale_log2;
-        if (masked) {
-          const int key = kv0 + t * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
-          if (!(key <= my_q && key < len)) sc = -INFINITY;
-        }
-        st[t][e] = sc;
-        mx = fmaxf(mx, sc);
-      }
+      for (int e = 0; e < 16; ++e) mx = fmaxf(mx, st[t][e]);
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_use = (mx == -INFINITY) ? 0.f : mx;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+    const float neg_m = -m_use * a.scale_log2;
     float psum = 0.f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const float p = __builtin_amdgcn_exp2f(st[t][e] - m_use);
+        const float p = __builtin_amdgcn_exp2f(fmaf(st[t][e], a.scale_log2, neg_m));
         st[t][e] = p;
         psum += p;
       }
     psum += __shfl_xor(psum, 32);
-    l_run = l_run * alpha + psum;
+    // the running maximum rarely moves after the first tiles: rescale O only when some query of the wavefront
+    // needs it (a wave-uniform branch)
+    const bool moved = mx != m_run;
+    if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * a.scale_log2);
+      l_run *= alpha;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
+    }
+    l_run += psum;
     m_run = mx;
-#pragma unroll
-    for (int t = 0; t < DT; ++t)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) o[t][e] *= alpha;
     // ---- O^T += V^T P^T : four k-steps of 16 keys; P^T fragment = 8 consecutive result registers
 #pragma unroll
     for (int t32 = 0; t32 < 2; ++t32)
