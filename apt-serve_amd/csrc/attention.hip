@@ -167,7 +167,10 @@ __device__ __forceinline__ void decode_wave(const AttnArgs& a, int seq, int head
   // query fragment of this lane: fp32, or, when the cache holds the query's 16-bit type, the packed pairs as
   // they are (v_dot2 multiplies the 16-bit pairs exactly and accumulates in fp32: 4 instructions per 8 elements
   // instead of 8 conversions and 8 FMAs, and half the registers)
-  constexpr bool kDot2 = (KV == KV_F16 && QT == APS_F16) || (KV == KV_BF16 && QT == APS_BF16);
+  // An fp8 cache under an fp16 query takes the same route: e4m3 values are exact in fp16, and one conversion
+  // yields a packed pair.
+  constexpr bool kDot2 = (KV == KV_F16 && QT == APS_F16) || (KV == KV_BF16 && QT == APS_BF16) ||
+                         (KV == KV_FP8 && QT == APS_F16);
   float qf[kDot2 ? 1 : EPL];
   uint32_t qpk[kDot2 ? EPL / 2 : 1];
   {
@@ -242,7 +245,16 @@ __device__ __forceinline__ void decode_wave(const AttnArgs& a, int seq, int head
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
       float d = 0.f;
-      if constexpr (kDot2) {
+      if constexpr (kDot2 && KV == KV_FP8) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int kw = (int)kq[g][i];
+          d = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(kw, 1.0f, false),
+                                     __builtin_bit_cast(half2_t, qpk[2 * i]), d, false);
+          d = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(kw, 1.0f, true),
+                                     __builtin_bit_cast(half2_t, qpk[2 * i + 1]), d, false);
+        }
+      } else if constexpr (kDot2) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const uint32_t kw = kq[g][i], qw = qpk[i];
@@ -375,7 +387,8 @@ constexpr int kRankInKernelMax = 512;  // up to this many sequences a workgroup 
 // Workgroup rows are dealt out longest sequence first (list scheduling): the order comes from seq_order, or,
 // for batches up to kRankInKernelMax, from ranking the lengths in LDS at the start of every workgroup.
 template <int QT, int KV, int D, int HPW, int DEPTH, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void paged_decode_group_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(64 * WAVES)
+void paged_decode_group_kernel(const AttnArgs a) {
   constexpr int EPL = Unpack<KV>::EPL, LPT = D / EPL, LPR = LPT * HPW;
   __shared__ int s_arrived, s_seq;
   __shared__ int s_len[kRankInKernelMax];

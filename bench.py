@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip attention / re-projection figures")
-    ap.add_argument("--extras", default="attention,prefill,metadata,write,reproject,layer,step_loop,cost,cpu",
+    ap.add_argument("--extras", default="literal,attention,prefill,metadata,write,ceilings,reproject,layer,step_loop,cost,cpu",
                     help="comma-separated subset of the extra figures to run")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="first run the plain copy kernel on 1 GiB three times (known traffic for counter scaling)")
@@ -204,6 +204,26 @@ def main():
     want = set() if args.no_extras else set(x for x in args.extras.split(",") if x)
     if want:
         extras = {}
+        if "literal" in want:
+            # the reference's own operator sequence through the drop-in module (no caller change): hidden_to_cache,
+            # torch.zeros holder, index_put of the newest rows, cache_to_hidden over every cached row
+            # (additional_designs/model_executor/models/aptserve_opt.py:108-121)
+            import mixed_cache_ops
+
+            def literal():
+                mixed_cache_ops.hidden_to_cache(hs, cache, md.slot_mapping, md.hidden_cache_use_input,
+                                                md.hidden_cache_store_tot)
+                h = torch.zeros(T, Hd, dtype=torch.float16, device=dev)
+                h[md.hidden_holder_upd] = hs
+                mixed_cache_ops.cache_to_hidden(h, cache, md.slot_mapping, md.hidden_cache_use_tot)
+            ms_lit = median(event_times(torch, literal, 20))
+            extras["gather_literal_dropin_sequence"] = {
+                "workload": "same batch: mixed_cache_ops.hidden_to_cache + torch.zeros + index_put + "
+                            "mixed_cache_ops.cache_to_hidden (the reference's calls, unchanged)",
+                "ms": ms_lit, "algorithmic_bytes": gather_alg,
+                "roofline": {"bound": "hbm", "achieved": gather_alg / ms_lit / 1e6, "peak": HBM_PEAK_GBS,
+                             "unit": "GB/s", "frac": gather_alg / ms_lit / 1e6 / HBM_PEAK_GBS, "traffic": None},
+                "note": "the zero fill writes the holder a second time: 1.5x the HBM traffic of the fused launch"}
         del holder
         for fp8 in ((False, True) if "attention" in want else ()):
             torch.cuda.empty_cache()
@@ -236,6 +256,10 @@ def main():
             extras["metadata_build_us_cpu_list_algorithm"] = median(t)
         if "write" in want:
             extras["kv_write_prefill_16384"] = write_figures(torch, ops, dev, args.seed)
+            extras["kv_write_prefill_16384_block_contiguous"] = write_figures(torch, ops, dev, args.seed, True)
+        if "ceilings" in want:
+            extras["stream_ceilings"] = stream_ceiling_figures(torch, dev)
+            torch.cuda.empty_cache()
         if "prefill" in want:
             extras["prompt_attention_4x2048"] = prompt_attention_figures(torch, ops, dev, args.seed)
         if "reproject" in want:
@@ -287,24 +311,50 @@ def prompt_attention_figures(torch, ops, dev, seed):
                          "traffic": None}}
 
 
-def write_figures(torch, ops, dev, seed):
+def write_figures(torch, ops, dev, seed, block_contiguous=False):
     """The cache write at a shape that can saturate HBM: a 16 384-token prompt batch at OPT-13B width,
     K and V rows scattered by slot_mapping (the decode-step write of configs[1] moves 7.9 MB and is
-    bounded by launch latency, not bandwidth)."""
+    bounded by launch latency, not bandwidth).  Slots: a random permutation of all slots (every 10 KiB row lands
+    somewhere else: the worst case), or, `block_contiguous`, what a prompt step produces: consecutive tokens fill
+    the 16 slots of a block, blocks in random order."""
     H, D, BS, T = 40, 128, 16, 16384
     N = T // BS + 64
     g = torch.Generator(device=dev).manual_seed(seed)
     kv = torch.randn(T, 2 * H * D, generator=g, device=dev).half()
     key, value = (x.view(T, H, D) for x in kv.chunk(2, -1))
     cache = torch.zeros(2, N, BS, H, D, dtype=torch.float16, device=dev)
-    slots = torch.randperm(N * BS, generator=g, device=dev)[:T].contiguous()
+    if block_contiguous:
+        blocks = torch.randperm(N, generator=g, device=dev)[:T // BS]
+        slots = (blocks[:, None] * BS + torch.arange(BS, device=dev)[None, :]).reshape(-1).contiguous()
+    else:
+        slots = torch.randperm(N * BS, generator=g, device=dev)[:T].contiguous()
     ms = median(event_times(torch, lambda: ops.reshape_and_cache_flash(key, value, cache[0], cache[1], slots, "auto"), 30))
     nbytes = T * 2 * (2 * H * D * 2)
     gbs = nbytes / ms / 1e6
-    return {"workload": "K/V cache write of 16384 tokens, 40x128 f16, random slots", "ms": ms,
+    return {"workload": "K/V cache write of 16384 tokens, 40x128 f16, " +
+                        ("slots block by block (a prompt step), blocks in random order" if block_contiguous
+                         else "random slots"), "ms": ms,
             "algorithmic_bytes": nbytes,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
+
+
+def stream_ceiling_figures(torch, dev):
+    """What plain streams sustain on this GPU (aps_stream_probe, 2 GiB of random fp16, one 16-byte chunk per
+    thread, workgroups in address order): the ceilings the row movers and the attention are held against."""
+    from aptserve_hip import _lib
+    lib = _lib.load()
+    nb = 2 << 30
+    a = torch.empty(nb // 2, dtype=torch.float16, device=dev)
+    for i in range(0, nb // 2, 1 << 28):
+        a[i:i + (1 << 28)] = torch.randn(1 << 28, device=dev).half()
+    b = torch.empty_like(a)
+    st = torch.cuda.current_stream().cuda_stream
+    out = {"bytes": nb, "data": "random fp16 N(0,1)"}
+    for mode, name, mult in ((0, "copy", 2), (1, "read", 1), (2, "fill", 1)):
+        ms = median(event_times(torch, lambda: lib.aps_stream_probe(mode, 1, b.data_ptr(), a.data_ptr(), nb, st), 20))
+        out[name] = {"ms": ms, "GB/s": mult * nb / ms / 1e6, "frac_of_hbm_peak": mult * nb / ms / 1e6 / HBM_PEAK_GBS}
+    return out
 
 
 def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile_steps=12, absorbed=False,
