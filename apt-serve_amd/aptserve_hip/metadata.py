@@ -16,6 +16,7 @@ that scales with the number of cached tokens.
 
 from __future__ import annotations
 
+import contextlib
 import itertools
 from dataclasses import dataclass
 from typing import List, Optional, Sequence
@@ -152,10 +153,10 @@ class _Staging:
             self.bufs[i] = torch.empty(max(n, 4096), dtype=torch.int32, pin_memory=True)
         return i, self.bufs[i][:n]
 
-    def upload(self, i: int, host: torch.Tensor, device) -> torch.Tensor:
+    def upload(self, i: int, host: torch.Tensor, device, stream) -> torch.Tensor:
         dev = host.to(device, non_blocking=True)
         ev = torch.cuda.Event()
-        ev.record(torch.cuda.current_stream(device))
+        ev.record(stream)
         self.events[i] = ev
         return dev
 
@@ -231,33 +232,53 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
     if np.any(lens <= 0):
         raise ValueError("sequence lengths must be positive")
     need_blocks = -(-lens // block_size)
+    max_len = int(lens.max())
+    # packed arrays carry no lengths of their own: every table is as long as its sequence needs, so the checks
+    # and reductions the ragged lists need fall away
+    arrays = isinstance(block_tables, np.ndarray)
     bt_lens = _table_lens(block_tables, need_blocks)
-    have_tables = bool(bt_lens.any())
-    W = int(bt_lens.max()) if have_tables else 0
-    if have_tables and np.any(bt_lens < need_blocks):
-        b = int(np.nonzero(bt_lens < need_blocks)[0][0])
-        raise ValueError(f"sequence {b}: private block table shorter than ceil(seq_len/block_size)")
+    if arrays:
+        have_tables = block_tables.shape[1] > 0
+        W = -(-max_len // block_size) if have_tables else 0
+    else:
+        have_tables = bool(bt_lens.any())
+        W = int(bt_lens.max()) if have_tables else 0
+        if have_tables and np.any(bt_lens < need_blocks):
+            b = int(np.nonzero(bt_lens < need_blocks)[0][0])
+            raise ValueError(f"sequence {b}: private block table shorter than ceil(seq_len/block_size)")
     lib = _lib.load()
     i64 = dict(dtype=torch.int64, device=device)
     i32 = dict(dtype=torch.int32, device=device)
+    stream = torch.cuda.current_stream(device)
+    on_device = (contextlib.nullcontext() if torch.cuda.current_device() == stream.device_index
+                 else torch.cuda.device(device))
 
     if not is_prompt:
         if len(block_tables_4_shared) != B:
             raise ValueError("block_tables_4_shared must have one entry per sequence")
-        bts_lens = _table_lens(block_tables_4_shared, need_blocks * hid) * hid   # K/V-cached sequences: ignored
-        if have_tables and np.any(bts_lens[hid] < need_blocks[hid]):
-            b = int(np.nonzero(hid & (bts_lens < need_blocks))[0][0])
-            raise ValueError(f"sequence {b}: shared block table shorter than ceil(seq_len/block_size)")
-        n_hs = int(hid.sum())
+        n_hs = int(np.count_nonzero(hid))
         n_kv = B - n_hs
-        n_hr = int(lens[hid].sum())
+        hid_lens = lens[hid]
+        n_hr = int(hid_lens.sum())
         num_tot = n_hr + n_kv
-        Ws = int(bts_lens.max()) if (have_tables and n_hs) else 0
-        # width of the table handed to attention: the longest *selected* table (:601-609)
-        Wo = int(np.where(hid, bts_lens, bt_lens).max()) if have_tables else 0
+        max_hid_len = int(hid_lens.max()) if n_hs else 0
+        shared_arrays = isinstance(block_tables_4_shared, np.ndarray)
+        if arrays and shared_arrays:
+            bts_lens = None
+            if have_tables and n_hs and -(-max_hid_len // block_size) > block_tables_4_shared.shape[1]:
+                raise ValueError("packed block table narrower than ceil(seq_len/block_size)")
+            Ws = -(-max_hid_len // block_size) if (have_tables and n_hs) else 0
+            Wo = W            # both tables are exactly as long as their sequences need
+        else:
+            bts_lens = _table_lens(block_tables_4_shared, need_blocks * hid) * hid   # K/V-cached sequences: ignored
+            if have_tables and np.any(bts_lens[hid] < need_blocks[hid]):
+                b = int(np.nonzero(hid & (bts_lens < need_blocks))[0][0])
+                raise ValueError(f"sequence {b}: shared block table shorter than ceil(seq_len/block_size)")
+            Ws = int(bts_lens.max()) if (have_tables and n_hs) else 0
+            # width of the table handed to attention: the longest *selected* table (:601-609)
+            Wo = int(np.where(hid, bts_lens, bt_lens).max()) if have_tables else 0
         # one packed upload: lens | flags | private tables | shared tables
-        arrays = isinstance(block_tables, np.ndarray) and (Ws == 0 or isinstance(block_tables_4_shared, np.ndarray))
-        stg, slot, host = _stage(device, 2 * B + B * W + B * Ws, zero=not arrays)
+        stg, slot, host = _stage(device, 2 * B + B * W + B * Ws, zero=not (arrays and (Ws == 0 or shared_arrays)))
         hv = host.numpy()
         hv[:B] = lens
         hv[B:2 * B] = hid
@@ -269,7 +290,7 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
             else:
                 shared = [t if h else () for t, h in zip(block_tables_4_shared, hid)]
                 _pack_tables(shared, bts_lens, hv[2 * B + B * W:].reshape(B, Ws))
-        packed = stg.upload(slot, host, device)
+        packed = stg.upload(slot, host, device, stream)
         d_lens, d_hid = packed[:B], packed[B:2 * B]
         d_bt = packed[2 * B:2 * B + B * W].view(B, W)
         d_bts = packed[2 * B + B * W:].view(B, Ws)
@@ -287,7 +308,7 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
         bt_out = bt_out.view(B, Wo)
         # per-block source for the hybrid attention: every block of a hidden sequence is a workspace block
         block_types = types32.view(torch.uint8)[:B * Wo].view(B, Wo) if n_types else None
-        with torch.cuda.device(device):
+        with on_device:
             st = lib.aps_build_decode_metadata(
                 d_lens.data_ptr(), d_hid.data_ptr(), d_bt.data_ptr() if W else None, W, W,
                 d_bts.data_ptr() if Ws else None, Ws, Ws, B, block_size, slot_mapping.data_ptr(),
@@ -300,7 +321,7 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
                 bt_out.data_ptr() if Wo else None, Wo, Wo,
                 None if block_types is None else block_types.data_ptr(), seq_start.data_ptr(),
                 query_start.data_ptr(), ctx.data_ptr(), positions.data_ptr(), totals.data_ptr(),
-                torch.cuda.current_stream(device).cuda_stream)
+                stream.cuda_stream)
         _lib.check(st, "build_decode_metadata")
         if check_totals:
             got = totals.tolist()
@@ -312,10 +333,10 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
             hidden_cache_use_tot=use_tot, kv_cache_use_tot=kv_use, hidden_cache_use_input=use_input,
             hidden_cache_store_tot=store_tot, hidden_holder_upd=upd, hidden_holder_pull=pull,
             seq_lens=lens.tolist(), seq_lens_tensor=d_lens, max_query_len=1, max_prefill_seq_len=0,
-            max_decode_seq_len=int(lens.max()), query_start_loc=query_start, seq_start_loc=seq_start,
+            max_decode_seq_len=max_len, query_start_loc=query_start, seq_start_loc=seq_start,
             context_lens_tensor=ctx, block_tables=bt_out, use_cuda_graph=False, input_positions=positions,
             block_types=block_types, holder_src=holder_src, kv_dest=kv_dest, hidden_slots=hidden_slots,
-            hidden_seq_start=hidden_seq_start, max_hidden_seq_len=int(lens[hid].max()) if n_hs else 0,
+            hidden_seq_start=hidden_seq_start, max_hidden_seq_len=max_hid_len,
             kv_cache_use_input=kv_use_input, new_token_slot=new_token_slot, kv_seq_lens=kv_seq_lens,
             max_kv_seq_len=int(lens[~hid].max()) if n_kv else 0, private_block_tables=d_bt)
 
@@ -334,7 +355,7 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
     hv[2 * B:3 * B] = ctxs
     if W:
         _pack_tables(block_tables, bt_lens, hv[3 * B:].reshape(B, W))
-    packed = stg.upload(slot, host, device)
+    packed = stg.upload(slot, host, device, stream)
     d_lens, d_hid, d_ctx_in = packed[:B], packed[B:2 * B], packed[2 * B:3 * B]
     d_bt = packed[3 * B:].view(B, W)
     sizes64 = [n_tok, n_tok, n_ht, n_kt, 4]
@@ -344,13 +365,13 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
     buf32 = torch.empty(sum(sizes32), **i32)
     seq_start, query_start, ctx = torch.split(buf32, sizes32)
     token_is_hidden = torch.empty(n_tok, dtype=torch.uint8, device=device)
-    with torch.cuda.device(device):
+    with on_device:
         st = lib.aps_build_prefill_metadata(
             d_lens.data_ptr(), d_ctx_in.data_ptr(), d_hid.data_ptr(), d_bt.data_ptr() if W else None, W, W, B,
             block_size, slot_mapping.data_ptr(), positions.data_ptr(), use_input.data_ptr() if n_ht else None,
             kv_use.data_ptr() if n_kt else None, token_is_hidden.data_ptr(), n_tok, n_ht, n_kt,
             seq_start.data_ptr(), query_start.data_ptr(),
-            ctx.data_ptr(), totals.data_ptr(), torch.cuda.current_stream(device).cuda_stream)
+            ctx.data_ptr(), totals.data_ptr(), stream.cuda_stream)
     _lib.check(st, "build_prefill_metadata")
     if check_totals:
         got = totals.tolist()
