@@ -8,6 +8,7 @@ HIP library these functions raise.
 
 from __future__ import annotations
 
+import contextlib
 from typing import Optional
 
 import torch
@@ -29,8 +30,22 @@ if hasattr(torch, "float8_e4m3fn"):
     _DTYPE_CODE[torch.float8_e4m3fn] = APS_FP8_E4M3
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    """Raw handle of torch's current stream on the tensor's device."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index)
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+_NO_SWITCH = contextlib.nullcontext()
+
+
+def _on(dev):
+    """Context that makes ``dev`` the current device for a launch; free when it already is."""
+    return _NO_SWITCH if torch.cuda.current_device() == dev.index else torch.cuda.device(dev)
 
 
 def _need(cond: bool, msg: str) -> None:
@@ -38,18 +53,26 @@ def _need(cond: bool, msg: str) -> None:
         raise ValueError(msg)
 
 
+# The two checks below run several times per operator call: the conditions are tested first and the message
+# (device and dtype names are slow to format) is only built for the one that failed.
 def _check_data(name: str, t: torch.Tensor, dev) -> None:
+    if (isinstance(t, torch.Tensor) and t.is_cuda and t.device == dev
+            and (t.dim() == 0 or t.stride(-1) == 1 or t.size(-1) <= 1)):
+        return
     _need(isinstance(t, torch.Tensor), f"{name} must be a tensor")
     _need(t.is_cuda, f"{name} must live on the GPU")
     _need(t.device == dev, f"{name} is on {t.device}, expected {dev}")
-    _need(t.dim() == 0 or t.stride(-1) == 1 or t.size(-1) <= 1, f"{name}: innermost dimension must be contiguous")
+    raise ValueError(f"{name}: innermost dimension must be contiguous")
 
 
 def _check_index(name: str, t: torch.Tensor, dev, dtype=torch.int64) -> None:
+    if (isinstance(t, torch.Tensor) and t.dtype == dtype and t.is_cuda and t.device == dev and t.dim() == 1
+            and (t.numel() <= 1 or t.stride(0) == 1)):
+        return
     _need(isinstance(t, torch.Tensor), f"{name} must be a tensor")
     _need(t.dtype == dtype, f"{name} must be {dtype}, got {t.dtype}")
     _need(t.is_cuda and t.device == dev, f"{name} must live on {dev}")
-    _need(t.dim() == 1 and (t.numel() <= 1 or t.stride(0) == 1), f"{name} must be a contiguous vector")
+    raise ValueError(f"{name} must be a contiguous vector")
 
 
 def _check_paged(paged_cache: torch.Tensor, width: int) -> None:
@@ -77,7 +100,7 @@ def hidden_to_cache(hidden, paged_cache, slot_mapping, src_idx, target_slot_idx)
         _check_index(n, t, dev)
     _need(src_idx.numel() == target_slot_idx.numel(), "src_idx and target_slot_idx lengths differ")
     slot_stride = paged_cache.stride(2)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().aps_hidden_to_cache(
             hidden.data_ptr(), paged_cache.data_ptr(), _ptr(slot_mapping), _ptr(src_idx), _ptr(target_slot_idx),
             src_idx.numel(), hidden.size(1), hidden.stride(0), slot_stride, paged_cache.numel() // slot_stride,
@@ -96,7 +119,7 @@ def cache_to_hidden(hidden, paged_cache, slot_mapping, dst_idx) -> None:
     _check_index("slot_mapping", slot_mapping, dev)
     _check_index("dst_idx", dst_idx, dev)
     slot_stride = paged_cache.stride(2)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().aps_cache_to_hidden(
             hidden.data_ptr(), paged_cache.data_ptr(), _ptr(slot_mapping), _ptr(dst_idx), dst_idx.numel(),
             hidden.size(1), hidden.stride(0), slot_stride, paged_cache.numel() // slot_stride, hidden.size(0),
@@ -126,7 +149,7 @@ def hybrid_decode_gather(holder, hidden_states, paged_cache, slot_mapping, hidde
     _need(slot_mapping.numel() == holder.size(0), "slot_mapping must have one entry per holder row")
     _need(hidden_cache_use_input.numel() == hidden_cache_store_tot.numel(), "store index lengths differ")
     slot_stride = paged_cache.stride(2)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().aps_hybrid_decode_gather(
             holder.data_ptr(), hidden_states.data_ptr(), paged_cache.data_ptr(), _ptr(slot_mapping),
             _ptr(hidden_holder_upd), hidden_holder_upd.numel(), _ptr(hidden_holder_pull),
@@ -155,7 +178,7 @@ def gather_hidden_rows(holder, hidden_states, paged_cache, holder_src, slot_mapp
     _need(slot_mapping.numel() == holder.size(0), "slot_mapping must have one entry per holder row")
     _need(hidden_cache_use_input.numel() == hidden_cache_store_tot.numel(), "store index lengths differ")
     slot_stride = paged_cache.stride(2)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().aps_gather_hidden_rows(
             holder.data_ptr(), hidden_states.data_ptr(), paged_cache.data_ptr(), _ptr(holder_src), holder.size(0),
             _ptr(slot_mapping), _ptr(hidden_cache_use_input), _ptr(hidden_cache_store_tot),
@@ -219,7 +242,7 @@ def reshape_and_cache_flash(key, value, key_cache, value_cache, slot_mapping, kv
         n = slot_mapping.numel()
         _need(n <= key.size(0) and n <= value.size(0), "slot_mapping longer than key/value")
         num_tokens = n
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().aps_reshape_and_cache_flash(
             key.data_ptr(), value.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), _ptr(slot_mapping),
             _ptr(token_idx), n, num_tokens, heads, head_size, key_cache.size(1), key.stride(0), value.stride(0),
@@ -289,7 +312,7 @@ def mixed_reshape_and_cache(key, value, hidden, kv_cache, slot_mapping, is_hidde
         hidden_stride = hcache.stride(2)
         hidden_slots = hcache.numel() // hidden_stride
     cache_code = _DTYPE_CODE[kv_cache.dtype] if key is not None else _DTYPE_CODE[src_dtype]
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().aps_mixed_reshape_and_cache(
             _ptr(key), _ptr(value), _ptr(hidden), kv_cache[0].data_ptr(), kv_cache[1].data_ptr(),
             None if hidden is None else hcache.data_ptr(), _ptr(slot_mapping), _ptr(is_hidden), T, heads, head_size, bs,
@@ -334,7 +357,7 @@ def mixed_kv_to_cache(key, value, k_cache, v_cache, shared_k_cache, shared_v_cac
         num_tot = min(num_tot, slot_mapping.numel())
     n_hidden = slot_mapping_shared.numel()
     flags = (MIXED_LITERAL_MODULO if literal_modulo else 0) | (MIXED_SKIP_MIRROR if skip_mirror else 0)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().aps_mixed_kv_to_cache(
             key.data_ptr(), value.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), shared_k_cache.data_ptr(),
             shared_v_cache.data_ptr(), _ptr(slot_mapping), _ptr(slot_mapping_shared), _ptr(kv_cache_use_tot),
@@ -424,7 +447,7 @@ def paged_decode_attention(q, k_cache, v_cache, block_tables, seq_lens, softmax_
     if partition_size <= 0:
         partition_size = lib.aps_decode_attention_partition_size(B, H, max(max_seq_len, 1), BS)
     if static_scratch:
-        with torch.cuda.device(dev):
+        with _on(dev):
             st = lib.aps_paged_decode_attention_static(
                 out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                 None if block_types is None else ws_k_cache.data_ptr(),
@@ -441,7 +464,7 @@ def paged_decode_attention(q, k_cache, v_cache, block_tables, seq_lens, softmax_
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     ws_ptr = workspace.data_ptr() if (need and workspace is not None) else None
     ws_bytes = workspace.numel() * workspace.element_size() if (need and workspace is not None) else 0
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = lib.aps_paged_decode_attention(
             out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
             None if block_types is None else ws_k_cache.data_ptr(),
@@ -504,7 +527,7 @@ def linear_nt(x, weight, bias=None, out=None, out_row_map=None, workspace=None, 
     if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)     # scratch is host-side plumbing
     ws_ptr = workspace.data_ptr() if need else None
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = lib.aps_linear_nt(
             x.data_ptr() if M else None, weight.data_ptr(), None if bias is None else bias.data_ptr(),
             out.data_ptr() if out.numel() else None, M, N, K, x.stride(0), weight.stride(0), out.stride(0),
@@ -561,7 +584,7 @@ def kv_reproject_to_cache(x, w_kv, b_kv, ws_k_cache, ws_v_cache, k_cache, v_cach
     need = lib.aps_linear_nt_workspace_bytes(T, 2 * Hd, K) if split_k else 0
     if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)     # scratch is host-side plumbing
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = lib.aps_kv_reproject_to_cache(
             x.data_ptr() if T else None, w_kv.data_ptr(), None if b_kv is None else b_kv.data_ptr(),
             _ptr(ws_k_cache), _ptr(ws_v_cache), _ptr(k_cache), _ptr(v_cache), _ptr(kv_dest), T, Hd, K, x.stride(0),
@@ -618,7 +641,7 @@ def kv_reproject_gathered(hidden_states, paged_cache, holder_src, w_kv, b_kv, ws
     if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)     # scratch is host-side plumbing
     slot_stride = paged_cache.stride(2)
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = lib.aps_kv_reproject_gathered(
             paged_cache.data_ptr(), slot_stride, paged_cache.numel() // slot_stride, hidden_states.data_ptr(),
             hidden_states.stride(0), hidden_states.size(0), holder_src.data_ptr(), T, w_kv.data_ptr(),
@@ -663,7 +686,7 @@ def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_se
         _check_data("out", out, dev)
         _need(out.shape == q.shape and out.dtype == q.dtype and out.stride(2) == 1 and out.stride(1) == D,
               "out must look like q")
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().aps_varlen_prefill_attention(
             out.data_ptr() if T else None, q.data_ptr() if T else None, k.data_ptr() if T else None,
             v.data_ptr() if T else None, _ptr(cu_seqlens_q), n_seq if T else 0, T, max_len, H, D, q.stride(0),
@@ -716,7 +739,7 @@ def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, se
     need = lib.aps_absorbed_attention_workspace_bytes(n_seqs, int(max_len), heads, head_size)
     if workspace is None or workspace.numel() * workspace.element_size() < need:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)      # scratch is host-side plumbing
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = lib.aps_absorbed_attention(
             q.data_ptr(), q.stride(0), seq_rows.data_ptr(), q.size(0), paged_cache.data_ptr(), paged_cache.stride(2),
             paged_cache.numel() // paged_cache.stride(2), hidden_slots.data_ptr(), hidden_seq_start.data_ptr(),
@@ -752,7 +775,7 @@ def copy_blocks(kv_caches, src_to_dsts, kinds=None) -> None:
         return
     bases = torch.tensor([c.data_ptr() for c in kv_caches], dtype=torch.int64).to(dev)
     _, N, BS, H, D = c0.shape
-    with torch.cuda.device(dev):
+    with _on(dev):
         st = _lib.load().aps_copy_cache_blocks(bases.data_ptr(), len(kv_caches), src_to_dsts.data_ptr(), _ptr(kinds), n,
                                                N, BS, H * D, c0.element_size(), _stream(c0))
     _lib.check(st, "copy_blocks")
