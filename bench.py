@@ -180,7 +180,8 @@ def main():
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     step_gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
     gather_ms = sum(a.elapsed_time(b) for a, b in gather_events) / len(gather_events)
-    # the gather launch also carries the B newest rows (upd) and the hidden stores; count only what 8(d) counts
+    # the gather launch also carries the B newest rows (upd) and the hidden stores; count only the rows
+    # gathered and the hidden stores, read once and written once
     gather_alg = gather_bytes + n_hidden_seqs * 2 * (Hd * 2)
     achieved = gather_alg / gather_ms / 1e6
 
