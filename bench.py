@@ -355,6 +355,15 @@ def stream_ceiling_figures(torch, dev):
     for mode, name, mult in ((0, "copy", 2), (1, "read", 1), (2, "fill", 1)):
         ms = median(event_times(torch, lambda: lib.aps_stream_probe(mode, 1, b.data_ptr(), a.data_ptr(), nb, st), 20))
         out[name] = {"ms": ms, "GB/s": mult * nb / ms / 1e6, "frac_of_hbm_peak": mult * nb / ms / 1e6 / HBM_PEAK_GBS}
+    # the same probes at the sizes of the smaller workloads: a launch's ramp-up and tail weigh more there
+    small = 16384 * 2 * 5120 * 2       # the K/V write of 16384 tokens: this many bytes read, as many written
+    ms = median(event_times(torch, lambda: lib.aps_stream_probe(0, 1, b.data_ptr(), a.data_ptr(), small, st), 20))
+    out["copy_of_kv_write_size"] = {"bytes_each_way": small, "ms": ms, "GB/s": 2 * small / ms / 1e6,
+                                    "frac_of_hbm_peak": 2 * small / ms / 1e6 / HBM_PEAK_GBS}
+    half = 885903360                   # the fp8 cache of config 4 (what its attention reads)
+    for name, n in (("read_of_fp8_attention_size", half), ("read_of_f16_attention_size", 2 * half)):
+        ms = median(event_times(torch, lambda: lib.aps_stream_probe(1, 1, b.data_ptr(), a.data_ptr(), n, st), 20))
+        out[name] = {"bytes": n, "ms": ms, "GB/s": n / ms / 1e6, "frac_of_hbm_peak": n / ms / 1e6 / HBM_PEAK_GBS}
     return out
 
 
