@@ -65,6 +65,28 @@ def test_packed_tables_give_the_same_metadata_as_lists(dev, frac, prompt):
     assert_same(md, oracle_metadata(batch))
 
 
+def test_packed_tables_wider_than_needed_and_too_narrow(dev):
+    """Packed tables may be wider than the longest sequence needs (a runner keeps them at a fixed width): the
+    extra columns are ignored.  Tables narrower than ceil(seq_len / block_size) are refused, the private one
+    and the shared one alike; mixing a packed private table with ragged shared lists works."""
+    batch = workloads.small_decode_batch(5, 11, 300, 0.5, 400)
+    ref = oracle_metadata(batch)
+    bt, bts = batch.packed_tables()
+    lens, hid = np.asarray(batch.seq_lens), np.asarray(batch.use_hidden, dtype=bool)
+    pad = lambda a: np.concatenate([a, np.full((a.shape[0], 7), 12345, dtype=a.dtype)], axis=1)
+    md = metadata.build_metadata(False, lens, hid, pad(bt), pad(bts), batch.block_size, dev, check_totals=True)
+    assert_same(md, ref)
+    md = metadata.build_metadata(False, lens, hid, bt, batch.block_tables_4_shared, batch.block_size, dev,
+                                 check_totals=True)
+    assert_same(md, ref)
+    need = int(-(-lens.max() // batch.block_size))
+    with pytest.raises(ValueError):
+        metadata.build_metadata(False, lens, hid, bt[:, :need - 1], bts, batch.block_size, dev)
+    need_h = int(-(-lens[hid].max() // batch.block_size))
+    with pytest.raises(ValueError):
+        metadata.build_metadata(False, lens, hid, bt, bts[:, :need_h - 1], batch.block_size, dev)
+
+
 @pytest.mark.parametrize("seed", range(4))
 @pytest.mark.parametrize("frac", [0.0, 0.4, 1.0])
 def test_prefill_metadata_small(dev, seed, frac):

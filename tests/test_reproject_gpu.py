@@ -196,6 +196,57 @@ def test_kv_reproject_into_cache_slots(dev, T, dtype):
                                   torch.from_numpy(dest).to(dev))
 
 
+@pytest.mark.parametrize("T", [60, 300, 1100])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_kv_reproject_reading_cached_rows_in_place(dev, T, dtype):
+    """``kv_reproject_gathered`` takes row t of its left operand from a slot of the paged cache or from a row
+    of the step's hidden states (aptserve_opt.py:112-121 assembles them in a holder first): the caches must end
+    up bit-identical to the holder assembled on the host and pushed through ``kv_reproject_to_cache``, rows whose
+    source does not exist (destination -1) must leave no trace, and every other slot keeps its content."""
+    H, D, BS, nblk, B = 4, 64, 16, 40, 9
+    Hd = H * D
+    rng = np.random.default_rng(100 + T)
+    paged = randn((2, nblk, BS, H, D), 5, dtype)
+    hs = randn((B, Hd), 6, dtype)
+    w = (randn((2 * Hd, Hd), 7) * 0.05).to(dtype)
+    b = randn((2 * Hd,), 8, dtype)
+    n_slots = 2 * nblk * BS
+    src = rng.integers(0, n_slots, T).astype(np.int64)
+    from_input = rng.random(T) < 0.15
+    src[from_input] = -(rng.integers(0, B, from_input.sum()) + 1)
+    ws_slots, priv_slots = 2 * nblk * BS, nblk * BS
+    dest = rng.permutation(ws_slots)[:T].astype(np.int64)
+    to_priv = rng.random(T) < 0.25
+    dest[to_priv] = -(rng.permutation(priv_slots)[:to_priv.sum()] + 2)
+    bad = rng.choice(T, size=3, replace=False)
+    src[bad[0]], src[bad[1]], src[bad[2]] = n_slots + 7, -(B + 3), -(2 ** 40)      # no such slot / row
+    dest[bad] = -1
+    flat = paged.view(n_slots, Hd)
+    holder = torch.zeros(T, Hd, dtype=dtype)
+    for t in range(T):
+        if t in bad:
+            continue
+        holder[t] = flat[src[t]] if src[t] >= 0 else hs[-(src[t] + 1)]
+    shapes = (2 * nblk, 2 * nblk, nblk, nblk)
+    want = [torch.full((n, BS, H, D), 3.0, dtype=dtype, device=dev) for n in shapes]
+    ops.kv_reproject_to_cache(holder.to(dev), w.to(dev), b.to(dev), *want, torch.from_numpy(dest).to(dev))
+    got = [torch.full((n, BS, H, D), 3.0, dtype=dtype, device=dev) for n in shapes]
+    ops.kv_reproject_gathered(hs.to(dev), paged.to(dev), torch.from_numpy(src).to(dev), w.to(dev), b.to(dev), *got,
+                              torch.from_numpy(dest).to(dev))
+    for g_, w_ in zip(got, want):
+        assert torch.equal(g_, w_)
+    # against the oracle's product, not only against the other HIP flow
+    ref = OR._linear_fp32(holder, w, b)
+    t = int(np.nonzero(dest >= 0)[0][0])
+    check(torch.cat([got[0].view(-1, Hd)[dest[t]], got[1].view(-1, Hd)[dest[t]]]).cpu()[None], ref[t][None], dtype)
+    with pytest.raises(ValueError):      # one destination per source row
+        ops.kv_reproject_gathered(hs.to(dev), paged.to(dev), torch.from_numpy(src).to(dev), w.to(dev), b.to(dev),
+                                  *got, torch.from_numpy(dest[:-1]).to(dev))
+    with pytest.raises(ValueError):      # the cache must hold the operand dtype
+        ops.kv_reproject_gathered(hs.to(dev), paged.float().to(dev), torch.from_numpy(src).to(dev), w.to(dev),
+                                  b.to(dev), *got, torch.from_numpy(dest).to(dev))
+
+
 def test_unsupported_shapes_raise(dev):
     x = torch.zeros(4, 64, dtype=torch.float16, device=dev)
     with pytest.raises(RuntimeError):
