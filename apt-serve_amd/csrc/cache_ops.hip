@@ -2,11 +2,11 @@
 //
 // Every operator here moves whole rows (a hidden vector, or the K or V vector
 // of one token) between a dense tensor and slots of a paged cache.  They share
-// one kernel shape, row_mover: every thread resolves the row descriptor
-// (source pointer, destination pointer) of the 16-byte chunk it owns and moves
-// that chunk with one non-temporal 128-bit load and store.  A row of OPT-13B is
-// 10 KiB = ten 1 KiB wavefront-wide transactions, so loads and stores are
-// fully coalesced; index loads of the lanes of one row hit the same address.
+// one kernel shape, row_mover: a wavefront owns one 1 KiB segment of a row (or
+// two), resolves the row descriptor (source pointer, destination pointer) once
+// with scalar index loads and every lane moves its 16-byte chunk with one
+// non-temporal 128-bit load and store.  A row of OPT-13B is 10 KiB = ten such
+// segments, so loads and stores are fully coalesced.
 #include <hip/hip_fp16.h>
 #include <hip/hip_bf16.h>
 
