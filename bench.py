@@ -275,10 +275,14 @@ def main():
             extras["opt13b_step_loop"] = step_loop_figures(torch, dev, args.seed, weights=w13)
             torch.cuda.empty_cache()
             extras["opt13b_step_loop_absorbed"] = step_loop_figures(torch, dev, args.seed, absorbed=True, weights=w13)
+            torch.cuda.empty_cache()
+            extras["opt13b_step_loop_reference_sequence"] = step_loop_figures(
+                torch, dev, args.seed, weights=w13, reference_sequence=True, profile_steps=0)
             del w13
-            # both flows ran the same schedule (fixed-cost clock): keep one copy, as a compact string
+            # all flows ran the same schedule (fixed-cost clock): keep no copy, only the comparison
             a_, b_ = extras["opt13b_step_loop"].pop("schedule"), extras["opt13b_step_loop_absorbed"].pop("schedule")
-            extras["opt13b_step_loop_same_schedule"] = a_ == b_
+            c_ = extras["opt13b_step_loop_reference_sequence"].pop("schedule")
+            extras["opt13b_step_loop_same_schedule"] = a_ == b_ == c_
         if "cost" in want:
             extras["cost_coef"] = cost_coef_figures(torch, dev)
         if not args.no_cpu and "cpu" in want:
@@ -368,7 +372,7 @@ def stream_ceiling_figures(torch, dev):
 
 
 def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile_steps=12, absorbed=False,
-                      weights=None):
+                      weights=None, reference_sequence=False):
     """BASELINE configs[4]: OPT-13B (random-init fp16, 40 layers) serving steps on the hybrid cache with
     synthetic arrivals (3 req/s, CV 1) and lognormal prompt/output lengths; half of the requests hidden-cached.
     The simulated clock runs on a fixed cost per step, so every data flow sees the same arrivals, admissions and
@@ -379,7 +383,11 @@ def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile
     N, BS = 6144, 16
     Hd, L = cfg.hidden_size, cfg.num_hidden_layers
     w = weights if weights is not None else opt_model.random_weights(cfg, seed, dev)
-    model = opt_model.HybridOPTModel(cfg, w, absorbed=absorbed)
+    # reference_sequence: the reference's own operator calls, one for one (hidden_to_cache, zero-filled holder,
+    # index_put, cache_to_hidden, kv-only projection, chunk, mixed_kv_to_cache with the mirror writes, attention of
+    # every sequence over the shared cache: aptserve_opt.py:108-124, aptserve_flash_attn.py:359-373,464-473)
+    flow_kw = dict(literal=True, fused=False) if reference_sequence else dict(absorbed=absorbed)
+    model = opt_model.HybridOPTModel(cfg, w, **flow_kw)
     kv, shared = backend.allocate_caches(cfg.num_hidden_layers, N, BS, cfg.num_attention_heads,
                                          cfg.hidden_size // cfg.num_attention_heads, torch.float16, dev)
     reqs = step_loop.synth_requests(seed, 96, rate=3.0, cv=1.0, hidden_fraction=0.5)
@@ -446,8 +454,11 @@ def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile
     return {"workload": "OPT-13B 40 layers fp16 random-init, eager; gamma arrivals 3 req/s cv 1; prompts "
                         "lognormal(5.5,1.0) in [4,2048]; outputs lognormal(5.0,0.9) in [4,1024]; 50% hidden-cached; "
                         "simulated clock on a fixed cost per step (12.5 ms decode, 10 ms + 20 us/token prompt); "
-                        + ("hidden-cached sequences attend on their hidden rows (absorbed projections)" if absorbed
-                           else "hidden-cached sequences are re-projected every layer (the reference's data flow)"),
+                        + ("the reference's operator sequence, call for call, on this library's kernels"
+                           if reference_sequence else
+                           "hidden-cached sequences attend on their hidden rows (absorbed projections)" if absorbed
+                           else "hidden-cached sequences are re-projected every layer (the reference's data flow, "
+                                "fused: in-place A rows, cache write in the GEMM epilogue, per-block source select)"),
             "warm_steps": warm_steps, "steps": len(log), "decode_steps": len(dec), "prefill_steps": len(pre),
             "schedule": [(e["kind"][0], e["seqs"], e["rows"]) for e in log],
             "preemptions": loop.preemptions,
@@ -486,12 +497,19 @@ def decode_layer_figures(torch, ops, workloads, metadata, dev, seed):
     res = {"workload": "decoder self-attention layer, OPT-13B 40x128, decode batch 256 (128 K/V + 128 hidden), "
                        "%d cached hidden rows" % int(md.hidden_slots.numel())}
     outs = {}
-    for name, kw in (("reprojection_ms", dict()), ("absorbed_ms", dict(absorbed=True))):
+    # reference_sequence: the reference's operator calls one for one on this library's kernels (zero-filled
+    # holder, index_put, cache_to_hidden, kv-only projection, chunk, mixed_kv_to_cache with the mirror writes)
+    for name, kw in (("reprojection_ms", dict()), ("absorbed_ms", dict(absorbed=True)),
+                     ("reference_sequence_ms", dict(literal=True, fused=False))):
         layer = backend.HybridOPTAttention(Hd, H, qkv_w, qkv_b, out_w, out_b, **kw)
         outs[name] = layer(hs, kv, shared, md)
         res[name] = median(event_times(torch, lambda: layer(hs, kv, shared, md), 10))
+        if name == "reference_sequence_ms":
+            del outs[name]
+            torch.cuda.empty_cache()
     res["max_abs_difference"] = (outs["reprojection_ms"].float() - outs["absorbed_ms"].float()).abs().max().item()
     res["speedup"] = res["reprojection_ms"] / res["absorbed_ms"]
+    res["reference_sequence_over_reprojection"] = res["reference_sequence_ms"] / res["reprojection_ms"]
     # the attention on hidden rows alone (query image, scores, softmax, weighted sum, value projection)
     q = torch.randn(len(batch.seq_lens), Hd, generator=g, device=dev).half()
     out = torch.empty_like(q)
