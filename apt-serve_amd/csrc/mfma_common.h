@@ -15,8 +15,11 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 typedef float float4v __attribute__((ext_vector_type(4)));
 
+// Buffer descriptor over [p, p + bytes): loads past the end return zeros and touch no memory.  For an operand of
+// `rows` rows `stride` bytes apart of which `row_bytes` are valid, bytes is (rows - 1) * stride + row_bytes, not
+// rows * stride: the last row of a strided view (a column slice of a wider tensor) ends where its storage ends.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
-  const uint32_t n = bytes > 0xffffffffll ? 0xffffffffu : (uint32_t)bytes;
+  const uint32_t n = bytes <= 0 ? 0u : (bytes > 0xffffffffll ? 0xffffffffu : (uint32_t)bytes);
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, n, 0x00020000);
 }
 

@@ -176,8 +176,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
   // ---- global -> LDS DMA addressing
   const int64_t row0 = (int64_t)pid_m * TBM, col0 = (int64_t)pid_n * BN;
-  const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(g.a + row0 * g.lda_b, (g.m - row0) * g.lda_b);
-  const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(g.w + col0 * g.ldw_b, (g.n - col0) * g.ldw_b);
+  const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(g.a + row0 * g.lda_b, (g.m - row0 - 1) * g.lda_b + g.k * 2);
+  const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(g.w + col0 * g.ldw_b, (g.n - col0 - 1) * g.ldw_b + g.k * 2);
   const int lrow = lane >> 3;  // row within the 8-row group of a wave-wide load
   // (row >> 1) % 8 of row 8*i + lane/8 is 4*(i&1) + lane/16: two swizzles, for even and odd groups
   const int lchunk0 = (lane & 7) ^ ((lane >> 4) & 7);
@@ -411,9 +411,9 @@ __global__ __launch_bounds__(kSkWaves * 64) void skinny_nt_kernel(const GemmArgs
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int64_t n0 = (int64_t)blockIdx.x * 16;
   const int64_t m0 = (int64_t)blockIdx.y * 16;  // 16 activation rows per workgroup row
-  const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(g.w + n0 * g.ldw_b, (g.n - n0) * g.ldw_b);
+  const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(g.w + n0 * g.ldw_b, (g.n - n0 - 1) * g.ldw_b + g.k * 2);
   const int64_t x_head_b = g.head_rows ? (n0 / g.head_rows) * g.x_head_stride_b : 0;
-  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(g.a + m0 * g.lda_b + x_head_b, (g.m - m0) * g.lda_b - x_head_b);
+  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(g.a + m0 * g.lda_b + x_head_b, (g.m - m0 - 1) * g.lda_b + g.k * 2);
   const int row = lane & 15, kg = lane >> 4;
   const uint32_t voff_w0 = (uint32_t)((lane >> 3) * g.ldw_b + (lane & 7) * 16);  // rows >= n: out of bounds, zero
   const uint32_t voff_w1 = voff_w0 + (uint32_t)(8 * g.ldw_b);
@@ -552,7 +552,7 @@ __global__ __launch_bounds__(kRsWaves * 64) void rowstream_nt_kernel(const GemmA
   const char* wrow = g.w + n_first * g.ldw_b + lane * 16;
   const int64_t x_head_b =
       g.head_rows ? (((int64_t)blockIdx.x * kRsWaves * kRsRows) / g.head_rows) * g.x_head_stride_b : 0;
-  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(g.a + x_head_b, g.m * g.lda_b - x_head_b);
+  const __amdgpu_buffer_rsrc_t rsrc_x = make_rsrc(g.a + x_head_b, (g.m - 1) * g.lda_b + g.k * 2);
   float acc[kRsRows][MT];
 #pragma unroll
   for (int i = 0; i < kRsRows; ++i)

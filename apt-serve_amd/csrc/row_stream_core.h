@@ -48,7 +48,8 @@ __device__ __forceinline__ void stream_rows_times_image(const char* rowp0, const
   const int src_odd = (8 * (c & 7) + g4 + 4 * (1 - upper)) * 4;
 
   // image: piece p = (row p / 64, chunk p % 64); thread tid moves pieces tid + j*threads.  Rows past the last
-  // one and k past the end of K re-read a valid address and are replaced by zeros.
+  // one and k past the end of K read the first 16 bytes of the image instead (the one address that is valid
+  // whatever the row count, the row length and the row stride are) and are replaced by zeros.
   const char* qsrc[kPerThread];
   bool qok[kPerThread];
   uint32_t qdst[kPerThread];
@@ -64,9 +65,9 @@ __device__ __forceinline__ void stream_rows_times_image(const char* rowp0, const
   auto fetch_q = [&](int chunk, u32x4(&q)[kPerThread]) {
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) {
-      int64_t off = (int64_t)chunk * (kScChunk * 2);
-      if (off + ((tid + j * kScThreads) & 63) * 16 >= k_bytes) off = 0;   // short last chunk: any valid address
-      q[j] = *(const u32x4*)(qsrc[j] + off);
+      const int64_t off = (int64_t)chunk * (kScChunk * 2);
+      const bool in_k = off + ((tid + j * kScThreads) & 63) * 16 < k_bytes;   // a short last chunk ends early
+      q[j] = *(const u32x4*)(in_k ? qsrc[j] + off : q_base);
     }
   };
   auto store_q = [&](int buf, int chunk, const u32x4(&q)[kPerThread]) {

@@ -247,6 +247,25 @@ def test_kv_reproject_reading_cached_rows_in_place(dev, T, dtype):
                                   b.to(dev), *got, torch.from_numpy(dest).to(dev))
 
 
+@pytest.mark.parametrize("M,N,K,split_k", [(5, 768, 1216, False),     # row-streaming kernel, K not a multiple of its 512-element pieces
+                                          (9, 256, 256, True),       # weight streaming, K shorter than one 512-element chunk
+                                          (12, 512, 192, False),     # 16-row kernel, odd number of 32-wide steps
+                                          (3, 512, 256, True), (48, 1280, 1344, True), (100, 2048, 384, False)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_activations_that_end_where_their_storage_ends(dev, M, N, K, split_k, dtype):
+    """x is the right half of a [M, 2K] tensor: row stride 2K, and the last row ends exactly where the storage
+    ends.  No kernel may read past a row's K elements there (the loads that cover a partial piece of K, or rows
+    past M, must be masked by the buffer bounds or redirected), and the product must not change."""
+    xs = randn((M, 2 * K), M + K, dtype)
+    w = (randn((N, K), 2) * 0.05).to(dtype)
+    b = randn((N,), 3, dtype)
+    ref = OR._linear_fp32(xs[:, K:], w, b)
+    out = ops.linear_nt(xs.to(dev)[:, K:], w.to(dev), b.to(dev), split_k=split_k)
+    check(out, ref, dtype)
+    out2 = ops.linear_nt(xs[:, K:].contiguous().to(dev), w.to(dev), b.to(dev), split_k=split_k)
+    assert torch.equal(out, out2)
+
+
 def test_unsupported_shapes_raise(dev):
     x = torch.zeros(4, 64, dtype=torch.float16, device=dev)
     with pytest.raises(RuntimeError):
