@@ -77,6 +77,8 @@ def _kv_rows(cache: torch.Tensor) -> torch.Tensor:
 def _store_rows(cache, slots, src) -> None:
     keep = slots >= 0
     s = slots[keep]
+    if s.numel() == 0:          # every slot is padding: nothing is stored
+        return
     bs = cache.size(1)
     _kv_rows(cache).index_put_((s // bs, s % bs), src[keep].reshape(int(keep.sum()), -1))
 

@@ -196,6 +196,15 @@ def test_reshape_and_cache_flash_closed_form():
     assert bits_equal(kc, kref) and bits_equal(vc, vref)
 
 
+def test_reshape_and_cache_flash_with_only_padding_slots_stores_nothing():
+    """Every slot is the padding value -1 (a step whose tokens all belong elsewhere): the caches stay as they are."""
+    key, value = randn((3, 2, 4), 0), randn((3, 2, 4), 1)
+    kc, vc = sentinel_cache((2, 16, 2, 4)), sentinel_cache((2, 16, 2, 4), seed=2)
+    k0, v0 = kc.clone(), vc.clone()
+    cache_ops.reshape_and_cache_flash(key, value, kc, vc, t64([-1, -1, -1]), "auto")
+    assert bits_equal(kc, k0) and bits_equal(vc, v0)
+
+
 def test_holder_assembly_equals_rows_by_definition():
     H, D, N, BS = 2, 4, 24, 16
     b, md = small_decode(4, 0.5, batch=6, max_len=40)
