@@ -600,7 +600,8 @@ def kv_reproject_gathered(hidden_states, paged_cache, holder_src, w_kv, b_kv, ws
     so the sequence ``torch.zeros`` / index_put / ``cache_to_hidden`` of
     additional_designs/model_executor/models/aptserve_opt.py:112-121 and its ``[num_tot, Hd]`` tensor disappear.
     Rows without a source must have ``kv_dest == -1`` (the metadata builder writes them so).  Cache contents are
-    bit-identical to ``gather_hidden_rows`` + ``kv_reproject_to_cache``."""
+    bit-identical to ``gather_hidden_rows`` + ``kv_reproject_to_cache`` for more than 48 rows (the same tile
+    kernel); with fewer rows that flow runs the weight-streaming kernels, which add in another order."""
     dev = hidden_states.device
     for n, t in (("hidden_states", hidden_states), ("paged_cache", paged_cache), ("w_kv", w_kv)):
         _check_data(n, t, dev)
