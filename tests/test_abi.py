@@ -1,7 +1,11 @@
 """The C-ABI library loads and exports every symbol the public header declares."""
 import ctypes
+import os
 import re
+import shutil
 import subprocess
+
+import pytest
 
 from aptserve_hip import _lib
 
@@ -98,3 +102,36 @@ def test_absorbed_attention_workspace_planning_is_host_only():
             assert f(n, 2048, heads, d) > prev
             prev = f(n, 2048, heads, d)
     assert f(0, 100, 40, 128) == 0 and f(4, 0, 40, 128) == 0
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None, reason="needs a C compiler")
+def test_header_binds_from_plain_c(tmp_path):
+    """A C99 program that includes the header, links the library and calls entry points that need no GPU: what
+    a cgo / JNI / FFI binding of the reference's maintainers would do first."""
+    src = tmp_path / "bind.c"
+    src.write_text(r"""
+#include <stdio.h>
+#include <string.h>
+#include "aptserve_hip.h"
+int main(void) {
+  if (aps_abi_version() != APS_ABI_VERSION) return 1;
+  if (strcmp(aps_status_string(APS_OK), "ok") != 0) return 2;
+  /* argument errors are reported as negative statuses before anything is launched */
+  if (aps_hidden_to_cache(NULL, NULL, NULL, NULL, NULL, -1, 0, 0, 0, 0, 0, 0, 0, NULL) >= 0) return 3;
+  if (aps_linear_nt_workspace_bytes(5, 5120, 5120) <= 0) return 4;      /* a decode step's projection splits K */
+  if (aps_decode_attention_workspace_bytes(4, 40, 128, 8192, 512) <= 0) return 5;   /* 16 partitions: flat path */
+  printf("abi %d static scratch %d bytes\n", aps_abi_version(), (int)APS_STATIC_SCRATCH_BYTES);
+  return 0;
+}
+""")
+    exe = tmp_path / "bind"
+    libdir = str(_lib.LIB_PATH.parent)
+    rocm = "/opt/rocm/lib"
+    cmd = ["gcc", "-std=c99", "-Wall", "-Werror", "-I", str(_lib.HEADER.parent), str(src), "-o", str(exe), "-L", libdir,
+           "-l:" + _lib.LIB_PATH.name, "-Wl,-rpath," + libdir, "-Wl,-rpath," + rocm, "-Wl,-rpath-link," + rocm]
+    built = subprocess.run(cmd, capture_output=True, text=True)
+    assert built.returncode == 0, built.stderr
+    env = dict(os.environ, LD_LIBRARY_PATH=os.pathsep.join(filter(None, [rocm, os.environ.get("LD_LIBRARY_PATH")])))
+    ran = subprocess.run([str(exe)], capture_output=True, text=True, env=env)
+    assert ran.returncode == 0, (ran.returncode, ran.stdout, ran.stderr)
+    assert ran.stdout.startswith("abi ")
