@@ -175,6 +175,9 @@ class StepLoop:
             if not self.running:
                 if not self.waiting:
                     return None
+                if self.waiting[0].arrival <= self.now:  # it has arrived, nothing else holds blocks, and it still
+                    raise RuntimeError(                  # does not fit: waiting longer would change nothing
+                        "the block pool cannot hold a single sequence of this length")
                 self.now = self.waiting[0].arrival      # idle until the next arrival
                 return self.step()
             self._make_room()

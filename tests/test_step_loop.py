@@ -62,3 +62,13 @@ def test_virtual_clock_is_independent_of_measured_time():
     cost = step_loop.fixed_step_cost()
     assert cost(dict(kind="decode", seqs=5, tokens=5)) == cost(dict(kind="decode", seqs=9, tokens=9))
     assert cost(dict(kind="prefill", seqs=1, tokens=2000)) > cost(dict(kind="prefill", seqs=1, tokens=20))
+
+
+def test_a_prompt_that_can_never_fit_raises_instead_of_waiting_forever():
+    """Nothing runs, the head of the queue has arrived and the empty pool still cannot take it: the loop says so
+    (it used to call itself again, with an unchanged clock, until the interpreter's recursion limit)."""
+    import pytest
+    big = step_loop.Request(0, 0.0, np.zeros(16 * 40, dtype=np.int64), 8, False)
+    loop = step_loop.StepLoop(None, None, [big], 24, 16, "cpu")
+    with pytest.raises(RuntimeError, match="cannot hold a single sequence"):
+        loop.step()
