@@ -228,51 +228,56 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
   };
 
-  // ---- LDS -> register fragment addressing (row = base + lane%32, chunk = 2*ks + lane/32, swizzled)
-  const int frow = lane & 31, fhalf = lane >> 5;
+  // ---- LDS -> register fragment addressing.  v_mfma_f32_16x16x32: lane l holds row (or weight row) l%16 and
+  // the 8 elements k = 8*(l/16) .. +7 of a 32-wide k-step, i.e. chunk 4*ks + l/16 of the row, swizzled.  The 16
+  // lanes the LDS serves per cycle read 16 consecutive rows at one chunk: 16 different 16-byte bank groups.
+  const int frow = lane & 15, fq = lane >> 4;
   const uint32_t a_row_off = (uint32_t)((wm * WM + frow) * (BK * 2));
   const uint32_t w_row_off = (uint32_t)((wn * WN + frow) * (BK * 2));
-  uint32_t chunk_off[4];
+  uint32_t chunk_off[2];
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) chunk_off[ks] = (uint32_t)(((2 * ks + fhalf) ^ ((frow >> 1) & 7)) * 16);
+  for (int ks = 0; ks < 2; ++ks) chunk_off[ks] = (uint32_t)(((4 * ks + fq) ^ ((frow >> 1) & 7)) * 16);
 
-  float16v acc[MI][2];
+  constexpr int RT = 2 * MI;   // 16-row tiles of a wavefront (its 64 columns are 4 tiles)
+  float4v acc[RT][4];
 #pragma unroll
-  for (int i = 0; i < MI; ++i)
+  for (int i = 0; i < RT; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
-  auto read_frags = [&](int kt, int ks, u32x4(&af)[MI], u32x4(&wf)[2]) {
+  auto read_frags = [&](int kt, int ks, u32x4(&af)[RT], u32x4(&wf)[4]) {
     const char* sa = lds + (kt & 1) * kStageBytes;
     const char* sw = sa + kTileBytes;
 #pragma unroll
-    for (int i = 0; i < MI; ++i) af[i] = *(const u32x4*)(sa + a_row_off + i * (32 * BK * 2) + chunk_off[ks]);
+    for (int i = 0; i < 4; ++i) wf[i] = *(const u32x4*)(sw + w_row_off + i * (16 * BK * 2) + chunk_off[ks]);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) wf[i] = *(const u32x4*)(sw + w_row_off + i * (32 * BK * 2) + chunk_off[ks]);
+    for (int i = 0; i < RT; ++i) af[i] = *(const u32x4*)(sa + a_row_off + i * (16 * BK * 2) + chunk_off[ks]);
   };
-  auto mfma8 = [&](const u32x4(&af)[MI], const u32x4(&wf)[2]) {
+  auto mfma_step = [&](const u32x4(&af)[RT], const u32x4(&wf)[4]) {
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
+    for (int i = 0; i < RT; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = mfma32<BF16>(af[i], wf[j], acc[i][j]);
+      for (int j = 0; j < 4; ++j) acc[i][j] = mfma16<BF16>(af[i], wf[j], acc[i][j]);
   };
-  auto interleave = [&]() {  // scheduling hint: the 6 LDS reads spread over the 8 MFMA of a k-step
+  auto interleave = [&]() {  // scheduling hint: the 12 LDS reads spread over the 32 MFMA of a k-step
     if constexpr (MI != 4) return;  // the small tiles are bound by the weight stream: the compiler's order will do
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 3, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
   };
 
   const int nk_total = (int)(g.k / BK);
   const int kt_base = kt_base_;
   const int nk = tail_part >= 0 ? min(g.tail_kt, nk_total - kt_base)
                                 : (g.partial ? min(g.kt_per_split, nk_total - kt_base) : nk_total);
-  u32x4 a0[MI], w0[2], a1[MI], w1[2];
+  u32x4 a0[RT], w0[4], a1[RT], w1[4];
   issue_loads(0);
   if (nk > 1) {
     issue_loads(1);
@@ -286,40 +291,36 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   read_frags(0, 0, a0, w0);
   int kt = 0;
   for (; kt + 2 < nk; ++kt) {  // steady state: a tile kt+2 exists, the body has no branches
-    read_frags(kt, 1, a1, w1); mfma8(a0, w0); interleave();
-    read_frags(kt, 2, a0, w0); mfma8(a1, w1); interleave();
-    read_frags(kt, 3, a1, w1); mfma8(a0, w0); interleave();
+    read_frags(kt, 1, a1, w1); mfma_step(a0, w0); interleave();
     APS_WAIT_LGKM0();  // every fragment of tile kt is in registers: its stage is free
     APS_WAIT_VM(0);    // tile kt+1 has landed (this wave's part; the barrier covers the others)
     APS_BARRIER();
     issue_loads(kt + 2);
-    read_frags(kt + 1, 0, a0, w0); mfma8(a1, w1); interleave();
+    read_frags(kt + 1, 0, a0, w0); mfma_step(a1, w1); interleave();
   }
   for (; kt < nk; ++kt) {  // last two tiles: nothing left to issue
-    read_frags(kt, 1, a1, w1); mfma8(a0, w0); interleave();
-    read_frags(kt, 2, a0, w0); mfma8(a1, w1); interleave();
-    read_frags(kt, 3, a1, w1); mfma8(a0, w0); interleave();
+    read_frags(kt, 1, a1, w1); mfma_step(a0, w0); interleave();
     APS_WAIT_LGKM0();
     APS_WAIT_VM(0);
     APS_BARRIER();
     if (kt + 1 < nk) read_frags(kt + 1, 0, a0, w0);
-    mfma8(a1, w1);
+    mfma_step(a1, w1);
   }
 
   // ---- epilogue: bias, round once, transpose through LDS, 128-bit row stores.
-  // Lane l of a 32x32 result tile holds column l%32 and rows 8*(e/4) + 4*(l/32) + e%4, e = 0..15.
+  // Lane l of a 16x16 result tile holds column l%16 and rows 4*(l/16) + e, e = 0..3.
   // Each wave owns a [32*MI rows][64 cols] fp16 image (row pitch 144 B).  Neighbouring lanes swap one value
   // so that every lane writes a 32-bit pair; the image is then read back 16 bytes per lane, 8 lanes per row.
   if (tail_part >= 0) {  // part of a tail tile: raw fp32 sums into its own [TBM][256] image
     float* pz = g.tail_partial + (int64_t)tail_slot * (TBM * BN);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int col = wn * WN + j * 32 + frow;
+    for (int j = 0; j < 4; ++j) {
+      const int col = wn * WN + j * 16 + frow;
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
+      for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int row = wm * WM + i * 32 + 8 * (e >> 2) + 4 * fhalf + (e & 3);
+        for (int e = 0; e < 4; ++e) {
+          const int row = wm * WM + i * 16 + 4 * fq + e;
           pz[row * BN + col] = acc[i][j][e];
         }
     }
@@ -328,13 +329,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   if (g.partial) {  // split-K: raw fp32 partial sums, lanes of a half-wave write 128 contiguous bytes
     float* pz = g.partial + (int64_t)blockIdx.y * g.m * g.n;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int64_t col = col0 + wn * WN + j * 32 + frow;
+    for (int j = 0; j < 4; ++j) {
+      const int64_t col = col0 + wn * WN + j * 16 + frow;
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
+      for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int64_t row = row0 + wm * WM + i * 32 + 8 * (e >> 2) + 4 * fhalf + (e & 3);
+        for (int e = 0; e < 4; ++e) {
+          const int64_t row = row0 + wm * WM + i * 16 + 4 * fq + e;
           if (row < g.m) pz[row * g.n + col] = acc[i][j][e];
         }
     }
@@ -345,17 +346,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   char* img = lds + wave * kEpiWaveBytes;
   const bool odd = lane & 1;
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int col = j * 32 + frow;  // column inside the wave's 64-column strip
+  for (int j = 0; j < 4; ++j) {
+    const int col = j * 16 + frow;  // column inside the wave's 64-column strip
     float bv = 0.f;
     if (g.bias) {
       const uint16_t bb = ((const uint16_t*)g.bias)[col0 + wn * WN + col];
       bv = BF16 ? __uint_as_float((uint32_t)bb << 16) : (float)__builtin_bit_cast(_Float16, bb);
     }
 #pragma unroll
-    for (int i = 0; i < MI; ++i) {
+    for (int i = 0; i < RT; ++i) {
 #pragma unroll
-      for (int e = 0; e < 16; e += 2) {
+      for (int e = 0; e < 4; e += 2) {
         const float v0 = acc[i][j][e] + bv, v1 = acc[i][j][e + 1] + bv;
         const uint32_t h0 = BF16 ? f32_to_bf16_bits(v0) : f32_to_f16_bits(v0);
         const uint32_t h1 = BF16 ? f32_to_bf16_bits(v1) : f32_to_f16_bits(v1);
@@ -363,7 +364,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         const uint32_t send = odd ? h0 : h1;
         const uint32_t recv = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send, 0xB1, 0xf, 0xf, true);
         const uint32_t pair = odd ? (recv | (h1 << 16)) : (h0 | (recv << 16));
-        const int row = i * 32 + 8 * (e >> 2) + 4 * fhalf + (e & 3) + (odd ? 1 : 0);
+        const int row = i * 16 + 4 * fq + e + (odd ? 1 : 0);
         *(uint32_t*)(img + row * kEpiPitch + (col & ~1) * 2) = pair;
       }
     }
