@@ -265,6 +265,7 @@ def main():
             extras["prompt_attention_4x2048"] = prompt_attention_figures(torch, ops, dev, args.seed)
         if "reproject" in want:
             extras.update(reproject_figures(torch, ops, dev, args.seed))
+            extras["mfma_ceilings"] = mfma_ceiling_figures(torch, dev)   # after the products: it heats the part
         torch.cuda.empty_cache()
         if "layer" in want:
             extras["decode_layer_config2"] = decode_layer_figures(torch, ops, workloads, metadata, dev, args.seed)
@@ -368,6 +369,28 @@ def stream_ceiling_figures(torch, dev):
     for name, n in (("read_of_fp8_attention_size", half), ("read_of_f16_attention_size", 2 * half)):
         ms = median(event_times(torch, lambda: lib.aps_stream_probe(1, 1, b.data_ptr(), a.data_ptr(), n, st), 20))
         out[name] = {"bytes": n, "ms": ms, "GB/s": n / ms / 1e6, "frac_of_hbm_peak": n / ms / 1e6 / HBM_PEAK_GBS}
+    return out
+
+
+def mfma_ceiling_figures(torch, dev):
+    """What the matrix cores sustain with nothing else running (aps_mfma_probe: 256 workgroups of 4 wavefronts,
+    operands in registers): under N(0,1) operands the part lowers its clock to stay inside its power limit, and how
+    far depends on the instruction shape.  The re-projection GEMM is held against the figure of its own shape."""
+    from aptserve_hip import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    sink = torch.empty(256 * 256, dtype=torch.float32, device=dev)
+    iters = 3200
+    flops = 256 * 4 * iters * 2 * 16 * 32 * 32 * 16
+    out = {"workgroups": 256, "iters": iters, "flops": flops}
+    g = torch.Generator(device=dev).manual_seed(0)
+    for data, ops_ in (("random_N01", torch.randn(16384, generator=g, device=dev).half()),
+                       ("zeros", torch.zeros(16384, dtype=torch.float16, device=dev))):
+        for shape, name in ((0, "32x32x16"), (1, "16x16x32")):
+            ms = median(event_times(torch, lambda: lib.aps_mfma_probe(shape, 0, ops_.data_ptr(), sink.data_ptr(), 256,
+                                                                        iters, st), 12))
+            out[f"f16_{name}_{data}"] = {"ms": ms, "tflops": flops / ms / 1e9,
+                                          "frac_of_mfma_peak": flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS}
     return out
 
 
@@ -537,17 +560,21 @@ def reproject_figures(torch, ops, dev, seed):
     for T in (4096, 16384):
         x = torch.randn(T, Hd, generator=g, device=dev).half()
         y = torch.empty(T, 2 * Hd, dtype=torch.float16, device=dev)
-        ms = median(event_times(torch, lambda: ops.kv_reproject(x, w, bias, out=y), 20))
+        # ~25 ms of the product itself before the timed launches: coming from lighter work the part needs that
+        # long to settle at the clock it sustains under matrix load (T=4096 timed cold reads 15 % slower)
+        warm = 64 if T == 4096 else 20
+        ms = median(event_times(torch, lambda: ops.kv_reproject(x, w, bias, out=y), 20, warm=warm))
         flops = 2.0 * T * Hd * 2 * Hd
         tf = flops / ms / 1e9
         out["kv_reproject_T%d" % T] = {
-            "workload": "config3 [T,5120]x[5120,10240] f16, f32 accumulate, T=%d" % T, "ms": ms, "tflops": tf,
+            "workload": "config3 [T,5120]x[5120,10240] f16, f32 accumulate, T=%d, %d warm-up launches" % (T, warm),
+            "ms": ms, "tflops": tf,
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": tf / MFMA_F16_PEAK_TFLOPS,
                          "traffic": PMC_TRAFFIC_BYTES["gemm_T%d" % T] if seed == 0 else None}}
         # the vendor BLAS on the same product (what the reference's F.linear call runs on this GPU), as a
         # stated comparison: same operands, same event timing
-        ms_blas = median(event_times(torch, lambda: torch.nn.functional.linear(x, w, bias), 20))
+        ms_blas = median(event_times(torch, lambda: torch.nn.functional.linear(x, w, bias), 20, warm=warm))
         out["kv_reproject_T%d" % T]["vendor_blas_F_linear"] = {
             "ms": ms_blas, "tflops": flops / ms_blas / 1e9, "frac_of_mfma_peak": flops / ms_blas / 1e9 / MFMA_F16_PEAK_TFLOPS,
             "kernel_over_vendor": ms_blas / ms}

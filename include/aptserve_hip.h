@@ -512,6 +512,18 @@ int aps_copy_bytes(void* dst, const void* src, int64_t nbytes,
 int aps_stream_probe(int mode, int chunks_per_thread, void* dst,
                      const void* src, int64_t nbytes, aps_stream_t stream);
 
+/* Matrix-core instructions alone, for measuring what the part sustains under
+ * the power they draw: `workgroups` workgroups of 4 wavefronts (one per SIMD)
+ * run `iters` rounds of 16 v_mfma_f32_32x32x16 (shape 0) or 32
+ * v_mfma_f32_16x16x32 (shape 1) on operands kept in registers, which they load
+ * once from `operands` (32 KiB of f16 / bf16 values, 16-byte aligned: random
+ * values make the part throttle, zeros do not).  Flops of a launch:
+ * workgroups * 4 * iters * 2 * 16 * 32*32*16.  `sink` receives one float per
+ * thread (workgroups * 256 floats).  No counterpart in the reference: the
+ * ceiling the re-projection GEMM is compared against comes from this. */
+int aps_mfma_probe(int shape, int dtype, const void* operands, void* sink,
+                   int workgroups, int iters, aps_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
