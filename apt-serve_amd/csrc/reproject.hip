@@ -5,15 +5,20 @@
 // are laid out.
 //
 // Tiling: one 512-thread workgroup (8 wavefronts, 2 x 4) owns a 256 x 256 tile
-// of C; each wavefront owns 128 x 64 = 4 x 2 MFMA 32x32x16 tiles (128 fp32
-// accumulator registers per lane), so two wavefronts fit on every SIMD.  That
-// matters more than the larger per-wave tile it replaces: a wavefront issues in
-// order, and while it is held at a global load the matrix core of its SIMD is
+// of C; each wavefront owns 128 x 64 = 8 x 4 tiles of v_mfma_f32_16x16x32 (128
+// fp32 accumulator registers per lane), so two wavefronts fit on every SIMD.
+// That matters more than the larger per-wave tile it replaces: a wavefront issues
+// in order, and while it is held at a global load the matrix core of its SIMD is
 // only kept busy by the other wavefront (with one wavefront per SIMD the main
-// loop took 1.4x the cycles).  The K loop moves BK = 64 at a time through a
-// two-stage LDS ring (2 x (32 + 32) KiB of the 160 KiB per CU; 144 KiB with the
-// epilogue images): tile t+1 is copied global -> LDS by buffer_load ... lds (no
-// VGPR round trip) while the matrix cores consume tile t.
+// loop took 1.4x the cycles).  The instruction shape is a matter of power: on
+// random operands the part lowers its clock until the matrix cores fit its power
+// limit, and 16x16x32 (32 multiply-adds per accumulator element and instruction)
+// needs less energy per flop than 32x32x16 (16): alone, with operands in
+// registers, they sustain 1.8 against 1.4-1.6 PFLOP/s (aps_mfma_probe).
+// The K loop moves BK = 64 at a time through a two-stage LDS ring (2 x (32 + 32)
+// KiB of the 160 KiB per CU; 144 KiB with the epilogue images): tile t+1 is
+// copied global -> LDS by buffer_load ... lds (no VGPR round trip) while the
+// matrix cores consume tile t.
 //
 // LDS layout: a tile is [256 rows][8 chunks of 16 B]; chunk c of row r lives at
 // position c ^ ((r >> 1) % 8).  The LDS of gfx950 serves a 128-bit read to 16
@@ -24,8 +29,9 @@
 // so the swizzle is applied on the global side: lane l of a wave-wide load
 // fetches chunk (l%8) ^ ((row>>1)%8) of row l/8 of its 8-row group.
 //
-// Schedule: fragments live in two register sets; while the matrix cores work
-// on k-step s the 6 ds_read_b128 of k-step s+1 are in flight (8 MFMA : 6 reads).
+// Schedule: a tile is two k-steps of 32; fragments live in two register sets;
+// while the matrix cores work on k-step s the 12 ds_read_b128 of k-step s+1 are
+// in flight (32 MFMA : 12 reads).
 // Before the last k-step of a tile every wave has its fragments in registers,
 // so after one barrier the stage can be refilled with tile t+2 while the last
 // k-step runs and the first fragments of tile t+1 stream in.  Waits and the
