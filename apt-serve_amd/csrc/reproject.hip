@@ -389,7 +389,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     if (!dst) continue;
     dst += ocol + rchunk * 8;
     if (g.out.aligned16)
-      *(u32x4*)dst = v;
+      __builtin_nontemporal_store(v, (u32x4*)dst);   // 4 MB per XCD and round: as much as its L2 holds
     else {
       uint32_t* d = (uint32_t*)dst;
       d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];

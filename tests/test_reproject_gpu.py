@@ -292,3 +292,22 @@ def test_config3_kv_reprojection_opt13b(dev):
     out2 = ops.kv_reproject(x2.to(dev), dw, db)
     rows = torch.from_numpy(np.random.default_rng(0).choice(16384, 384, replace=False))
     check(out2[rows.to(dev)], OR._linear_fp32(x2[rows], w, b))
+
+
+def test_matrix_core_probe_runs_and_adds_what_it_multiplies(dev):
+    """aps_mfma_probe is a measurement aid, but its kernels are real: with all-ones operands every accumulator of a
+    16x16x32 product grows by 32 per round (16 per round for 32x32x16), and a thread sums all of its accumulators."""
+    from aptserve_hip import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    ones = torch.ones(16384, dtype=torch.float16, device=dev)
+    zeros = torch.zeros(16384, dtype=torch.float16, device=dev)
+    sink = torch.empty(4 * 256, dtype=torch.float32, device=dev)
+    iters = 3
+    for shape, per_thread in ((0, 16 * 16 * 16.0), (1, 32 * 4 * 32.0)):
+        assert lib.aps_mfma_probe(shape, 0, ones.data_ptr(), sink.data_ptr(), 4, iters, st) == 0
+        torch.cuda.synchronize()
+        assert torch.all(sink == per_thread * iters), (shape, sink[:4])
+        assert lib.aps_mfma_probe(shape, 0, zeros.data_ptr(), sink.data_ptr(), 4, iters, st) == 0
+        torch.cuda.synchronize()
+        assert torch.all(sink == 0)
