@@ -753,6 +753,22 @@ def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, se
 
 # ------------------------------------------------------------------ block maintenance
 
+_LAYER_BASES = {}
+
+
+def _layer_bases(kv_caches, dev):
+    """Device vector of the layer caches' base addresses.  The caches of a model live as long as its engine, so
+    the vector is uploaded once per set of caches and not with a blocking copy in every call."""
+    key = (dev.index, tuple(c.data_ptr() for c in kv_caches))
+    bases = _LAYER_BASES.get(key)
+    if bases is None:
+        if len(_LAYER_BASES) >= 16:
+            _LAYER_BASES.clear()
+        bases = torch.tensor(key[1], dtype=torch.int64).to(dev)
+        _LAYER_BASES[key] = bases
+    return bases
+
+
 def copy_blocks(kv_caches, src_to_dsts, kinds=None) -> None:
     """``FlashAttentionBackend.copy_blocks`` (additional_designs/attention/backends/aptserve_flash_attn.py:58-65)
     for the caches of all layers in one launch; ``src_to_dsts`` int64 ``[n, 2]`` on the device.
@@ -774,7 +790,7 @@ def copy_blocks(kv_caches, src_to_dsts, kinds=None) -> None:
               and kinds.numel() == n, "kinds must be a contiguous uint8/bool vector, one entry per pair")
     if n == 0:
         return
-    bases = torch.tensor([c.data_ptr() for c in kv_caches], dtype=torch.int64).to(dev)
+    bases = _layer_bases(kv_caches, dev)
     _, N, BS, H, D = c0.shape
     with _on(dev):
         st = _lib.load().aps_copy_cache_blocks(bases.data_ptr(), len(kv_caches), src_to_dsts.data_ptr(), _ptr(kinds), n,

@@ -311,10 +311,39 @@ def prompt_attention_figures(torch, ops, dev, seed):
                                                                       causal=True, out=out), 10))
     flops = sum(2 * 2 * L * L * H * D / 2 for L in lens)
     tf = flops / ms / 1e9
+    # the same launch on all-zero inputs: the part keeps its clock there, so the difference is what the power the
+    # real operands draw costs, and the zero-input time is what the instruction schedule alone would allow
+    q.zero_(); k.zero_(); v.zero_()
+    for _ in range(20):
+        ops.flash_attn_varlen_func(q, k, v, cu, cu, max(lens), max(lens), causal=True, out=out)
+    ms0 = median(event_times(torch, lambda: ops.flash_attn_varlen_func(q, k, v, cu, cu, max(lens), max(lens),
+                                                                       causal=True, out=out), 10))
     return {"workload": "causal varlen attention, 4 prompts x 2048 tokens, 40 heads x 128, fp16", "ms": ms,
             "tokens_per_s": T / ms * 1e3, "algorithmic_flops": flops,
             "roofline": {"bound": "mfma", "achieved": tf, "peak": 2500.0, "unit": "TFLOP/s", "frac": tf / 2500.0,
-                         "traffic": None}}
+                         "traffic": None},
+            "ms_on_zero_inputs": ms0, "issue_mix": issue_mix_figures(torch, dev)}
+
+
+def issue_mix_figures(torch, dev):
+    """How a SIMD issues matrix and vector instructions side by side (aps_mfma_probe shapes 2..6, zero operands so
+    that the clock stays up; 256 workgroups, a round = 16 v_mfma_f32_32x32x16 and / or 16 x [v_exp_f32 + 3
+    v_fma_f32]).  The prompt attention's softmax is vector work of about the size of its matrix work: the two
+    overlap when they alternate inside a wavefront's instruction stream and hardly when wavefronts issue them in
+    runs, which is how a compiler-scheduled attention loop issues them."""
+    from aptserve_hip import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
+    zeros = torch.zeros(16384, dtype=torch.float16, device=dev)
+    iters = 2000
+    out = {"workgroups": 256, "iters": iters}
+    for shape, name in ((0, "mfma_only_16_accumulators_1_wave_per_simd"), (4, "vector_only_1_wave_per_simd"),
+                        (3, "mfma_run_then_vector_run_1_wave_per_simd"), (2, "alternating_1_wave_per_simd"),
+                        (6, "mfma_run_then_vector_run_2_waves_per_simd"), (5, "alternating_2_waves_per_simd")):
+        out[name + "_ms"] = median(event_times(torch, lambda: lib.aps_mfma_probe(
+            shape, 0, zeros.data_ptr(), sink.data_ptr(), 256, iters, st), 8))
+    return out
 
 
 def write_figures(torch, ops, dev, seed, block_contiguous=False):

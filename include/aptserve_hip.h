@@ -519,8 +519,15 @@ int aps_stream_probe(int mode, int chunks_per_thread, void* dst,
  * once from `operands` (32 KiB of f16 / bf16 values, 16-byte aligned: random
  * values make the part throttle, zeros do not).  Flops of a launch:
  * workgroups * 4 * iters * 2 * 16 * 32*32*16.  `sink` receives one float per
- * thread (workgroups * 256 floats).  No counterpart in the reference: the
- * ceiling the re-projection GEMM is compared against comes from this. */
+ * thread (workgroups * 256 floats).  Shapes 2..6 measure how a SIMD issues
+ * matrix and vector instructions side by side; a round is 16
+ * v_mfma_f32_32x32x16 and / or 16 vector units (one v_exp_f32 and three
+ * v_fma_f32 on registers): 2 the two kinds alternating instruction by
+ * instruction, 3 all the MFMAs and then all the vector units, 4 the vector
+ * units alone, all with one wavefront per SIMD; 5 and 6 are 2 and 3 with two
+ * wavefronts per SIMD (workgroups of 8 wavefronts; sink: workgroups * 512
+ * floats).  No counterpart in the reference: the ceilings the re-projection
+ * GEMM and the prompt attention are compared against come from this. */
 int aps_mfma_probe(int shape, int dtype, const void* operands, void* sink,
                    int workgroups, int iters, aps_stream_t stream);
 

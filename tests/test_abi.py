@@ -47,7 +47,8 @@ def test_argument_errors_return_without_launching():
     assert lib.aps_hidden_to_cache(None, None, None, None, None, 4, 768, 768, 768, 0, 0, 0, 2, None) == -1
     assert lib.aps_hidden_to_cache(None, None, None, None, None, 4, 768, 768, 768, 0, 0, 0, 3, None) == -1
     # the matrix-core probe: unknown shape / dtype / null buffers are errors, an empty launch is not
-    assert lib.aps_mfma_probe(2, 0, 16, 16, 1, 1, None) == -1
+    assert lib.aps_mfma_probe(7, 0, 16, 16, 1, 1, None) == -1
+    assert lib.aps_mfma_probe(-1, 0, 16, 16, 1, 1, None) == -1
     assert lib.aps_mfma_probe(0, 5, 16, 16, 1, 1, None) == -1
     assert lib.aps_mfma_probe(0, 0, None, None, 1, 1, None) == -1
     assert lib.aps_mfma_probe(1, 0, 16, 16, 0, 1, None) == 0

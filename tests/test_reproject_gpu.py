@@ -311,3 +311,26 @@ def test_matrix_core_probe_runs_and_adds_what_it_multiplies(dev):
         assert lib.aps_mfma_probe(shape, 0, zeros.data_ptr(), sink.data_ptr(), 4, iters, st) == 0
         torch.cuda.synchronize()
         assert torch.all(sink == 0)
+
+
+def test_issue_mix_probe_shapes_compute_what_they_say(dev):
+    """Shapes 2..6 of aps_mfma_probe interleave MFMAs with vector units (v_exp_f32 and three v_fma_f32 on eight
+    register values per lane, two units per value and round).  With zero operands the products are zero and every
+    value follows x -> fma(fma(fma(2^x, c0, c1), c0, c1), c0, c1) from 0, whatever the order of issue."""
+    import numpy as np
+    from aptserve_hip import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    zeros = torch.zeros(16384, dtype=torch.float16, device=dev)
+    iters = 3
+    x = np.float64(0.0)
+    c0, c1 = np.float64(np.float32(1e-3)), np.float64(np.float32(0.5))
+    for _ in range(2 * iters):
+        x = np.float64(np.float32(np.exp2(x)))
+        for _ in range(3):
+            x = np.float64(np.float32(x * c0 + c1))
+    for shape, threads in ((2, 256), (3, 256), (4, 256), (5, 512), (6, 512)):
+        sink = torch.full((4 * threads,), float("nan"), dtype=torch.float32, device=dev)
+        assert lib.aps_mfma_probe(shape, 0, zeros.data_ptr(), sink.data_ptr(), 4, iters, st) == 0
+        torch.cuda.synchronize()
+        assert torch.allclose(sink, torch.full_like(sink, 8 * float(x)), rtol=1e-5, atol=0), (shape, sink[:4])
