@@ -398,6 +398,15 @@ def stream_ceiling_figures(torch, dev):
     for name, n in (("read_of_fp8_attention_size", half), ("read_of_f16_attention_size", 2 * half)):
         ms = median(event_times(torch, lambda: lib.aps_stream_probe(1, 1, b.data_ptr(), a.data_ptr(), n, st), 20))
         out[name] = {"bytes": n, "ms": ms, "GB/s": n / ms / 1e6, "frac_of_hbm_peak": n / ms / 1e6 / HBM_PEAK_GBS}
+    # the same buffer read again and again: sizes that stay in the 256 MB memory-side cache stream no faster than
+    # 2 GiB from HBM, i.e. a second pass over rows that a first pass left in that cache is not a faster pass
+    for mib in (64, 128, 256):
+        n = mib << 20
+        for _ in range(5):
+            lib.aps_stream_probe(1, 1, b.data_ptr(), a.data_ptr(), n, st)
+        ms = median(event_times(torch, lambda: lib.aps_stream_probe(1, 1, b.data_ptr(), a.data_ptr(), n, st), 20))
+        out[f"read_of_{mib}MiB_repeated"] = {"bytes": n, "ms": ms, "GB/s": n / ms / 1e6,
+                                             "frac_of_hbm_peak": n / ms / 1e6 / HBM_PEAK_GBS}
     return out
 
 
