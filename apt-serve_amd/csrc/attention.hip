@@ -625,6 +625,15 @@ int aps_decode_attention_partition_size(int64_t batch, int num_heads, int64_t ma
   int64_t part = 512;
   while (part > 32 && batch * num_heads * ((max_seq_len + part - 1) / part) < 4096) part >>= 1;
   if (part % block_size != 0) part = (part + block_size - 1) / block_size * block_size;
+  // few sequences whose longest still fits the eight wavefronts of one workgroup at partitions of at most 128
+  // tokens: take those instead, one launch whose partial results merge in LDS (5 sequences of up to 1000 tokens:
+  // 19 against 23-25 us per call; with longer partitions a wavefront walks too many tiles one after the other:
+  // one sequence of 2048 tokens, 32 against 23 us)
+  if ((max_seq_len + part - 1) / part > kMaxGroupWaves) {
+    const int64_t eighth = (max_seq_len + kMaxGroupWaves - 1) / kMaxGroupWaves;
+    const int64_t gp = (eighth + block_size - 1) / block_size * block_size;
+    if (gp <= 128) part = gp;
+  }
   // plenty of sequences: lengthen the partitions until a sequence fits the wavefronts of one workgroup (the
   // partial results then merge in LDS), as far as the 64 block ids a wavefront holds allow
   if (batch * num_heads >= 1024)
