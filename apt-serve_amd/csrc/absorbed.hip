@@ -10,7 +10,7 @@
 //   1. qt[s][h][:]  = scale*log2(e) * W_k[h]^T q[s][h]            nn_few_rows_kernel (B = rows of W_k)
 //   2. S[s][h][t]   = <qt[s][h], h_t>                               seq_plan_kernel (work list of the ragged
 //                                                                   batch), hidden_scores_kernel (paged rows)
-//   3. P[s][h][:]   = softmax_t, 16-bit, zero padded                softmax_rows_kernel
+//   3. P[s][h][:]   = softmax_t, 16-bit, zero padded to 32 tokens   softmax_rows_kernel
 //   4. ctx[s][h][:] = sum_t P[s][h][t] h_t                          nn_few_rows_kernel (B = paged rows)
 //   5. out[s][h*D+d] = <W_v[h*D+d], ctx[s][h]> + b_v                head_proj_kernel; up to 16 sequences: the
 //                                                                   weight-streaming kernels of the projection
@@ -401,7 +401,8 @@ __global__ __launch_bounds__(kScThreads) void head_proj_kernel(const HeadProjArg
 }
 
 // ------------------------------------------------------------------ softmax over the tokens of a row
-// P[z][h][t] = exp2(S - max) / sum for t < L(z), 0 for L <= t < lp; S already carries scale*log2(e).
+// P[z][h][t] = exp2(S - max) / sum for t < L(z), 0 for L <= t < the next multiple of 32; S already carries
+// scale*log2(e).
 template <bool BF16>
 __global__ __launch_bounds__(256) void softmax_rows_kernel(float* __restrict__ s, uint16_t* __restrict__ p,
                                                            const int64_t* __restrict__ row_start, int heads,
@@ -452,7 +453,10 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(float* __restrict__ s
   __syncthreads();
   sum = (red[0] + red[1]) + (red[2] + red[3]);
   const float inv = 1.f / sum;
-  for (int64_t t = threadIdx.x * 4; t < lp; t += 1024) {   // zero padded up to lp
+  // zero padded to the next multiple of 32 tokens: the weighted sum reads a row's probabilities 32 at a time and
+  // never past its sequence
+  const int64_t pad_to = min(lp, (int64_t)((L + 31) / 32 * 32));
+  for (int64_t t = threadIdx.x * 4; t < pad_to; t += 1024) {
     float4 v = {0.f, 0.f, 0.f, 0.f};
     if (t < L) v = *(const float4*)(src + t);
     uint16_t o[4];
@@ -643,7 +647,7 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     const int st = launch_status();
     if (st != APS_OK) return st;
   }
-  // 3. P = softmax over the tokens, zero padded to lp
+  // 3. P = softmax over the tokens, zero padded to whole groups of 32 tokens
   {
     const dim3 grid((unsigned)num_heads, (unsigned)n_seqs);
     if (bf16)
