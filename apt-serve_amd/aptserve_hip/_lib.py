@@ -67,25 +67,31 @@ _lib = None
 _protos = None
 
 
+def bind(lib_path: Path, header: Path):
+    """``ctypes.CDLL`` of ``lib_path`` with the prototypes ``header`` declares; raises if it has not been built."""
+    # torch first: its HIP runtime must be the one the library binds to, so
+    # that streams and device pointers mean the same thing on both sides.
+    import torch  # noqa: F401
+
+    if not lib_path.exists():
+        raise ImportError(
+            f"{lib_path} is missing: build it with `python {PKG_DIR / 'build.py'}` "
+            "(hipcc, gfx950). There is no fallback path.")
+    lib = ctypes.CDLL(str(lib_path))
+    protos = parse_header(header)
+    for name, (restype, argtypes, _) in protos.items():
+        fn = getattr(lib, name)  # AttributeError if the header names a symbol the library lacks
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return lib, protos
+
+
 def load() -> ctypes.CDLL:
     """Load the library once; raises if it has not been built."""
     global _lib, _protos
     if _lib is not None:
         return _lib
-    # torch first: its HIP runtime must be the one the library binds to, so
-    # that streams and device pointers mean the same thing on both sides.
-    import torch  # noqa: F401
-
-    if not LIB_PATH.exists():
-        raise ImportError(
-            f"{LIB_PATH} is missing: build it with `python {PKG_DIR / 'build.py'}` "
-            "(hipcc, gfx950). There is no fallback path.")
-    lib = ctypes.CDLL(str(LIB_PATH))
-    _protos = parse_header()
-    for name, (restype, argtypes, _) in _protos.items():
-        fn = getattr(lib, name)  # AttributeError if the header names a symbol the library lacks
-        fn.restype = restype
-        fn.argtypes = argtypes
+    lib, _protos = bind(LIB_PATH, HEADER)
     if lib.aps_abi_version() != _abi_version_of_header():
         raise ImportError("libaptserve_hip.so was built from a different header; rebuild it")
     runtimes = {l.split()[-1] for l in open("/proc/self/maps") if "libamdhip64" in l}

@@ -1,4 +1,5 @@
-"""Build libaptserve_hip.so from csrc/*.hip with hipcc for gfx950.
+"""Build libaptserve_hip.so from csrc/*.hip, and the benchmark's measurement kernels
+(csrc/probes/*.hip) into libaptserve_probes.so, with hipcc for gfx950.
 
 Run ``python apt-serve_amd/aptserve_hip/build.py`` (add ``--force`` to
 recompile objects that look up to date).  The library is written next to this
@@ -19,6 +20,7 @@ CSRC = PKG_DIR.parent / "csrc"
 INCLUDE = PKG_DIR.parent.parent / "include"
 BUILD_DIR = PKG_DIR.parent / "build"
 LIB_PATH = PKG_DIR / "libaptserve_hip.so"
+PROBES_LIB_PATH = PKG_DIR / "libaptserve_probes.so"
 
 HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
@@ -49,11 +51,10 @@ def _compile(src: Path, obj: Path) -> None:
         sys.stderr.write(err + "\n")
 
 
-def build(force: bool = False, verbose: bool = True) -> Path:
+def _build_lib(sources, lib_path: Path, force: bool, verbose: bool) -> Path:
     BUILD_DIR.mkdir(exist_ok=True)
-    sources = sorted(CSRC.glob("*.hip"))
     if not sources:
-        raise RuntimeError(f"no HIP sources under {CSRC}")
+        raise RuntimeError(f"no HIP sources for {lib_path.name}")
     jobs = []
     objs = []
     for src in sources:
@@ -62,18 +63,26 @@ def build(force: bool = False, verbose: bool = True) -> Path:
         if force or _stale(obj, src):
             jobs.append((src, obj))
     if verbose:
-        print(f"[aptserve_hip.build] compiling {len(jobs)}/{len(sources)} sources for gfx950", flush=True)
+        print(f"[aptserve_hip.build] {lib_path.name}: compiling {len(jobs)}/{len(sources)} sources for gfx950",
+              flush=True)
     with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
         list(ex.map(lambda j: _compile(*j), jobs))
-    if jobs or not LIB_PATH.exists():
+    if jobs or not lib_path.exists():
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc",
-               *map(str, objs), "-o", str(LIB_PATH)]
+               *map(str, objs), "-o", str(lib_path)]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"link failed:\n{' '.join(cmd)}\n{r.stdout}\n{r.stderr}")
     if verbose:
-        print(f"[aptserve_hip.build] {LIB_PATH}", flush=True)
-    return LIB_PATH
+        print(f"[aptserve_hip.build] {lib_path}", flush=True)
+    return lib_path
+
+
+def build(force: bool = False, verbose: bool = True) -> Path:
+    """Compile both libraries; returns the path of the product library."""
+    lib = _build_lib(sorted(CSRC.glob("*.hip")), LIB_PATH, force, verbose)
+    _build_lib(sorted((CSRC / "probes").glob("*.hip")), PROBES_LIB_PATH, force, verbose)
+    return lib
 
 
 if __name__ == "__main__":

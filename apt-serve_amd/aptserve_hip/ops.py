@@ -188,6 +188,51 @@ def gather_hidden_rows(holder, hidden_states, paged_cache, holder_src, slot_mapp
     _lib.check(st, "gather_hidden_rows")
 
 
+def decode_step_cache_ops(holder, hidden_states, paged_cache, holder_src, slot_mapping, hidden_cache_use_input,
+                          hidden_cache_store_tot, key, value, kv_cache_use_input, new_token_slot) -> None:
+    """The cache traffic of one decode layer in one launch: ``gather_hidden_rows`` (store of the newest hidden
+    rows, holder assembly: additional_designs/model_executor/models/aptserve_opt.py:108-121) and the write of
+    the newest K/V rows of the K/V-cached sequences into the two planes of ``paged_cache``
+    (``reshape_and_cache_flash``, additional_designs/attention/backends/aptserve_flash_attn.py:338-345).
+    ``key`` / ``value`` ``[batch, H*D]`` or ``[batch, H, D]``; ``kv_cache_use_input`` and ``new_token_slot``
+    from the metadata builder.  Same bytes in the cache and the holder as the two separate calls."""
+    dev = holder.device
+    for n, t in (("holder", holder), ("hidden_states", hidden_states), ("paged_cache", paged_cache),
+                 ("key", key), ("value", value)):
+        _check_data(n, t, dev)
+    _need(holder.dim() == 2 and hidden_states.dim() == 2, "holder and hidden_states must be 2-D")
+    width = hidden_states.size(1)
+    _need(holder.size(1) == width, "holder and hidden_states widths differ")
+    _need(holder.dtype == hidden_states.dtype == paged_cache.dtype == key.dtype == value.dtype, "dtypes differ")
+    _check_paged(paged_cache, width)
+    _need(paged_cache.size(0) == 2 and paged_cache.size(3) * paged_cache.size(4) == width,
+          "paged_cache must be (2, num_blocks, block_size, heads, head_dim) with heads*head_dim == hidden width")
+    key = _as_thd("key", key, paged_cache.size(3), paged_cache.size(4))
+    value = _as_thd("value", value, paged_cache.size(3), paged_cache.size(4))
+    B = hidden_states.size(0)
+    _need(key.size(0) == B and value.size(0) == B, "one key / value row per sequence expected")
+    for n, t in (("holder_src", holder_src), ("slot_mapping", slot_mapping),
+                 ("hidden_cache_use_input", hidden_cache_use_input),
+                 ("hidden_cache_store_tot", hidden_cache_store_tot), ("kv_cache_use_input", kv_cache_use_input),
+                 ("new_token_slot", new_token_slot)):
+        _check_index(n, t, dev)
+    _need(holder_src.numel() == holder.size(0), "holder_src must have one entry per holder row")
+    _need(slot_mapping.numel() == holder.size(0), "slot_mapping must have one entry per holder row")
+    _need(hidden_cache_use_input.numel() == hidden_cache_store_tot.numel(), "store index lengths differ")
+    _need(new_token_slot.numel() == B, "new_token_slot must have one entry per sequence")
+    slot_stride = paged_cache.stride(2)
+    with _on(dev):
+        st = _lib.load().aps_decode_step_cache_ops(
+            holder.data_ptr(), hidden_states.data_ptr(), paged_cache.data_ptr(), _ptr(holder_src), holder.size(0),
+            _ptr(slot_mapping), _ptr(hidden_cache_use_input), _ptr(hidden_cache_store_tot),
+            hidden_cache_store_tot.numel(), B, width, holder.stride(0), hidden_states.stride(0), slot_stride,
+            paged_cache.numel() // slot_stride, key.data_ptr(), value.data_ptr(), paged_cache[0].data_ptr(),
+            paged_cache[1].data_ptr(), _ptr(kv_cache_use_input), _ptr(new_token_slot), kv_cache_use_input.numel(),
+            key.stride(0), value.stride(0), paged_cache.size(2), paged_cache.stride(1), paged_cache.size(1),
+            holder.element_size(), _stream(holder))
+    _lib.check(st, "decode_step_cache_ops")
+
+
 # --------------------------------------------------------------------- a3 / a4
 
 def _check_kv_cache(name: str, c: torch.Tensor, heads: int, head_size: int) -> None:
@@ -365,17 +410,6 @@ def mixed_kv_to_cache(key, value, k_cache, v_cache, shared_k_cache, shared_v_cac
             k_cache.size(1), key.stride(0), value.stride(0), k_cache.stride(0), k_cache.size(0),
             shared_k_cache.stride(0), shared_k_cache.size(0), key.element_size(), flags, _stream(key))
     _lib.check(st, "mixed_kv_to_cache")
-
-
-def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
-    """Plain device copy (calibration kernel for hardware counters)."""
-    _need(dst.is_cuda and src.is_cuda and dst.device == src.device, "both tensors must be on one GPU")
-    _need(dst.is_contiguous() and src.is_contiguous(), "tensors must be contiguous")
-    nbytes = src.numel() * src.element_size()
-    _need(nbytes == dst.numel() * dst.element_size(), "sizes differ")
-    with torch.cuda.device(src.device):
-        st = _lib.load().aps_copy_bytes(dst.data_ptr(), src.data_ptr(), nbytes, _stream(src))
-    _lib.check(st, "copy_bytes")
 
 
 # --------------------------------------------------------------------- a8
@@ -681,6 +715,7 @@ def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_se
     max_len = int(max_seqlen_q if max_seqlen_q is not None else (max_seqlen_k if max_seqlen_k is not None else T))
     if softmax_scale is None:
         softmax_scale = D ** -0.5
+    _need(0.0 < float(softmax_scale) < float("inf"), "softmax_scale must be positive and finite")
     if out is None:
         out = torch.empty(T, H, D, dtype=q.dtype, device=dev)
     else:

@@ -46,6 +46,14 @@ class Request:
     def seq_len(self) -> int:
         return len(self.prompt_ids) + len(self.generated)
 
+    @property
+    def token_ids(self) -> np.ndarray:
+        """Prompt and everything generated so far: what a prompt step feeds the model (after a recompute
+        preemption the generated tokens are part of it)."""
+        if not self.generated:
+            return self.prompt_ids
+        return np.concatenate([self.prompt_ids, np.asarray(self.generated, dtype=np.int64)])
+
 
 def synth_requests(seed: int, n: int, rate: float = 3.0, cv: float = 1.0, hidden_fraction: float = 0.5,
                    vocab: int = 50272, max_len: int = 2048, prompt_mu: float = 5.5, prompt_sigma: float = 1.0,
@@ -136,21 +144,24 @@ class StepLoop:
         batch, tokens = [], 0
         while self.waiting and self.waiting[0].arrival <= self.now and len(self.running) + len(batch) < self.max_seqs:
             r = self.waiting[0]
-            p_need, s_need = self.pool.blocks_needed(r, len(r.prompt_ids) + 1, self.block_size)
-            if tokens + len(r.prompt_ids) > self.max_prompt_tokens and batch:
+            n_tok = r.seq_len                    # a preempted request comes back with its generated tokens
+            p_need, s_need = self.pool.blocks_needed(r, n_tok + 1, self.block_size)
+            if tokens + n_tok > self.max_prompt_tokens and batch:
                 break
             if p_need > len(self.pool.free_private) - 8 or s_need > len(self.pool.free_shared) - 8:
                 break
-            self.pool.grow(r, len(r.prompt_ids), self.block_size)
+            self.pool.grow(r, n_tok, self.block_size)
             batch.append(self.waiting.pop(0))
-            tokens += len(r.prompt_ids)
+            tokens += n_tok
         return batch
 
     def _make_room(self) -> None:
         """Before a decode step: if the free lists cannot take the blocks the running sequences are about to
-        need, the most recently admitted sequences are preempted in recompute mode (blocks released, generated
-        tokens dropped, back to the head of the queue), as the reference does when it runs out of blocks
-        (additional_designs/core/aptserve_scheduler.py:2118-2130)."""
+        need, the most recently admitted sequences are preempted in recompute mode as the reference does when it
+        runs out of blocks (additional_designs/core/aptserve_scheduler.py:2118-2130, `_preempt_by_recompute`):
+        the blocks are released and the computed-token count starts over, but the generated tokens are kept
+        (the next prompt step of the request runs over prompt + outputs), the request falls back to the K/V
+        cache (`use_hidden = False`) and goes to the head of the queue."""
         while self.running:
             need_p = need_s = 0
             for r in self.running:
@@ -163,7 +174,7 @@ class StepLoop:
                 raise RuntimeError("the block pool cannot hold a single sequence of this length")
             victim = self.running.pop()
             self.pool.release(victim)
-            victim.generated = []
+            victim.use_hidden = False
             self.waiting.insert(0, victim)
             self.preemptions += 1
 
@@ -190,7 +201,7 @@ class StepLoop:
                                      [r.block_table for r in batch], [r.shared_table for r in batch],
                                      self.block_size, self.device)
         if is_prompt:
-            ids = np.concatenate([r.prompt_ids for r in batch])
+            ids = np.concatenate([r.token_ids for r in batch])
         else:
             ids = np.fromiter((r.generated[-1] for r in batch), dtype=np.int64, count=len(batch))
         input_ids = torch.from_numpy(ids).to(self.device, non_blocking=True)

@@ -192,6 +192,36 @@ struct ResolvedGatherOp {
   }
 };
 
+// The cache traffic of one decode layer as a single launch: the holder assembly of ResolvedGatherOp (rows
+// [0, n_rows)), the stores of the newest hidden rows ([n_rows, n_rows + n_store)) and, behind them, the newest
+// K and V rows of the K/V-cached sequences (item = 2*i + plane over kv_use_input).  A K or V row has the width
+// of a hidden row (heads * head_size), so all three kinds share one segment grid.
+struct DecodeStepOp {
+  static constexpr int kChunks = 1;
+  ResolvedGatherOp g;
+  const char* key; const char* value; char* k_cache; char* v_cache;
+  const int64_t* kv_use_input; const int64_t* new_token_slot;
+  int64_t n_kv, key_stride_b, value_stride_b, block_stride_b, row_b, num_blocks;
+  BlockSplit split;
+  __device__ RowDesc operator()(int64_t i) const {
+    const int64_t n_g = g.n_rows + g.n_store;
+    if (i < n_g) return g(i);
+    RowDesc r{nullptr, nullptr};
+    const int64_t item = i - n_g;
+    const int64_t b = kv_use_input[item >> 1];
+    if (b < 0 || b >= g.n_inputs) return r;
+    const int64_t slot = new_token_slot[b];
+    if (slot < 0) return r;
+    int64_t blk, in_blk;
+    split(slot, blk, in_blk);
+    if (blk >= num_blocks) return r;
+    const int64_t off = blk * block_stride_b + in_blk * row_b;
+    if (item & 1) { r.src = value + b * value_stride_b; r.dst = v_cache + off; }
+    else          { r.src = key + b * key_stride_b;     r.dst = k_cache + off; }
+    return r;
+  }
+};
+
 // item = 2*t + plane (0 = K, 1 = V)
 struct KvScatterOp {
   static constexpr int kChunks = 1;
@@ -487,53 +517,6 @@ int dispatch_kv_scatter_fp8(const void* key, const void* value, void* key_cache,
   }
 }
 
-// Plain streams in the shape of the row movers: a workgroup owns 256 * U consecutive 16-byte chunks and every
-// thread moves U of them (all loads, then all stores); no loop, workgroups are dispatched in address order.
-template <int U>
-__global__ __launch_bounds__(kMaxThreads) void copy_bytes_kernel(VecOf<16>::type* __restrict__ dst,
-                                                                  const VecOf<16>::type* __restrict__ src,
-                                                                  int64_t n_vec) {
-  const int64_t base = (int64_t)blockIdx.x * (kMaxThreads * U) + threadIdx.x;
-  VecOf<16>::type v[U];
-#pragma unroll
-  for (int j = 0; j < U; ++j)
-    if (base + j * kMaxThreads < n_vec) v[j] = __builtin_nontemporal_load(src + base + j * kMaxThreads);
-#pragma unroll
-  for (int j = 0; j < U; ++j)
-    if (base + j * kMaxThreads < n_vec) __builtin_nontemporal_store(v[j], dst + base + j * kMaxThreads);
-}
-
-template <int U>
-__global__ __launch_bounds__(kMaxThreads) void read_bytes_kernel(uint32_t* __restrict__ sink,
-                                                                  const VecOf<16>::type* __restrict__ src,
-                                                                  int64_t n_vec) {
-  const int64_t base = (int64_t)blockIdx.x * (kMaxThreads * U) + threadIdx.x;
-  uint32_t x = 0;
-  VecOf<16>::type v[U];
-#pragma unroll
-  for (int j = 0; j < U; ++j) {
-    v[j] = VecOf<16>::type{0u, 0u, 0u, 0u};
-    if (base + j * kMaxThreads < n_vec) v[j] = __builtin_nontemporal_load(src + base + j * kMaxThreads);
-  }
-#pragma unroll
-  for (int j = 0; j < U; ++j) x ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
-  if (x == 0x9e3779b9u && sink) *sink = x;  // keeps the loads alive; practically never taken
-}
-
-template <int U>
-__global__ __launch_bounds__(kMaxThreads) void fill_bytes_kernel(VecOf<16>::type* __restrict__ dst, int64_t n_vec,
-                                                                  uint32_t seed) {
-  const int64_t base = (int64_t)blockIdx.x * (kMaxThreads * U) + threadIdx.x;
-#pragma unroll
-  for (int j = 0; j < U; ++j) {
-    const int64_t i = base + j * kMaxThreads;
-    // not a constant pattern: what the memory sustains depends on the data
-    const uint32_t h = ((uint32_t)i * 2654435761u) ^ seed;
-    const VecOf<16>::type v = {h, h * 0x85ebca6bu, h ^ 0xc2b2ae35u, h * 0x27d4eb2fu};
-    if (i < n_vec) __builtin_nontemporal_store(v, dst + i);
-  }
-}
-
 }  // namespace
 }  // namespace aps
 
@@ -634,6 +617,46 @@ int aps_gather_hidden_rows(void* holder, const void* hidden_states, void* paged_
                                    (uint64_t)(holder_stride * e), (uint64_t)(hidden_stride * e),
                                    (uint64_t)(slot_stride * e), (uint64_t)(hidden_size * e)});
   return launch_rows(op, n_rows + n_store, hidden_size * e, vb, (hipStream_t)stream);
+}
+
+int aps_decode_step_cache_ops(void* holder, const void* hidden_states, void* paged_cache, const int64_t* holder_src,
+                              int64_t n_rows, const int64_t* slot_mapping, const int64_t* hidden_cache_use_input,
+                              const int64_t* hidden_cache_store_tot, int64_t n_store, int64_t num_inputs,
+                              int64_t hidden_size, int64_t holder_stride, int64_t hidden_stride, int64_t slot_stride,
+                              int64_t num_slots, const void* key, const void* value, void* key_cache,
+                              void* value_cache, const int64_t* kv_cache_use_input, const int64_t* new_token_slot,
+                              int64_t n_kv, int64_t key_stride, int64_t value_stride, int block_size,
+                              int64_t block_stride, int64_t num_blocks, int elem_size, aps_stream_t stream) {
+  if (n_rows < 0 || n_store < 0 || n_kv < 0 || num_inputs < 0 || hidden_size < 0 || !valid_elem(elem_size))
+    return APS_ERR_INVALID_ARG;
+  if (n_rows + n_store + n_kv == 0 || hidden_size == 0) return APS_OK;
+  if ((n_rows || n_store) && (!holder || !hidden_states || !paged_cache)) return APS_ERR_INVALID_ARG;
+  if (n_rows && !holder_src) return APS_ERR_INVALID_ARG;
+  if (n_store && (!slot_mapping || !hidden_cache_use_input || !hidden_cache_store_tot)) return APS_ERR_INVALID_ARG;
+  if ((n_rows || n_store) &&
+      (holder_stride < hidden_size || hidden_stride < hidden_size || slot_stride < hidden_size))
+    return APS_ERR_INVALID_ARG;
+  if (n_kv) {
+    if (!key || !value || !key_cache || !value_cache || !kv_cache_use_input || !new_token_slot || block_size <= 0)
+      return APS_ERR_INVALID_ARG;
+    if (key_stride < hidden_size || value_stride < hidden_size || block_stride < hidden_size * block_size)
+      return APS_ERR_INVALID_ARG;
+  }
+  const int64_t e = elem_size;
+  DecodeStepOp op{ResolvedGatherOp{(char*)holder, (const char*)hidden_states, (char*)paged_cache, holder_src,
+                                   slot_mapping, hidden_cache_use_input, hidden_cache_store_tot, n_rows, n_store,
+                                   num_inputs, holder_stride * e, hidden_stride * e, slot_stride * e, num_slots},
+                  (const char*)key, (const char*)value, (char*)key_cache, (char*)value_cache, kv_cache_use_input,
+                  new_token_slot, n_kv, key_stride * e, value_stride * e, block_stride * e, hidden_size * e,
+                  num_blocks, BlockSplit(block_size > 0 ? block_size : 1)};
+  uint64_t bits = (uint64_t)(hidden_size * e);
+  if (n_rows || n_store)
+    bits |= addr(holder) | addr(hidden_states) | addr(paged_cache) | (uint64_t)(holder_stride * e) |
+            (uint64_t)(hidden_stride * e) | (uint64_t)(slot_stride * e);
+  if (n_kv)
+    bits |= addr(key) | addr(value) | addr(key_cache) | addr(value_cache) | (uint64_t)(key_stride * e) |
+            (uint64_t)(value_stride * e) | (uint64_t)(block_stride * e);
+  return launch_rows(op, n_rows + n_store + 2 * n_kv, hidden_size * e, common_vec_bytes({bits}), (hipStream_t)stream);
 }
 
 int aps_reshape_and_cache_flash(const void* key, const void* value, void* key_cache, void* value_cache,
@@ -786,37 +809,6 @@ int aps_swap_cache_blocks(const void* src_cache, void* dst_cache, const int64_t*
     }
   }
   return APS_OK;
-}
-
-int aps_copy_bytes(void* dst, const void* src, int64_t nbytes, aps_stream_t stream) {
-  return aps_stream_probe(0, 1, dst, src, nbytes, stream);
-}
-
-int aps_stream_probe(int mode, int chunks_per_thread, void* dst, const void* src, int64_t nbytes,
-                     aps_stream_t stream) {
-  if (nbytes < 0 || mode < 0 || mode > 2) return APS_ERR_INVALID_ARG;
-  if (chunks_per_thread != 1 && chunks_per_thread != 4) return APS_ERR_INVALID_ARG;
-  if (nbytes == 0) return APS_OK;
-  if ((mode != 2 && !src) || !dst) return APS_ERR_INVALID_ARG;
-  if (common_vec_bytes({mode == 1 ? 0 : addr(dst), addr(src), (uint64_t)nbytes}) != 16) return APS_ERR_UNSUPPORTED;
-  const int64_t n_vec = nbytes / 16;
-  const int64_t per_block = (int64_t)kMaxThreads * chunks_per_thread;
-  const int64_t grid = (n_vec + per_block - 1) / per_block;
-  if (grid >= (int64_t)1 << 31) return APS_ERR_UNSUPPORTED;
-  hipStream_t s = (hipStream_t)stream;
-  const dim3 g((unsigned)grid), b(kMaxThreads);
-  VecOf<16>::type* d = (VecOf<16>::type*)dst;
-  const VecOf<16>::type* sp = (const VecOf<16>::type*)src;
-  if (chunks_per_thread == 1) {
-    if (mode == 0) APS_LAUNCH(copy_bytes_kernel<1>, g, b, 0, s, d, sp, n_vec);
-    else if (mode == 1) APS_LAUNCH(read_bytes_kernel<1>, g, b, 0, s, (uint32_t*)dst, sp, n_vec);
-    else APS_LAUNCH(fill_bytes_kernel<1>, g, b, 0, s, d, n_vec, 0x3c003c00u);
-  } else {
-    if (mode == 0) APS_LAUNCH(copy_bytes_kernel<4>, g, b, 0, s, d, sp, n_vec);
-    else if (mode == 1) APS_LAUNCH(read_bytes_kernel<4>, g, b, 0, s, (uint32_t*)dst, sp, n_vec);
-    else APS_LAUNCH(fill_bytes_kernel<4>, g, b, 0, s, d, n_vec, 0x3c003c00u);
-  }
-  return launch_status();
 }
 
 }  // extern "C"

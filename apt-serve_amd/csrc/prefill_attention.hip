@@ -276,6 +276,8 @@ int aps_varlen_prefill_attention(void* out, const void* q, const void* k, const 
                                  int head_size, int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t out_stride,
                                  float softmax_scale, int dtype, aps_stream_t stream) {
   if (num_seqs < 0 || num_tokens < 0 || max_seqlen < 0 || num_heads <= 0 || head_size <= 0) return APS_ERR_INVALID_ARG;
+  // the running maximum is taken on raw scores and the scale folded into the exponent: a positive, finite scale only
+  if (!(softmax_scale > 0.f) || softmax_scale > 3.0e38f) return APS_ERR_INVALID_ARG;
   if (num_seqs == 0 || num_tokens == 0 || max_seqlen == 0) return APS_OK;
   if (!out || !q || !k || !v || !cu_seqlens) return APS_ERR_INVALID_ARG;
   if (dtype != APS_F16 && dtype != APS_BF16) return APS_ERR_UNSUPPORTED;

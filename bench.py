@@ -25,7 +25,7 @@ for p in (ROOT, ROOT / "apt-serve_amd"):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (seed 0 workloads), scaled by what the
 # same counters read for the 1 GiB copy kernel (x2.000 and x1.000); summary in profiles/bench_step_hbm_counters.txt
-PMC_TRAFFIC_BYTES = {"gather": 1809.9e6, "attention_f16": 1793.3e6, "attention_fp8": 898.3e6,
+PMC_TRAFFIC_BYTES = {"step": 1809.9e6, "attention_f16": 1793.3e6, "attention_fp8": 898.3e6,
                      "gemm_T4096": 878.6e6, "gemm_T16384": 2853.0e6}
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 
@@ -138,52 +138,60 @@ def main():
     kv = torch.randn(B, 2 * Hd, generator=g, device=dev).half()
     key, value = (x.view(B, H, D) for x in kv.chunk(2, -1))
     holder = torch.empty(T, Hd, dtype=torch.float16, device=dev)
-    kv_seq_idx = torch.tensor([i for i, h in enumerate(batch.use_hidden) if not h], dtype=torch.int64, device=dev)
-    new_slots = torch.full((B,), -1, dtype=torch.int64, device=dev)
-    new_slots[kv_seq_idx] = md.slot_mapping[md.kv_cache_use_tot]
+    kv_seq_idx, new_slots = md.kv_cache_use_input, md.new_token_slot
 
     write_bytes = n_kv_seqs * 2 * (2 * Hd * 2) + n_hidden_seqs * 2 * (Hd * 2)   # read + write of each new row
     gather_bytes = n_hidden_rows * 2 * (Hd * 2)                                 # read + write of each context row
     step_bytes = write_bytes + gather_bytes
 
-    gather_events = []
-
-    def step(timed=False):
-        # new K/V rows of the K/V-cached sequences -> private cache
-        ops.reshape_and_cache_flash(key, value, cache[0], cache[1], new_slots, "auto", token_idx=kv_seq_idx)
-        # new hidden rows -> hidden blocks, and the holder of every row that is re-projected
-        if timed:
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-        ops.gather_hidden_rows(holder, hs, cache, md.holder_src, md.slot_mapping, md.hidden_cache_use_input,
-                               md.hidden_cache_store_tot)
-        if timed:
-            b.record()
-            gather_events.append((a, b))
+    def step():
+        # one launch: new hidden rows -> hidden blocks, new K/V rows of the K/V-cached sequences -> private
+        # cache, and the holder of every row that is re-projected
+        ops.decode_step_cache_ops(holder, hs, cache, md.holder_src, md.slot_mapping, md.hidden_cache_use_input,
+                                  md.hidden_cache_store_tot, key, value, md.kv_cache_use_input, md.new_token_slot)
 
     if args.pmc_calibrate:
+        from aptserve_hip import probes
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)
         for _ in range(3):
-            ops.copy_bytes(dst, src)
+            probes.copy_bytes(dst, src)
         torch.cuda.synchronize()
         del src, dst
 
+    # events are created and recorded once before the timed region: creating one costs a runtime call
+    span = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+    n_launch_timed = max(args.steps, 200)
+    launch_events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                     for _ in range(n_launch_timed)]
+    for e in (*span, *launch_events[0]):
+        e.record()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # ---- the timed region: exactly `steps` steps, nothing but their launches between the two synchronisations
     t0 = time.perf_counter()
+    span[0].record()
     for _ in range(args.steps):
-        step(timed=True)
+        step()
+    span[1].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ms_per_step_events = span[0].elapsed_time(span[1]) / args.steps
     step_gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
-    gather_ms = sum(a.elapsed_time(b) for a, b in gather_events) / len(gather_events)
-    # the gather launch also carries the B newest rows (upd) and the hidden stores; count only the rows
-    # gathered and the hidden stores, read once and written once
-    gather_alg = gather_bytes + n_hidden_seqs * 2 * (Hd * 2)
-    achieved = gather_alg / gather_ms / 1e6
+    # ---- second pass, outside the timed region: every launch between its own pair of HIP events (on the stream
+    # the kernel is launched on: torch's current stream is the one ops hands to the library)
+    for a, b in launch_events:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    launch_ms = [a.elapsed_time(b) for a, b in launch_events]
+    avg_launch_ms = sum(launch_ms) / len(launch_ms)
+    # algorithmic bytes of the launch = the step's: every gathered row, stored hidden row and new K/V row read
+    # once and written once (the B newest rows that also enter the holder are not counted)
+    achieved = step_bytes / avg_launch_ms / 1e6
 
     result = {
         "metric": "hybrid-cache write/gather GB/s + decode attn tokens/s, OPT-13B shapes, 1 MI355X",
@@ -194,18 +202,23 @@ def main():
                                "decode batch 256 (128 K/V + 128 hidden), lognormal(6.2,0.8) contexts in [16,2048]",
                    "seed": args.seed, "hidden_rows_gathered": n_hidden_rows, "rows_total": T,
                    "step_bytes": step_bytes, "write_bytes": write_bytes, "gather_bytes": gather_bytes,
-                   "launches_per_step": 2},
+                   "launches_per_step": 1},
+        "ms_per_step_hip_events": ms_per_step_events,
+        "timing": "ms_per_step: host clock around the %d steps between two synchronisations; "
+                  "ms_per_step_hip_events: one HIP event pair around the same steps on the stream" % args.steps,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": PMC_TRAFFIC_BYTES["gather"] if args.seed == 0 else None,
-                     "kernel": "row_mover<16,ResolvedGatherOp>",
-                     "algorithmic_bytes_per_launch": gather_alg, "avg_launch_ms": gather_ms},
+                     "traffic": PMC_TRAFFIC_BYTES["step"] if args.seed == 0 else None,
+                     "kernel": "row_mover<16,1,DecodeStepOp>",
+                     "algorithmic_bytes_per_launch": step_bytes, "avg_launch_ms": avg_launch_ms,
+                     "median_launch_ms": median(launch_ms), "launches_timed": len(launch_ms)},
     }
 
     want = set() if args.no_extras else set(x for x in args.extras.split(",") if x)
     if want:
         extras = {}
         if "literal" in want:
+            gather_alg = gather_bytes + n_hidden_seqs * 2 * (Hd * 2)   # without the K/V rows, which it does not move
             # the reference's own operator sequence through the drop-in module (no caller change): hidden_to_cache,
             # torch.zeros holder, index_put of the newest rows, cache_to_hidden over every cached row
             # (additional_designs/model_executor/models/aptserve_opt.py:108-121)
@@ -331,8 +344,8 @@ def issue_mix_figures(torch, dev):
     v_fma_f32]).  The prompt attention's softmax is vector work of about the size of its matrix work: the two
     overlap when they alternate inside a wavefront's instruction stream and hardly when wavefronts issue them in
     runs, which is how a compiler-scheduled attention loop issues them."""
-    from aptserve_hip import _lib
-    lib = _lib.load()
+    from aptserve_hip import probes
+    lib = probes.load()
     st = torch.cuda.current_stream().cuda_stream
     sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
     zeros = torch.zeros(16384, dtype=torch.float16, device=dev)
@@ -377,8 +390,8 @@ def write_figures(torch, ops, dev, seed, block_contiguous=False):
 def stream_ceiling_figures(torch, dev):
     """What plain streams sustain on this GPU (aps_stream_probe, 2 GiB of random fp16, one 16-byte chunk per
     thread, workgroups in address order): the ceilings the row movers and the attention are held against."""
-    from aptserve_hip import _lib
-    lib = _lib.load()
+    from aptserve_hip import probes
+    lib = probes.load()
     nb = 2 << 30
     a = torch.empty(nb // 2, dtype=torch.float16, device=dev)
     for i in range(0, nb // 2, 1 << 28):
@@ -414,8 +427,8 @@ def mfma_ceiling_figures(torch, dev):
     """What the matrix cores sustain with nothing else running (aps_mfma_probe: 256 workgroups of 4 wavefronts,
     operands in registers): under N(0,1) operands the part lowers its clock to stay inside its power limit, and how
     far depends on the instruction shape.  The re-projection GEMM is held against the figure of its own shape."""
-    from aptserve_hip import _lib
-    lib = _lib.load()
+    from aptserve_hip import probes
+    lib = probes.load()
     st = torch.cuda.current_stream().cuda_stream
     sink = torch.empty(256 * 256, dtype=torch.float32, device=dev)
     iters = 3200
@@ -636,9 +649,9 @@ def cost_coef_figures(torch, dev):
     """The scheduler's profit coefficient (additional_designs/engine/aptserve_llm_engine.py:316-354: 40 layers of
     the QKV product timed over growing token counts, slope over 16-token blocks / 5) at OPT-13B shape, measured
     on this library's two data flows and with the reference's own recipe (F.linear, whose operands the reference
-    creates in fp32; fp16 beside it).  Every fourth point of the reference's range(1, 4101, 100)."""
+    creates in fp32; fp16 beside it), on the reference's own sampling range(1, 4101, 100)."""
     from aptserve_hip import cost_model
-    counts = tuple(range(1, 4101, 400))
+    counts = tuple(range(1, 4101, 100))
     out = {"token_counts": list(counts), "layers": 40, "block_size": 16, "unit": "seconds per block / 5"}
     for name, kw in (("reprojection", dict(mode="reprojection")), ("absorbed", dict(mode="absorbed")),
                      ("reference_recipe_F_linear_fp16", dict(mode="reference_recipe")),

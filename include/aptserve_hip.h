@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define APS_ABI_VERSION 5
+#define APS_ABI_VERSION 6
 
 typedef void* aps_stream_t; /* a hipStream_t; NULL = the null stream */
 
@@ -121,6 +121,35 @@ int aps_gather_hidden_rows(void* holder, const void* hidden_states,
                            int64_t hidden_stride, int64_t slot_stride,
                            int64_t num_slots, int elem_size,
                            aps_stream_t stream);
+
+/* The cache traffic of one decode layer in ONE launch: the holder assembly and
+ * hidden stores of aps_gather_hidden_rows (same arguments, same result) plus the
+ * write of the newest K/V rows of the K/V-cached sequences.  Replaces the call
+ * sequence model_executor/models/aptserve_opt.py:108-121 (hidden_to_cache, zero
+ * fill, index_put, cache_to_hidden) and the reshape_and_cache_flash of the new
+ * K/V rows, attention/backends/aptserve_flash_attn.py:338-345:
+ *   for i in [0, n_kv): b = kv_cache_use_input[i]; s = new_token_slot[b];
+ *     key_cache[s/BS, s%BS] = key[b];  value_cache[s/BS, s%BS] = value[b]
+ * (s < 0, s >= num_blocks*BS or b outside [0, num_inputs) skipped).  key/value
+ * [num_inputs, hidden_size] with row strides key_stride / value_stride; the
+ * caches [num_blocks, block_size, hidden_size] with block stride block_stride
+ * (they may be the two planes of paged_cache); kv_cache_use_input and
+ * new_token_slot as aps_build_decode_metadata writes them.  A K or V row has the
+ * width of a hidden row (hidden_size = heads * head_size) and the dtype of the
+ * hidden rows.  Bit-identical to aps_reshape_and_cache_flash (token_idx =
+ * kv_cache_use_input) followed by aps_gather_hidden_rows; the destinations of
+ * the three kinds of rows are disjoint, so no order between them is needed. */
+int aps_decode_step_cache_ops(
+    void* holder, const void* hidden_states, void* paged_cache,
+    const int64_t* holder_src, int64_t n_rows, const int64_t* slot_mapping,
+    const int64_t* hidden_cache_use_input,
+    const int64_t* hidden_cache_store_tot, int64_t n_store, int64_t num_inputs,
+    int64_t hidden_size, int64_t holder_stride, int64_t hidden_stride,
+    int64_t slot_stride, int64_t num_slots, const void* key, const void* value,
+    void* key_cache, void* value_cache, const int64_t* kv_cache_use_input,
+    const int64_t* new_token_slot, int64_t n_kv, int64_t key_stride,
+    int64_t value_stride, int block_size, int64_t block_stride,
+    int64_t num_blocks, int elem_size, aps_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * K/V row scatter into [num_blocks, block_size, H, D] caches.
@@ -246,7 +275,10 @@ int aps_paged_decode_attention(
  * array: calls that overlap in time on the same GPU (two streams, two
  * threads) race; calls on one stream are ordered and safe.  Nothing in the
  * array has to start at zero (every partial that is read was written by the
- * same call), so it is never cleared. */
+ * same call), so it is never cleared.  The first call on a device looks the
+ * array's device address up (hipGetSymbolAddress, which may load the library's
+ * code object): make that call outside a stream capture; every later call on
+ * the device only enqueues kernels and may be captured. */
 #define APS_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)
 int aps_paged_decode_attention_static(
     void* out, const void* q, const void* k_cache, const void* v_cache,
@@ -273,6 +305,8 @@ int aps_paged_decode_attention_static(
  * is skipped (its rows of out are not written).  max_seqlen: host-side bound
  * of the sequence lengths (sizes the grid): queries at positions >= max_seqlen
  * of a longer sequence are not computed, so it must not be an underestimate.
+ * softmax_scale must be positive and finite (the kernel takes the running
+ * maximum on unscaled scores); anything else is APS_ERR_INVALID_ARG.
  * ------------------------------------------------------------------------ */
 int aps_varlen_prefill_attention(void* out, const void* q, const void* k,
                                  const void* v, const int32_t* cu_seqlens,
@@ -497,39 +531,6 @@ int aps_swap_cache_blocks(const void* src_cache, void* dst_cache,
                           int64_t n_pairs, int64_t src_num_blocks,
                           int64_t dst_num_blocks, int64_t block_bytes,
                           aps_stream_t stream);
-
-/* Plain device copy of nbytes (16-byte aligned pointers): the known-size
- * kernel that hardware counters of the kernels above are scaled against. */
-int aps_copy_bytes(void* dst, const void* src, int64_t nbytes,
-                   aps_stream_t stream);
-
-/* Plain streams over nbytes (16-byte aligned), for measuring what the part
- * sustains: mode 0 copies src to dst (as aps_copy_bytes), mode 1 only reads
- * src (dst: 4 bytes that are practically never written), mode 2 only writes
- * dst with a non-constant pattern (src unused).  chunks_per_thread 1 or 4
- * 16-byte chunks in flight per thread.  The ceilings the row movers and the
- * attention are compared against come from these. */
-int aps_stream_probe(int mode, int chunks_per_thread, void* dst,
-                     const void* src, int64_t nbytes, aps_stream_t stream);
-
-/* Matrix-core instructions alone, for measuring what the part sustains under
- * the power they draw: `workgroups` workgroups of 4 wavefronts (one per SIMD)
- * run `iters` rounds of 16 v_mfma_f32_32x32x16 (shape 0) or 32
- * v_mfma_f32_16x16x32 (shape 1) on operands kept in registers, which they load
- * once from `operands` (32 KiB of f16 / bf16 values, 16-byte aligned: random
- * values make the part throttle, zeros do not).  Flops of a launch:
- * workgroups * 4 * iters * 2 * 16 * 32*32*16.  `sink` receives one float per
- * thread (workgroups * 256 floats).  Shapes 2..6 measure how a SIMD issues
- * matrix and vector instructions side by side; a round is 16
- * v_mfma_f32_32x32x16 and / or 16 vector units (one v_exp_f32 and three
- * v_fma_f32 on registers): 2 the two kinds alternating instruction by
- * instruction, 3 all the MFMAs and then all the vector units, 4 the vector
- * units alone, all with one wavefront per SIMD; 5 and 6 are 2 and 3 with two
- * wavefronts per SIMD (workgroups of 8 wavefronts; sink: workgroups * 512
- * floats).  No counterpart in the reference: the ceilings the re-projection
- * GEMM and the prompt attention are compared against come from this. */
-int aps_mfma_probe(int shape, int dtype, const void* operands, void* sink,
-                   int workgroups, int iters, aps_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -7,22 +7,35 @@ import subprocess
 
 import pytest
 
-from aptserve_hip import _lib
+from aptserve_hip import _lib, probes
+
+LIBS = [(_lib.LIB_PATH, _lib.HEADER), (probes.LIB_PATH, probes.HEADER)]
 
 
-def test_header_parses_and_every_symbol_is_exported():
-    protos = _lib.parse_header()
-    assert "aps_hidden_to_cache" in protos and "aps_cache_to_hidden" in protos
-    assert "aps_mixed_kv_to_cache" in protos
-    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+@pytest.mark.parametrize("lib_path,header", LIBS, ids=["product", "probes"])
+def test_header_parses_and_every_symbol_is_exported(lib_path, header):
+    protos = _lib.parse_header(header)
+    if header == _lib.HEADER:
+        assert "aps_hidden_to_cache" in protos and "aps_cache_to_hidden" in protos
+        assert "aps_mixed_kv_to_cache" in protos and "aps_decode_step_cache_ops" in protos
+    lib = ctypes.CDLL(str(lib_path))
     for name in protos:
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
 
 
-def test_no_undeclared_exports():
-    out = subprocess.run(["nm", "-D", "--defined-only", str(_lib.LIB_PATH)], capture_output=True, text=True).stdout
+@pytest.mark.parametrize("lib_path,header", LIBS, ids=["product", "probes"])
+def test_no_undeclared_exports(lib_path, header):
+    out = subprocess.run(["nm", "-D", "--defined-only", str(lib_path)], capture_output=True, text=True).stdout
     exported = set(re.findall(r" T (aps_\w+)", out))
-    assert exported == set(_lib.parse_header()), "header and library disagree about the ABI"
+    assert exported == set(_lib.parse_header(header)), "header and library disagree about the ABI"
+
+
+def test_product_abi_holds_no_measurement_kernels():
+    """The library a maintainer of the reference binds exports operators only: the copy / stream / matrix-core
+    probes of the benchmark live in a library of their own."""
+    protos = set(_lib.parse_header())
+    assert not {n for n in protos if "probe" in n or n == "aps_copy_bytes"}
+    assert {"aps_copy_bytes", "aps_stream_probe", "aps_mfma_probe"} == set(_lib.parse_header(probes.HEADER))
 
 
 def test_loader_sets_prototypes_and_version():
@@ -41,17 +54,21 @@ def test_signatures_carry_no_torch_types():
 def test_argument_errors_return_without_launching():
     lib = _lib.load()
     # negative sizes / null pointers are rejected on the host, before any GPU call
-    assert lib.aps_copy_bytes(None, None, -1, None) == -1
-    assert lib.aps_copy_bytes(None, None, 0, None) == 0
+    pl = probes.load()
+    assert pl.aps_copy_bytes(None, None, -1, None) == -1
+    assert pl.aps_copy_bytes(None, None, 0, None) == 0
     assert lib.aps_hidden_to_cache(None, None, None, None, None, 0, 768, 768, 768, 0, 0, 0, 2, None) == 0
     assert lib.aps_hidden_to_cache(None, None, None, None, None, 4, 768, 768, 768, 0, 0, 0, 2, None) == -1
     assert lib.aps_hidden_to_cache(None, None, None, None, None, 4, 768, 768, 768, 0, 0, 0, 3, None) == -1
+    # prompt attention: a zero, negative or non-finite softmax scale is rejected on the host
+    for bad in (0.0, -1.0, float("nan"), float("inf")):
+        assert lib.aps_varlen_prefill_attention(16, 16, 16, 16, 16, 1, 8, 8, 2, 64, 128, 128, 128, 128, bad, 0, None) == -1
     # the matrix-core probe: unknown shape / dtype / null buffers are errors, an empty launch is not
-    assert lib.aps_mfma_probe(7, 0, 16, 16, 1, 1, None) == -1
-    assert lib.aps_mfma_probe(-1, 0, 16, 16, 1, 1, None) == -1
-    assert lib.aps_mfma_probe(0, 5, 16, 16, 1, 1, None) == -1
-    assert lib.aps_mfma_probe(0, 0, None, None, 1, 1, None) == -1
-    assert lib.aps_mfma_probe(1, 0, 16, 16, 0, 1, None) == 0
+    assert pl.aps_mfma_probe(7, 0, 16, 16, 1, 1, None) == -1
+    assert pl.aps_mfma_probe(-1, 0, 16, 16, 1, 1, None) == -1
+    assert pl.aps_mfma_probe(0, 5, 16, 16, 1, 1, None) == -1
+    assert pl.aps_mfma_probe(0, 0, None, None, 1, 1, None) == -1
+    assert pl.aps_mfma_probe(1, 0, 16, 16, 0, 1, None) == 0
 
 
 def test_linear_workspace_planning_is_host_only_and_consistent():

@@ -279,6 +279,58 @@ def test_resolved_gather_zero_fills_padding_rows(dev):
     assert torch.equal(g.cpu().view(-1, 8)[6], hs[0])
 
 
+@pytest.mark.parametrize("seed,frac", [(0, 0.5), (1, 0.3), (2, 1.0), (3, 0.0)])
+@pytest.mark.parametrize("H,D,dtype", [(2, 4, torch.float16), (12, 64, torch.bfloat16), (40, 128, torch.float16),
+                                       (3, 8, torch.float32)])
+def test_decode_step_cache_ops_one_launch(dev, seed, frac, H, D, dtype):
+    """One launch for a decode layer's cache traffic: hidden stores, holder assembly and the newest K/V rows of
+    the K/V-cached sequences, against the oracle's separate operators (aptserve_opt.py:108-121,
+    aptserve_flash_attn.py:338-345); key / value are the chunk views of one [B, 2*Hd] projection."""
+    from aptserve_hip import metadata
+    N, BS = 64, 16
+    b = workloads.small_decode_batch(seed, 9, 90, frac, N)
+    md = oracle_metadata(b)
+    gmd = metadata.build_from_batch(b, dev)
+    B, T, Hd = len(b.seq_lens), md["num_tot_tokens"], H * D
+    hs = randn((B, Hd), seed, dtype)
+    kv = randn((B, 2 * Hd), seed + 7, dtype)
+    k, v = (x.view(B, H, D) for x in kv.chunk(2, -1))
+    cache = sentinel_cache((2, N, BS, H, D), dtype)
+    ref = cache.clone()
+    sm = t64(md["slot_mapping"])
+    O.hidden_to_cache(hs, ref, sm, t64(md["hidden_cache_use_input"]), t64(md["hidden_cache_store_tot"]))
+    holder_ref = O.assemble_hidden_holder(hs, ref, sm, T, t64(md["hidden_holder_upd"]),
+                                          t64(md["hidden_cache_use_tot"]))
+    seq_idx = torch.tensor([i for i, h in enumerate(b.use_hidden) if not h], dtype=torch.int64)
+    O.reshape_and_cache_flash(k[seq_idx], v[seq_idx], ref[0], ref[1], sm[t64(md["kv_cache_use_tot"])], "auto")
+    g = cache.to(dev)
+    holder = sentinel_cache((T, Hd), dtype, seed=5).to(dev)
+    dkv = kv.to(dev)
+    dk, dv = dkv.chunk(2, -1)
+    ops.decode_step_cache_ops(holder, hs.to(dev), g, gmd.holder_src, gmd.slot_mapping, gmd.hidden_cache_use_input,
+                              gmd.hidden_cache_store_tot, dk, dv, gmd.kv_cache_use_input, gmd.new_token_slot)
+    assert bits_equal(holder, holder_ref)
+    assert bits_equal(g, ref)
+
+
+def test_decode_step_cache_ops_skips_bad_rows(dev):
+    """Padding slots, out-of-range sequence positions and slots past the cache are skipped, not written."""
+    H, D, N, BS = 1, 8, 4, 16
+    cache = sentinel_cache((2, N, BS, H, D))
+    g = cache.to(dev)
+    hs, k, v = randn((3, 8), 0), randn((3, 8), 1), randn((3, 8), 2)
+    holder = sentinel_cache((2, 8), seed=5).to(dev)
+    src = t64([5, -2], dev)                       # a cache slot, then row 1 of the inputs
+    ops.decode_step_cache_ops(holder, hs.to(dev), g, src, t64([5, 9], dev), t64([], dev), t64([], dev), k.to(dev),
+                              v.to(dev), t64([0, 2, 7, -1, 1], dev), t64([3, -1, N * BS], dev))
+    ref = cache.clone()
+    ref[0].view(-1, 8)[3] = k[0]
+    ref[1].view(-1, 8)[3] = v[0]
+    assert bits_equal(g, ref)
+    h = holder.cpu()
+    assert torch.equal(h[0], cache.view(-1, 8)[5]) and torch.equal(h[1], hs[1])
+
+
 # ---------------------------------------------------------------- K/V writes
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
@@ -448,6 +500,14 @@ def test_config2_write_and_gather_opt13b_full_size(dev):
     rows = torch.cat([slots, slots + N * BS])
     assert bits_equal(g.view(-1, Hd)[rows.to(dev)], ref.view(-1, Hd)[rows])
     assert int(g.view(torch.int16).sum(dtype=torch.int64)) == int(ref.view(torch.int16).sum(dtype=torch.int64))
+    # the whole step as one launch on a second copy of the initial cache: same cache bytes, same holder
+    g3 = cheap_pattern((2, N, BS, H, D)).to(dev)
+    holder4 = torch.empty(T, Hd, dtype=torch.float16, device=dev)
+    ops.decode_step_cache_ops(holder4, dhs, g3, gmd.holder_src, gmd.slot_mapping, gmd.hidden_cache_use_input,
+                              gmd.hidden_cache_store_tot, dk, dv, gmd.kv_cache_use_input, gmd.new_token_slot)
+    assert torch.equal(g3, g)
+    del g3
+    assert bits_equal(holder4, holder_ref)
 
 
 # --------------------------------------------------------------- error paths

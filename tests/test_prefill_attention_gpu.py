@@ -67,5 +67,8 @@ def test_argument_validation(dev):
         ops.flash_attn_varlen_func(q, q, q, cu_seqlens_q=cu, max_seqlen_q=8, causal=False)
     with pytest.raises(ValueError):
         ops.flash_attn_varlen_func(q, q, q, cu_seqlens_q=cu.long(), max_seqlen_q=8)
+    for bad in (0.0, -0.125, float("nan"), float("inf")):     # the kernel's running maximum assumes a positive scale
+        with pytest.raises(ValueError):
+            ops.flash_attn_varlen_func(q, q, q, cu_seqlens_q=cu, max_seqlen_q=8, softmax_scale=bad)
     e = torch.zeros(0, 2, 64, dtype=torch.float16, device=dev)
     assert ops.flash_attn_varlen_func(e, e, e, cu_seqlens_q=cu[:1], max_seqlen_q=0).shape == (0, 2, 64)

@@ -297,8 +297,8 @@ def test_config3_kv_reprojection_opt13b(dev):
 def test_matrix_core_probe_runs_and_adds_what_it_multiplies(dev):
     """aps_mfma_probe is a measurement aid, but its kernels are real: with all-ones operands every accumulator of a
     16x16x32 product grows by 32 per round (16 per round for 32x32x16), and a thread sums all of its accumulators."""
-    from aptserve_hip import _lib
-    lib = _lib.load()
+    from aptserve_hip import probes
+    lib = probes.load()
     st = torch.cuda.current_stream().cuda_stream
     ones = torch.ones(16384, dtype=torch.float16, device=dev)
     zeros = torch.zeros(16384, dtype=torch.float16, device=dev)
@@ -318,8 +318,8 @@ def test_issue_mix_probe_shapes_compute_what_they_say(dev):
     register values per lane, two units per value and round).  With zero operands the products are zero and every
     value follows x -> fma(fma(fma(2^x, c0, c1), c0, c1), c0, c1) from 0, whatever the order of issue."""
     import numpy as np
-    from aptserve_hip import _lib
-    lib = _lib.load()
+    from aptserve_hip import probes
+    lib = probes.load()
     st = torch.cuda.current_stream().cuda_stream
     zeros = torch.zeros(16384, dtype=torch.float16, device=dev)
     iters = 3

@@ -55,7 +55,33 @@ def test_decode_growth_preempts_instead_of_running_out_of_blocks():
         small.running.append(r)
     small._make_room()                  # 4 sequences want 4 blocks, 1 is free: the newest ones are preempted
     assert small.preemptions == 2 and [r.rid for r in small.running] == [0, 1]
-    assert [r.rid for r in small.waiting] == [2, 3] and all(not r.generated and not r.block_table for r in small.waiting)
+    assert [r.rid for r in small.waiting] == [2, 3] and all(not r.block_table for r in small.waiting)
+    # recompute preemption keeps what was generated (it is re-prefilled with the prompt) and drops the hidden cache
+    assert all(r.generated == [1] and r.seq_len == 17 and len(r.token_ids) == 17 for r in small.waiting)
+
+
+def test_preempted_request_keeps_its_tokens_and_falls_back_to_the_kv_cache():
+    """additional_designs/core/aptserve_scheduler.py:2118-2130: the victim of a recompute preemption keeps its
+    output tokens, restarts its computed-token count and has use_hidden cleared; its next prompt step covers
+    prompt + outputs, so no token is generated (or counted) twice."""
+    reqs = [step_loop.Request(i, 0.0, np.arange(16, dtype=np.int64), 64, True) for i in range(3)]
+    loop = step_loop.StepLoop(None, None, [], 2, 16, "cpu")     # 2 private + 2 shared blocks
+    for r in reqs[:2]:
+        loop.pool.grow(r, 16, 16)
+        r.generated = [100 + r.rid]
+        loop.running.append(r)
+    # each hidden sequence now needs a second shared block: none is free, so the newer one is preempted
+    loop._make_room()
+    assert loop.preemptions == 1 and [r.rid for r in loop.running] == [0]
+    v = loop.waiting[0]
+    assert v.rid == 1 and v.generated == [101] and v.use_hidden is False and not v.block_table and not v.shared_table
+    assert list(v.token_ids) == list(range(16)) + [101]
+    # when it is admitted again it is sized on prompt + outputs, as a K/V sequence
+    loop.running.clear()
+    loop.pool.release(reqs[0])
+    loop.pool = step_loop.BlockPool(16)
+    batch = loop._admit()
+    assert batch == [v] and len(v.block_table) == 2 and not v.shared_table
 
 
 def test_virtual_clock_is_independent_of_measured_time():
