@@ -41,7 +41,8 @@ def _stale(obj: Path, src: Path) -> bool:
 
 
 def _compile(src: Path, obj: Path) -> None:
-    cmd = [HIPCC, *FLAGS, "-c", str(src), "-o", str(obj)]
+    # APS_EXTRA_FLAGS: additional -D switches for a one-off build (the kernels' tuning macros)
+    cmd = [HIPCC, *FLAGS, *os.environ.get("APS_EXTRA_FLAGS", "").split(), "-c", str(src), "-o", str(obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     # hipcc's host pass does not know the device-only target feature and says so
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)

@@ -17,6 +17,8 @@
 //                                                                   file, x chosen per head
 // Per cached token and layer that is 2 x Hd x 2 bytes of HBM reads and ~4*H*Hd flops, against a
 // gather, a 4*Hd*Hd-flop GEMM, a cache write and an attention read for the re-projection flow.
+#include <type_traits>
+
 #include "aps_common.h"
 #include "mfma_common.h"
 #include "row_stream_core.h"
@@ -24,10 +26,10 @@
 namespace aps {
 namespace {
 
-// ------------------------------------------------------------------ NN product with few rows
-// out[z][m][n] = alpha * sum_k A[z][m][k] * B[row(z,k)][n],  m < m_rows (tiles of 16*MT rows), k < K(z).
-// B rows are n-contiguous; row(z,k) = row_ids[row_start[z] + k] (paged rows) or z*k_fixed + k.
-// A is K-contiguous and readable (finite, normally zero) up to the next multiple of 32 in k.
+// ------------------------------------------------------------------ NN product with few rows (wide heads)
+// out[z][m][n] = alpha * sum_k A[z][m][k] * B[z*k_fixed + k][n],  m < m_rows (tiles of 16*MT rows), k < k_fixed:
+// the absorbed queries of heads wider than 128 (query_image_kernel keeps a head's whole slab of W_k in registers
+// and stops there).  B rows are n-contiguous; A is K-contiguous, row m of A is row a_row_ids[m].
 //
 // The matrix core wants, per lane, 8 consecutive k of one column.  A lane therefore loads an 8x8
 // block (8 rows k, 16 bytes = 8 columns each; the 16 lanes of a quarter-wave read 256 contiguous
@@ -35,24 +37,17 @@ namespace {
 // column 8c+j from lane (g, c).  No LDS for the data; a workgroup of 4 wavefronts covers 512 columns.
 struct NnArgs {
   const char* a; int64_t a_batch_stride_b, lda_b; int m_rows;
-  const int64_t* a_row_ids; int64_t num_a_rows;  // nullable: row m of A is row a_row_ids[m] (rows of lda_b bytes)
+  const int64_t* a_row_ids; int64_t num_a_rows;
   const char* b; int64_t b_row_stride_b, num_b_rows;
-  const int64_t* row_ids; const int64_t* row_start; int k_fixed;
+  int k_fixed;
   int64_t n;
   char* out; int64_t out_batch_stride, out_row_stride;  // elements
-  float* partial;  // non-null: fp32 partial sums [k part][batch][m_rows][n] instead of out
-  int batches, k_per_part, m_tiles;
+  int batches, m_tiles;
   float alpha;
-  const int32_t* batch_order;  // nullable: the y-th batch dispatched is batch_order[y] (longest first)
 };
 
-// 4 wavefronts per workgroup, two workgroups per CU (256 registers per wavefront: a 3-deep ring of row blocks
-// beside 96 accumulator registers).  Eight wavefronts per CU with two blocks in flight each stream faster than four
-// with three (188 against 205 us on 87 591 rows): loads return in order per wavefront, so the number of
-// independent streams counts, not only the bytes in flight.
 constexpr int kNnWaves = 4;
 constexpr int kNnRing = 3;
-constexpr int kNnMaxPart = 4096;  // rows of B per k-partition when they are addressed through row_ids
 
 template <bool BF16, int MT>
 __global__ __launch_bounds__(kNnWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void nn_few_rows_kernel(
@@ -60,25 +55,9 @@ __global__ __launch_bounds__(kNnWaves * 64) __attribute__((amdgpu_waves_per_eu(2
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int g4 = lane >> 4, c = lane & 15;
-  const int zi = blockIdx.y / g.m_tiles;
-  const int z = g.batch_order ? g.batch_order[zi] : zi;
+  const int z = blockIdx.y / g.m_tiles;
   const int m0 = (blockIdx.y % g.m_tiles) * (16 * MT);
-  int64_t rs = 0;
-  int K = g.k_fixed;
-  if (g.row_ids) {
-    rs = g.row_start[z];
-    K = (int)(g.row_start[z + 1] - rs);
-  }
-  const int kbeg = blockIdx.z * g.k_per_part;
-  const int kend = min(K, kbeg + g.k_per_part);
-  // Row ids of this partition go to LDS first: read from there they cost an LDS access instead of a global
-  // load whose result every row load would have to wait for, one after the other.
-  __shared__ __attribute__((aligned(16))) int64_t ids[kNnMaxPart];
-  if (g.row_ids) {
-    const int staged = (kend - kbeg + 31) / 32 * 32;
-    for (int i = tid; i < staged; i += kNnWaves * 64) ids[i] = kbeg + i < kend ? g.row_ids[rs + kbeg + i] : -1;
-    __syncthreads();
-  }
+  const int kend = g.k_fixed;
   const int64_t col0 = (int64_t)blockIdx.x * (kNnWaves * 128) + wave * 128 + 8 * c;
   const bool col_ok = col0 < g.n;
   const char* a_base = g.a + (int64_t)z * g.a_batch_stride_b;  // uniform; rows of a batch lie within 4 GiB of it
@@ -88,12 +67,12 @@ __global__ __launch_bounds__(kNnWaves * 64) __attribute__((amdgpu_waves_per_eu(2
   for (int ht = 0; ht < MT; ++ht) {
     const int m = m0 + 16 * ht + c;
     a_ok[ht] = m < g.m_rows;
-    int64_t arow = m;
-    if (a_ok[ht] && g.a_row_ids) {
+    int64_t arow = 0;
+    if (a_ok[ht]) {
       arow = g.a_row_ids[m];
       a_ok[ht] = arow >= 0 && arow < g.num_a_rows;
     }
-    if (!a_ok[ht]) arow = g.a_row_ids ? 0 : m0;  // a row that exists; its product is discarded
+    if (!a_ok[ht]) arow = 0;  // a row that exists; its product is discarded
     a_off[ht] = (uint32_t)(arow * g.lda_b + g4 * 16);
   }
   float4v acc[MT][8];
@@ -104,34 +83,22 @@ __global__ __launch_bounds__(kNnWaves * 64) __attribute__((amdgpu_waves_per_eu(2
 
   // Loads are unconditional (a row or column that does not exist reads row 0 / column 0 and is replaced by
   // zeros afterwards): with per-lane branches around them the wait counts before the MFMAs degrade to
-  // "everything outstanding", which serialises the two register sets.
+  // "everything outstanding", which serialises the register sets.
   const char* b_col = g.b + (col_ok ? col0 : 0) * 2;
   auto load_step = [&](int t0, u32x4(&r)[8], u32x4(&pf)[MT], uint32_t& bad) {
-    int64_t row[8];
-    if (g.row_ids) {
-      const u32x4* src = (const u32x4*)(ids + (t0 - kbeg + 8 * g4));  // 8 ids = 64 bytes, 64-byte aligned
-      const u32x4 q0 = src[0], q1 = src[1], q2 = src[2], q3 = src[3];
-      row[0] = (int64_t)q0[0] | ((int64_t)q0[1] << 32); row[1] = (int64_t)q0[2] | ((int64_t)q0[3] << 32);
-      row[2] = (int64_t)q1[0] | ((int64_t)q1[1] << 32); row[3] = (int64_t)q1[2] | ((int64_t)q1[3] << 32);
-      row[4] = (int64_t)q2[0] | ((int64_t)q2[1] << 32); row[5] = (int64_t)q2[2] | ((int64_t)q2[3] << 32);
-      row[6] = (int64_t)q3[0] | ((int64_t)q3[1] << 32); row[7] = (int64_t)q3[2] | ((int64_t)q3[3] << 32);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) row[i] = (int64_t)z * g.k_fixed + t0 + 8 * g4 + i;
-    }
     bad = 0;  // bit i: row i of this lane does not exist; applied when the block is consumed
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const bool ok = col_ok && (t0 + 8 * g4 + i < kend) && row[i] >= 0 && row[i] < g.num_b_rows;
+      const int64_t row = (int64_t)z * g.k_fixed + t0 + 8 * g4 + i;
+      const bool ok = col_ok && (t0 + 8 * g4 + i < kend) && row < g.num_b_rows;
       if (!ok) bad |= 1u << i;
-      const int64_t rr = ok ? row[i] : 0;
-      r[i] = __builtin_nontemporal_load((const u32x4*)(b_col + rr * g.b_row_stride_b));
+      r[i] = __builtin_nontemporal_load((const u32x4*)(b_col + (ok ? row : 0) * g.b_row_stride_b));
     }
 #pragma unroll
     for (int ht = 0; ht < MT; ++ht) pf[ht] = *(const u32x4*)(a_base + (a_off[ht] + (uint32_t)t0 * 2));
   };
   auto mac_step = [&](u32x4(&r)[8], u32x4(&pf)[MT], uint32_t bad) {
-    if (__builtin_amdgcn_ballot_w64(bad != 0) != 0) {  // rare: the last step of a sequence
+    if (__builtin_amdgcn_ballot_w64(bad != 0) != 0) {
 #pragma unroll
       for (int i = 0; i < 8; ++i)
         if (bad & (1u << i)) r[i] = u32x4{0u, 0u, 0u, 0u};
@@ -157,7 +124,7 @@ __global__ __launch_bounds__(kNnWaves * 64) __attribute__((amdgpu_waves_per_eu(2
   // ring of kNnRing row blocks: two steps (16 KiB per wavefront) are in flight while one is multiplied
   u32x4 r[kNnRing][8], pf[kNnRing][MT];
   uint32_t bad[kNnRing];
-  int t0 = kbeg;
+  int t0 = 0;
 #pragma unroll
   for (int d = 0; d < kNnRing - 1; ++d)
     if (t0 + 32 * d < kend) load_step(t0 + 32 * d, r[d], pf[d], bad[d]);
@@ -182,52 +149,17 @@ __global__ __launch_bounds__(kNnWaves * 64) __attribute__((amdgpu_waves_per_eu(2
     for (int i = 0; i < 4; ++i) {
       const int m = m0 + 16 * ht + 4 * g4 + i;
       if (m >= g.m_rows) continue;
-      if (g.partial) {
-        float* dst = g.partial + (((int64_t)blockIdx.z * g.batches + z) * g.m_rows + m) * g.n + col0;
-        *(float4v*)dst = float4v{acc[ht][0][i], acc[ht][1][i], acc[ht][2][i], acc[ht][3][i]};
-        *(float4v*)(dst + 4) = float4v{acc[ht][4][i], acc[ht][5][i], acc[ht][6][i], acc[ht][7][i]};
-      } else {
-        uint16_t h[8];
+      uint16_t h[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float v = acc[ht][j][i] * g.alpha;
-          h[j] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
-        }
-        u32x4 o;
-#pragma unroll
-        for (int p = 0; p < 4; ++p) o[p] = (uint32_t)h[2 * p] | ((uint32_t)h[2 * p + 1] << 16);
-        *(u32x4*)(g.out + ((int64_t)z * g.out_batch_stride + (int64_t)m * g.out_row_stride + col0) * 2) = o;
+      for (int j = 0; j < 8; ++j) {
+        const float v = acc[ht][j][i] * g.alpha;
+        h[j] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
       }
+      u32x4 o;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) o[p] = (uint32_t)h[2 * p] | ((uint32_t)h[2 * p + 1] << 16);
+      *(u32x4*)(g.out + ((int64_t)z * g.out_batch_stride + (int64_t)m * g.out_row_stride + col0) * 2) = o;
     }
-}
-
-// out[z][m][n] = alpha * sum_p partial[p][z][m][n], 4 columns per thread
-template <bool BF16>
-__global__ __launch_bounds__(256) void nn_reduce_kernel(const float* __restrict__ partial, char* out, int parts,
-                                                        int batches, int m_rows, int64_t n, int64_t out_batch_stride,
-                                                        int64_t out_row_stride, float alpha) {
-  const int64_t per_part = (int64_t)batches * m_rows * n;
-  const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
-  if (idx >= per_part) return;
-  float4v s = *(const float4v*)(partial + idx);
-  int p = 1;
-  for (; p + 3 < parts; p += 4) {  // four independent loads in flight; additions in the order of one at a time
-    const float4v v0 = *(const float4v*)(partial + p * per_part + idx);
-    const float4v v1 = *(const float4v*)(partial + (p + 1) * per_part + idx);
-    const float4v v2 = *(const float4v*)(partial + (p + 2) * per_part + idx);
-    const float4v v3 = *(const float4v*)(partial + (p + 3) * per_part + idx);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) s[i] = (((s[i] + v0[i]) + v1[i]) + v2[i]) + v3[i];
-  }
-  for (; p < parts; ++p) {
-    const float4v v = *(const float4v*)(partial + p * per_part + idx);
-    s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
-  }
-  const int64_t col = idx % n, zm = idx / n;
-  const int64_t m = zm % m_rows, z = zm / m_rows;
-  uint16_t* o = (uint16_t*)out + z * out_batch_stride + m * out_row_stride + col;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) o[i] = BF16 ? f32_to_bf16_bits(s[i] * alpha) : f32_to_f16_bits(s[i] * alpha);
 }
 
 // ------------------------------------------------------------------ scores over paged hidden rows
@@ -252,9 +184,11 @@ struct ScoreArgs {
 //                   sum works through all rows of its sequence and workgroups start in grid order: longest first
 //                   keeps the last ones short (list scheduling: within a few % of ideal instead of 20-35 % over).
 constexpr int kMaxOrderedSeqs = 4096;  // lengths are ranked out of LDS, quadratic work; larger batches balance anyway
-__global__ __launch_bounds__(256) void seq_plan_kernel(const int64_t* __restrict__ row_start, int n_seqs,
-                                                       int tile_tokens, int32_t* __restrict__ tile_start,
-                                                       int32_t* __restrict__ order) {
+__device__ __forceinline__ void plan_ragged_batch(const int64_t* __restrict__ row_start, int n_seqs, int tile_tokens,
+                                                  int32_t* __restrict__ tile_start, int32_t* __restrict__ order,
+                                                  u32x4* __restrict__ zero_row, int zero_vecs) {
+  // the row of zeros that tokens without a cached row read in the weighted sum
+  for (int i = threadIdx.x; i < zero_vecs; i += 256) zero_row[i] = u32x4{0u, 0u, 0u, 0u};
   __shared__ int32_t part[256];
   __shared__ int32_t carry;
   __shared__ int32_t lens[kMaxOrderedSeqs];
@@ -290,6 +224,116 @@ __global__ __launch_bounds__(256) void seq_plan_kernel(const int64_t* __restrict
   }
 }
 
+__global__ __launch_bounds__(256) void seq_plan_kernel(const int64_t* __restrict__ row_start, int n_seqs,
+                                                       int tile_tokens, int32_t* __restrict__ tile_start,
+                                                       int32_t* __restrict__ order, u32x4* __restrict__ zero_row,
+                                                       int zero_vecs) {
+  plan_ragged_batch(row_start, n_seqs, tile_tokens, tile_start, order, zero_row, zero_vecs);
+}
+
+// ------------------------------------------------------------------ absorbed queries
+// qt[s][h][n] = alpha * sum_d q[seq_rows[s]][h*D + d] * W_k[h*D + d][n]:  per head a product of few rows (the
+// sequences) with the head's D rows of W_k.  A wavefront owns (head, 128 columns): it loads its D x 128 slab of W_k
+// once — all loads in flight together, 32 KiB per wavefront — keeps it in registers in MFMA operand order (8x8
+// blocks transposed with v_perm_b32) and then walks the sequences 16 at a time.  W_k crosses HBM once whatever the
+// number of sequences (the generic kernel re-read it for every 48 sequences and kept 4 of its D rows per lane in
+// flight).  KS = D / 32 <= 4.  One extra workgroup (blockIdx.y == heads) plans the ragged batch for the kernels
+// that follow (the scores kernel's tile list, the weighted sum's longest-first order) instead of a launch of its own.
+struct QImageArgs {
+  const char* q; int64_t q_stride_b; const int64_t* seq_rows; int64_t num_q_rows; int n_seqs;
+  const char* w; int64_t w_stride_b;
+  int heads; int64_t hidden;
+  char* qt;
+  float alpha;
+  const int64_t* row_start; int tile_tokens; int32_t* tile_start; int32_t* order;
+  u32x4* zero_row; int zero_vecs;
+};
+
+template <bool BF16, int KS>
+__global__ __launch_bounds__(256) void query_image_kernel(const QImageArgs g) {
+  if ((int)blockIdx.y == g.heads) {
+    if (blockIdx.x == 0)
+      plan_ragged_batch(g.row_start, g.n_seqs, g.tile_tokens, g.tile_start, g.order, g.zero_row, g.zero_vecs);
+    return;
+  }
+  constexpr int D = KS * 32;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int g4 = lane >> 4, c = lane & 15;
+  const int h = blockIdx.y;
+  const int64_t col0 = (int64_t)blockIdx.x * 512 + wave * 128 + 8 * c;
+  const bool col_ok = col0 < g.hidden;
+  const char* b_col = g.w + (col_ok ? col0 : 0) * 2 + (int64_t)h * D * g.w_stride_b;
+  u32x4 tcol[KS][8];
+  {
+    u32x4 r[KS][8];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        r[ks][i] = __builtin_nontemporal_load((const u32x4*)(b_col + (int64_t)(32 * ks + 8 * g4 + i) * g.w_stride_b));
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+          tcol[ks][j][p] = __builtin_amdgcn_perm(r[ks][2 * p + 1][j >> 1], r[ks][2 * p][j >> 1], sel);
+      }
+  }
+  // A operand of a tile of 16 sequences: lane (g4, c) = sequence m0 + c, d = 32 ks + 8 g4 .. + 7
+  auto load_a = [&](int m0, u32x4(&pf)[KS], bool& ok) {
+    const int m = m0 + c;
+    int64_t row = 0;
+    ok = m < g.n_seqs;
+    if (ok) {
+      row = g.seq_rows[m];
+      ok = row >= 0 && row < g.num_q_rows;
+    }
+    const char* a = g.q + (ok ? row : 0) * g.q_stride_b + ((int64_t)h * D + 8 * g4) * 2;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) pf[ks] = *(const u32x4*)(a + ks * 64);
+  };
+  u32x4 pf[2][KS];
+  bool ok[2];
+  load_a(0, pf[0], ok[0]);
+  for (int m0 = 0; m0 < g.n_seqs; m0 += 32) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int mm = m0 + 16 * u;
+      if (mm < g.n_seqs) {
+        if (mm + 16 < g.n_seqs) load_a(mm + 16, pf[u ^ 1], ok[u ^ 1]);
+        float4v acc[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const u32x4 a = ok[u] ? pf[u][ks] : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[j] = mfma16<BF16>(a, tcol[ks][j], acc[j]);
+        }
+        if (col_ok) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int m = mm + 4 * g4 + i;
+            if (m >= g.n_seqs) continue;
+            uint16_t hh[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float v = acc[j][i] * g.alpha;
+              hh[j] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+            }
+            u32x4 o;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) o[p] = (uint32_t)hh[2 * p] | ((uint32_t)hh[2 * p + 1] << 16);
+            *(u32x4*)(g.qt + (((int64_t)m * g.heads + h) * g.hidden + col0) * 2) = o;
+          }
+        }
+      }
+    }
+  }
+}
 
 template <bool BF16, int NHT>
 __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreArgs g) {
@@ -400,81 +444,372 @@ __global__ __launch_bounds__(kScThreads) void head_proj_kernel(const HeadProjArg
     }
 }
 
-// ------------------------------------------------------------------ softmax over the tokens of a row
-// P[z][h][t] = exp2(S - max) / sum for t < L(z), 0 for L <= t < the next multiple of 32; S already carries
-// scale*log2(e).
-template <bool BF16>
-__global__ __launch_bounds__(256) void softmax_rows_kernel(float* __restrict__ s, uint16_t* __restrict__ p,
-                                                           const int64_t* __restrict__ row_start, int heads,
-                                                           int64_t lp, int parts, int64_t part_stride) {
-  // Rows up to kCached scores are summed over the K parts once, 4 tokens per thread and step with the loads of
-  // all parts of a step independent of each other, and kept in LDS for the other two passes; longer rows keep
-  // their sums in part 0 of the global buffer (a thread meets the same tokens in every pass).
-  constexpr int kCached = 4096;
-  __shared__ __attribute__((aligned(16))) float cache[kCached];
-  __shared__ float red[4];
-  const int z = blockIdx.y, h = blockIdx.x;
-  const int L = (int)min(row_start[z + 1] - row_start[z], lp);  // a sequence longer than the stated maximum: its head
-  float* row = s + ((int64_t)z * heads + h) * lp;   // 16-byte aligned: lp is a multiple of 32
-  uint16_t* out = p + ((int64_t)z * heads + h) * lp;
-  const bool in_lds = L <= kCached;
-  float mx = -INFINITY;
-  for (int t = threadIdx.x * 4; t < L; t += 1024) {
-    float4 v = *(const float4*)(row + t);
-    for (int kp = 1; kp < parts; ++kp) {
-      const float4 q = *(const float4*)(row + kp * part_stride + t);
-      v.x += q.x; v.y += q.y; v.z += q.z; v.w += q.w;
+// ------------------------------------------------------------------ softmax and weighted sum of paged rows
+// ctx[z][h][:] = sum_t softmax_t(S[z][h][:])[t] * hidden row t of sequence z, in one pass over the rows.
+//
+// A workgroup of kWsWaves wavefronts owns one sequence (or one partition of its tokens) and kWsWaves * 128
+// columns; a wavefront owns 128 columns and walks the rows 32 tokens at a time: a lane loads an 8x8 block (8
+// rows, 16 bytes = 8 columns each; 16 lanes read 256 contiguous bytes of a row), transposes it in registers with
+// v_perm_b32 and feeds 8 MFMAs per 16 heads.  The softmax is an online one, 96 tokens (a chunk = 3 steps) at a
+// time: the threads of the workgroup read the fp32 scores of the next chunk of all heads once (adding the partial
+// scores of a K-split scores pass), keep a running maximum and sum per head, and leave p = exp2(s - max) as
+// 16-bit values in LDS, where every wavefront fetches its MFMA operand — the scores are read once per workgroup
+// instead of the probabilities once per 128 columns (those redundant reads were a quarter of the traffic of the
+// kernel this replaces), and no softmax pass or probability buffer exists.  When a chunk moves a head's maximum
+// the accumulators of that head are rescaled.
+// The loop body is straight-line code: three steps, the three slots of the register ring at fixed positions, every
+// load unconditional (a row, column or token that does not exist reads a valid address and is replaced by zeros),
+// so that the compiler's wait counts before the MFMAs are exact and two steps (16 KiB per wavefront) stay in
+// flight while one is multiplied; with loads under branches it waited for all but the newest step.
+// Partitions (kparts > 1: few sequences, or sequences beyond kWsMaxPart tokens) leave unnormalised fp32 sums and
+// their (max, sum) pairs for wsum_combine_kernel.
+#ifndef APS_WS_WAVES
+#define APS_WS_WAVES 8
+#endif
+#ifndef APS_WS_RING
+#define APS_WS_RING 3
+#endif
+#ifndef APS_WS_OCC
+#define APS_WS_OCC 2
+#endif
+constexpr int kWsWaves = APS_WS_WAVES, kWsThreads = kWsWaves * 64, kWsRing = APS_WS_RING, kWsChunk = 32 * kWsRing;
+constexpr int kWsMaxPart = 4096;                  // tokens of a partition (their slots are staged in LDS)
+constexpr int kWsIds = (kWsMaxPart + kWsChunk - 1) / kWsChunk * kWsChunk + 32 * (kWsRing - 1);
+constexpr int kWsPStride = kWsChunk * 2 + 16;     // bytes between heads of a probability chunk (13 x 16: odd)
+constexpr int kWsHeadsPerPass = kWsThreads / 32;  // heads whose chunk scores the workgroup reads at a time
+
+// max over the 32 lanes of a half wave, in every lane: butterflies inside a row of 16 lanes are DPP moves
+// (quad permutes, then the mirrors of 8 and 16 lanes: a maximum does not care which partner a lane meets), the
+// last exchange between the two rows one ds_bpermute.
+__device__ __forceinline__ float half_wave_max(float x) {
+  int v = __float_as_int(x);
+#define APS_DPP_MAX(ctrl)                                                                                     \
+  v = __float_as_int(fmaxf(__int_as_float(v), __int_as_float(__builtin_amdgcn_update_dpp(v, v, ctrl, 0xf, 0xf, false))))
+  APS_DPP_MAX(0xb1);   // quad_perm [1,0,3,2]
+  APS_DPP_MAX(0x4e);   // quad_perm [2,3,0,1]
+  APS_DPP_MAX(0x141);  // row_half_mirror
+  APS_DPP_MAX(0x140);  // row_mirror
+#undef APS_DPP_MAX
+  const float y = __int_as_float(v);
+  return fmaxf(y, __shfl_xor(y, 16));
+}
+
+struct WsumArgs {
+  const float* s; int64_t s_batch_stride, s_row_stride, s_part_stride; int score_parts;  // S[part][z][h][t]
+  const char* cache; int64_t slot_stride_b, num_slots;
+  const int64_t* row_ids; const int64_t* row_start;
+  const char* zero_row;                                   // n zeros (what a token without a cached row reads)
+  int heads, m_tiles, n_seqs, k_per_part;
+  int64_t n;
+  char* out; int64_t out_batch_stride, out_row_stride;   // elements: ctx[z][h][n]
+  float* partial; float* partial_ml;                      // kparts > 1: [part][z][h][n] and [part][z][h][2]
+  const int32_t* order;                                   // nullable: the y-th sequence dispatched (longest first)
+};
+
+template <bool BF16, int MT, bool PARTS>
+__global__ __launch_bounds__(kWsThreads) __attribute__((amdgpu_waves_per_eu(APS_WS_OCC, APS_WS_OCC))) void hidden_wsum_kernel(
+    const WsumArgs g) {
+  constexpr int NJ = 16 * MT / kWsHeadsPerPass;   // score quads per thread and chunk
+  static_assert(16 * MT % kWsHeadsPerPass == 0, "heads are spread evenly over the passes");
+  __shared__ __attribute__((aligned(16))) int32_t ids[kWsIds];
+  __shared__ __attribute__((aligned(16))) char p_lds[2][16 * MT * kWsPStride];
+  __shared__ __attribute__((aligned(16))) float scale_s[2][16 * MT];
+  __shared__ __attribute__((aligned(16))) float fin_s[2][16 * MT];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int g4 = lane >> 4, c = lane & 15;
+  const int zi = blockIdx.y / g.m_tiles;
+  const int z = g.order ? g.order[zi] : zi;
+  const int m0 = (blockIdx.y % g.m_tiles) * (16 * MT);
+  const int64_t rs = g.row_start[z];
+  const int K = (int)min(g.row_start[z + 1] - rs, g.s_row_stride);  // a sequence beyond the stated maximum: its head
+  const int kbeg = blockIdx.z * g.k_per_part;
+  const int kend = min(K, kbeg + g.k_per_part);
+  const int n_tok = max(kend - kbeg, 0);
+  const int nchunks = (n_tok + kWsChunk - 1) / kWsChunk;
+  {  // slots of the partition, -1 for everything a step may touch past its end
+    const int staged = nchunks * kWsChunk + 32 * (kWsRing - 1);
+    for (int i = tid; i < staged; i += kWsThreads) {
+      int64_t slot = -1;
+      if (i < n_tok) slot = g.row_ids[rs + kbeg + i];
+      ids[i] = (slot >= 0 && slot < g.num_slots) ? (int32_t)slot : -1;
     }
-    if (in_lds) *(float4*)(cache + t) = v;
-    else if (parts > 1) *(float4*)(row + t) = v;
-    mx = fmaxf(mx, v.x);                       // tokens t+1.. past L hold finite padding of the scores kernel or
-    if (t + 1 < L) mx = fmaxf(mx, v.y);        // stale values: only tokens below L count
-    if (t + 2 < L) mx = fmaxf(mx, v.z);
-    if (t + 3 < L) mx = fmaxf(mx, v.w);
   }
+  const int64_t col0 = (int64_t)blockIdx.x * (kWsWaves * 128) + wave * 128 + 8 * c;
+  const bool col_ok = col0 < g.n;
+  const char* b_col = g.cache + (col_ok ? col0 : 0) * 2;
+  const char* z_col = g.zero_row + (col_ok ? col0 : 0) * 2;
+
+  // ---- softmax side: thread (hl, tq) owns the token quads tq + 32 qq of a chunk for the heads hl + HP * j
+  constexpr int QJ = (kWsChunk / 4 + 31) / 32;
+  const int hl = tid >> 5, tq = tid & 31;
+  const float kNegInf = -INFINITY;
+  // running maximum and sum of every (thread, head) live in LDS between chunks: the streaming steps need the
+  // registers (a spilled value costs a scratch load, whose wait drains the ring of row loads)
+  __shared__ float ml_s[2][NJ][kWsThreads];
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
-  __syncthreads();
-  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-  __syncthreads();
-  const float* src = in_lds ? cache : row;     // each thread re-reads what it wrote itself
-  float sum = 0.f;
-  for (int t = threadIdx.x * 4; t < L; t += 1024) {
-    const float4 v = *(const float4*)(src + t);
-    sum += exp2f(v.x - mx);
-    if (t + 1 < L) sum += exp2f(v.y - mx);
-    if (t + 2 < L) sum += exp2f(v.z - mx);
-    if (t + 3 < L) sum += exp2f(v.w - mx);
+  for (int j = 0; j < NJ; ++j) {
+    ml_s[0][j][tid] = kNegInf;
+    ml_s[1][j][tid] = 0.f;
   }
+  // the scores of one sequence span less than 4 GiB: a uniform base and 32-bit offsets
+  const char* s_base = (const char*)(g.s + (int64_t)z * g.s_batch_stride);
+  auto s_off = [&](int j, int ts) {
+    const int head = m0 + hl + kWsHeadsPerPass * j;
+    return (uint32_t)(((int64_t)(head < g.heads ? head : 0) * g.s_row_stride + ts) * 4);
+  };
+  // first token of quad qq of this thread in `chunk`, and where to read it: a quad past the chunk or the
+  // partition reads the row's first quad (valid memory, never used)
+  auto quad_t = [&](int chunk, int qq) { return kbeg + chunk * kWsChunk + 4 * (tq + 32 * qq); };
+  auto quad_ok = [&](int qq) { return tq + 32 * qq < kWsChunk / 4; };
+  auto fetch_s = [&](int chunk, float4v(&sv)[NJ][QJ]) {
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = sum;
+    for (int qq = 0; qq < QJ; ++qq) {
+      const int t = quad_t(chunk, qq);
+      const int ts = (quad_ok(qq) && t < kend) ? t : 0;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) sv[j][qq] = *(const float4v*)(s_base + s_off(j, ts));
+    }
+  };
+  auto store_p = [&](int chunk, int buf, float4v(&sv)[NJ][QJ], int j) {
+    {
+      const bool head_ok = m0 + hl + kWsHeadsPerPass * j < g.heads;
+      bool ok[QJ][4];
+      float cmax = kNegInf;
+#pragma unroll
+      for (int qq = 0; qq < QJ; ++qq) {
+        const int t = quad_t(chunk, qq);
+        const int ts = (quad_ok(qq) && t < kend) ? t : 0;
+        if constexpr (PARTS) {  // the partial scores of a K-split scores pass (few tiles: small batches)
+          const char* sp = s_base + s_off(j, ts);
+          const int64_t stride_b = g.s_part_stride * 4;
+          int part = 1;
+          for (; part + 3 < g.score_parts; part += 4) {  // four independent loads in flight, added in part order
+            const float4v o0 = *(const float4v*)(sp + part * stride_b);
+            const float4v o1 = *(const float4v*)(sp + (part + 1) * stride_b);
+            const float4v o2 = *(const float4v*)(sp + (part + 2) * stride_b);
+            const float4v o3 = *(const float4v*)(sp + (part + 3) * stride_b);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sv[j][qq][i] = (((sv[j][qq][i] + o0[i]) + o1[i]) + o2[i]) + o3[i];
+          }
+          for (; part < g.score_parts; ++part) {
+            const float4v o = *(const float4v*)(sp + part * stride_b);
+            sv[j][qq][0] += o[0]; sv[j][qq][1] += o[1]; sv[j][qq][2] += o[2]; sv[j][qq][3] += o[3];
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          ok[qq][i] = head_ok && quad_ok(qq) && t + i < kend;
+          cmax = fmaxf(cmax, ok[qq][i] ? sv[j][qq][i] : kNegInf);
+        }
+      }
+      cmax = half_wave_max(cmax);  // the 32 lanes of a head
+      const float m_old = ml_s[0][j][tid];
+      const float m_new = fmaxf(m_old, cmax);
+      const float scale = m_new == kNegInf ? 1.f : __builtin_amdgcn_exp2f(m_old - m_new);
+      float sum = 0.f;
+#pragma unroll
+      for (int qq = 0; qq < QJ; ++qq) {
+        uint16_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          // v_exp_f32: arguments are <= 0 here and results below 2^-126 may flush to zero
+          const float e = ok[qq][i] ? __builtin_amdgcn_exp2f(sv[j][qq][i] - m_new) : 0.f;
+          sum += e;
+          o[i] = BF16 ? f32_to_bf16_bits(e) : f32_to_f16_bits(e);
+        }
+        // no branch in this loop body (the wait counts of the row loads stay exact): a quad past the chunk goes
+        // to the spare slot behind the head's row, and all 32 lanes of a head store its (identical) scale
+        const int q_dst = quad_ok(qq) ? tq + 32 * qq : kWsChunk / 4;
+        *(uint2*)(p_lds[buf] + (hl + kWsHeadsPerPass * j) * kWsPStride + q_dst * 8) =
+            uint2{(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
+      }
+      ml_s[1][j][tid] = ml_s[1][j][tid] * scale + sum;
+      ml_s[0][j][tid] = m_new;
+      scale_s[buf][hl + kWsHeadsPerPass * j] = scale;
+    }
+  };
+
+  // ---- streaming side
+  float4v acc[MT][8];
+#pragma unroll
+  for (int ht = 0; ht < MT; ++ht)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[ht][j] = float4v{0.f, 0.f, 0.f, 0.f};
+  // rows of the step that starts at token kbeg + i0: unconditional loads; a slot of -1 (a token past the
+  // partition, a padding slot) reads the row of zeros the caller keeps for that purpose, a column past the row
+  // reads column 0 (its sums are never stored)
+  auto load_step = [&](int i0, u32x4(&r)[8]) {
+    const u32x4* src = (const u32x4*)(ids + i0 + 8 * g4);  // 8 slots = 32 bytes, 32-byte aligned
+    const u32x4 q0 = src[0], q1 = src[1];
+    const int32_t slot[8] = {(int32_t)q0[0], (int32_t)q0[1], (int32_t)q0[2], (int32_t)q0[3],
+                             (int32_t)q1[0], (int32_t)q1[1], (int32_t)q1[2], (int32_t)q1[3]};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const char* src_row = slot[i] >= 0 ? b_col + (int64_t)slot[i] * g.slot_stride_b : z_col;
+      r[i] = __builtin_nontemporal_load((const u32x4*)src_row);
+    }
+  };
+#ifndef APS_WS_ABL
+#define APS_WS_ABL 0
+#endif
+  auto mac_step = [&](u32x4(&r)[8], const char* prow) {
+    if constexpr ((APS_WS_ABL & 1) != 0) {  // timing experiment: consume the loads, no products
+      uint32_t x = 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x ^= r[i][0] ^ r[i][1] ^ r[i][2] ^ r[i][3];
+      acc[0][0][0] += __uint_as_float(x & 0xffu);
+      return;
+    }
+    u32x4 pf[MT];
+#pragma unroll
+    for (int ht = 0; ht < MT; ++ht) pf[ht] = *(const u32x4*)(prow + ht * 16 * kWsPStride);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      u32x4 tcol;  // column j of the 8x8 block: dword p = (row 2p, row 2p+1)
+      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) tcol[p] = __builtin_amdgcn_perm(r[2 * p + 1][j >> 1], r[2 * p][j >> 1], sel);
+#pragma unroll
+      for (int ht = 0; ht < MT; ++ht) acc[ht][j] = mfma16<BF16>(pf[ht], tcol, acc[ht][j]);
+    }
+  };
+
+  float4v sv[NJ][QJ];
+  // The loop has no prologue: it starts one chunk early on a ring of zeros and a buffer of zero probabilities
+  // (and prepares chunk 0 on that trip), so that the loads in flight at its head are the same on entry and on
+  // every later trip.
+  for (int i = tid; i < 16 * MT * kWsPStride / 16; i += kWsThreads)
+    ((u32x4*)p_lds[1])[i] = u32x4{0u, 0u, 0u, 0u};
+  if (tid < 16 * MT) scale_s[1][tid] = 1.f;
+  u32x4 r[kWsRing][8];
+#pragma unroll
+  for (int d = 0; d < kWsRing; ++d)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[d][i] = u32x4{0u, 0u, 0u, 0u};
+  __syncthreads();  // slots, running maxima and the zero buffer are in LDS
+  // (peeling the last chunk off without its requests was measured: the second copy of the body costs more in
+  // spilled registers than the padded requests do)
+  for (int chunk = -1; chunk < nchunks; ++chunk) {
+    const int buf = chunk & 1;
+    {  // heads whose maximum moved with this chunk: bring their sums to the new maximum
+      float4v sc[MT];
+      bool moved = false;
+#pragma unroll
+      for (int ht = 0; ht < MT; ++ht) {
+        sc[ht] = *(const float4v*)(&scale_s[buf][16 * ht + 4 * g4]);
+        moved = moved || sc[ht][0] != 1.f || sc[ht][1] != 1.f || sc[ht][2] != 1.f || sc[ht][3] != 1.f;
+      }
+      if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+        for (int ht = 0; ht < MT; ++ht)
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[ht][j][i] *= sc[ht][i];
+      }
+    }
+#pragma unroll
+    for (int st = 0; st < kWsRing; ++st) {
+      // rows of the step kWsRing - 1 ahead (before token 0 in the first trip: the padded tail of the slot list)
+      const int i0 = chunk * kWsChunk + 32 * (st + kWsRing - 1);
+      load_step(i0 >= 0 ? i0 : nchunks * kWsChunk, r[(st + kWsRing - 1) % kWsRing]);
+      // scores of the next chunk: behind the first rows of this one, so that they are old loads by the time they
+      // are used (loads return in order: waiting for a recent one would drain the ring of rows)
+      if ((APS_WS_ABL & 2) == 0 && st == 0) fetch_s(chunk + 1, sv);
+      mac_step(r[st], p_lds[buf] + c * kWsPStride + (32 * st + 8 * g4) * 2);
+      // the softmax of the next chunk, a group of heads per step, between the products of this one: on its own at
+      // the end of the chunk it is a stretch of dependent LDS and transcendental latencies in which nothing streams
+      if ((APS_WS_ABL & 2) == 0 && st >= 1) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+          if (st == 1 + j * (kWsRing - 1) / NJ) store_p(chunk + 1, buf ^ 1, sv, j);
+      }
+    }
+    APS_WAIT_LGKM0();
+    if ((APS_WS_ABL & 4) == 0) APS_BARRIER();  // everyone has left this chunk's buffer, the next one is complete
+  }
+
+  // ---- totals of the softmax: (max, sum) per head
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    float l = ml_s[1][j][tid];
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) l += __shfl_xor(l, off);
+    if (tq == 0) {
+      fin_s[0][hl + kWsHeadsPerPass * j] = ml_s[0][j][tid];
+      fin_s[1][hl + kWsHeadsPerPass * j] = l;
+    }
+  }
   __syncthreads();
-  sum = (red[0] + red[1]) + (red[2] + red[3]);
-  const float inv = 1.f / sum;
-  // zero padded to the next multiple of 32 tokens: the weighted sum reads a row's probabilities 32 at a time and
-  // never past its sequence
-  const int64_t pad_to = min(lp, (int64_t)((L + 31) / 32 * 32));
-  for (int64_t t = threadIdx.x * 4; t < pad_to; t += 1024) {
-    float4 v = {0.f, 0.f, 0.f, 0.f};
-    if (t < L) v = *(const float4*)(src + t);
-    uint16_t o[4];
-    const float e[4] = {v.x, v.y, v.z, v.w};
+  if (g.partial_ml && blockIdx.x == 0 && tid < 16 * MT && m0 + tid < g.heads) {
+    float* ml = g.partial_ml + (((int64_t)blockIdx.z * g.n_seqs + z) * g.heads + m0 + tid) * 2;
+    ml[0] = fin_s[0][tid];
+    ml[1] = fin_s[1][tid];
+  }
+  // lane (g4, c) holds heads m0 + 16*ht + 4*g4 + i and columns col0 .. col0+7 (MFMA j = column j)
+  if (!col_ok) return;
+#pragma unroll
+  for (int ht = 0; ht < MT; ++ht)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float pv = t + i < L ? exp2f(e[i] - mx) * inv : 0.f;
-      o[i] = BF16 ? f32_to_bf16_bits(pv) : f32_to_f16_bits(pv);
+      const int m = m0 + 16 * ht + 4 * g4 + i;
+      if (m >= g.heads) continue;
+      if (g.partial) {
+        float* dst = g.partial + (((int64_t)blockIdx.z * g.n_seqs + z) * g.heads + m) * g.n + col0;
+        *(float4v*)dst = float4v{acc[ht][0][i], acc[ht][1][i], acc[ht][2][i], acc[ht][3][i]};
+        *(float4v*)(dst + 4) = float4v{acc[ht][4][i], acc[ht][5][i], acc[ht][6][i], acc[ht][7][i]};
+      } else {
+        const float l = fin_s[1][16 * ht + 4 * g4 + i];
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+        uint16_t h[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float v = acc[ht][j][i] * inv;
+          h[j] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+        }
+        u32x4 o;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) o[p] = (uint32_t)h[2 * p] | ((uint32_t)h[2 * p + 1] << 16);
+        *(u32x4*)(g.out + ((int64_t)z * g.out_batch_stride + (int64_t)m * g.out_row_stride + col0) * 2) = o;
+      }
     }
-    *(uint2*)(out + t) = uint2{(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
+}
+
+// ctx[z][h][n] = sum_p w_p * partial[p][z][h][n] / sum_p w_p * l_p with w_p = 2^(m_p - max_p m_p): the partitions
+// of a sequence put on one scale, added in the order of the partitions, 4 columns per thread.
+template <bool BF16>
+__global__ __launch_bounds__(256) void wsum_combine_kernel(const float* __restrict__ partial,
+                                                           const float* __restrict__ ml, char* out, int parts,
+                                                           int n_seqs, int heads, int64_t n, int64_t out_batch_stride,
+                                                           int64_t out_row_stride) {
+  const int64_t per_part = (int64_t)n_seqs * heads * n;
+  const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (idx >= per_part) return;
+  const int64_t col = idx % n, zh = idx / n;
+  float mx = -INFINITY;
+  for (int p = 0; p < parts; ++p) mx = fmaxf(mx, ml[((int64_t)p * n_seqs * heads + zh) * 2]);
+  float4v num = {0.f, 0.f, 0.f, 0.f};
+  float den = 0.f;
+  for (int p = 0; p < parts; ++p) {
+    const float mp = ml[((int64_t)p * n_seqs * heads + zh) * 2], lp = ml[((int64_t)p * n_seqs * heads + zh) * 2 + 1];
+    if (mp == -INFINITY) continue;  // a partition past the end of its sequence
+    const float w = exp2f(mp - mx);
+    const float4v v = *(const float4v*)(partial + p * per_part + idx);
+    num[0] += v[0] * w; num[1] += v[1] * w; num[2] += v[2] * w; num[3] += v[3] * w;
+    den += lp * w;
   }
+  const float inv = den > 0.f ? 1.f / den : 0.f;
+  const int64_t h = zh % heads, z = zh / heads;
+  uint16_t* o = (uint16_t*)out + z * out_batch_stride + h * out_row_stride + col;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = BF16 ? f32_to_bf16_bits(num[i] * inv) : f32_to_f16_bits(num[i] * inv);
 }
 
 template <bool BF16>
-int launch_nn(const NnArgs& g, int kparts, hipStream_t s) {
+int launch_nn(const NnArgs& g, hipStream_t s) {
   const int mt = g.m_tiles > 1 ? 3 : (g.m_rows <= 16 ? 1 : (g.m_rows <= 32 ? 2 : 3));  // row tiles are 16*mt rows
-  const dim3 grid((unsigned)((g.n + kNnWaves * 128 - 1) / (kNnWaves * 128)), (unsigned)(g.batches * g.m_tiles),
-                  (unsigned)kparts);
+  const dim3 grid((unsigned)((g.n + kNnWaves * 128 - 1) / (kNnWaves * 128)), (unsigned)(g.batches * g.m_tiles));
   if (mt == 1)
     APS_LAUNCH((nn_few_rows_kernel<BF16, 1>), grid, dim3(kNnWaves * 64), 0, s, g);
   else if (mt == 2)
@@ -487,31 +822,33 @@ int launch_nn(const NnArgs& g, int kparts, hipStream_t s) {
 inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
 struct Plan {
-  int64_t lp;        // padded row length of S and P
+  int64_t lp;        // padded row length of S
   int kparts;        // token partitions of the weighted sum
-  int score_parts;   // parts of K in the scores kernel (partial scores summed by the softmax)
+  int score_parts;   // parts of K in the scores kernel (partial scores, added by the weighted sum as it reads them)
   int64_t score_k_per_part;
   int k_per_part;
-  int64_t off_qt, off_s, off_p, off_ctx, off_tiles, off_order, off_partial, total;
+  int64_t off_qt, off_s, off_ctx, off_tiles, off_order, off_zero, off_partial, off_ml, total;
 };
 
 Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   Plan p{};
   p.lp = align_up(max_len > 0 ? max_len : 1, 32);
-  const int64_t col_tiles = (hidden + kNnWaves * 128 - 1) / (kNnWaves * 128);
+  const int64_t col_tiles = (hidden + kWsWaves * 128 - 1) / (kWsWaves * 128) * ((heads + 47) / 48);
   int64_t parts = 1;
   // Fewer workgroups than CUs (few sequences): split the tokens.  A workgroup walks its tokens one after the
-  // other at ~29 GB/s, so without a split the longest sequence sets the kernel's time.  The host knows only the
-  // longest length; with lengths spread like a serving batch's the rows in all are about a third of
-  // n_seqs * longest, and a part should hold about 1/256 of the work of one column tile.
+  // other, so without a split the longest sequence sets the kernel's time.  The host knows only the longest
+  // length; with lengths spread like a serving batch's the rows in all are about a third of n_seqs * longest,
+  // and a part should hold about 1/256 of the work of one column tile.
+  // Every partition of every sequence leaves fp32 sums of heads x hidden values for the combining kernel: at
+  // least two chunks of tokens per partition keep that traffic below what the rows themselves are.
   if (n_seqs * col_tiles < 256) {
     int64_t target = n_seqs * p.lp * col_tiles / 3 / 256;
-    if (target < 64) target = 64;
+    if (target < 2 * kWsChunk) target = 2 * kWsChunk;
     parts = (p.lp + target - 1) / target;
     if (parts > 32) parts = 32;
   }
-  while (p.lp / parts > kNnMaxPart) parts *= 2;
-  p.k_per_part = (int)align_up((p.lp + parts - 1) / parts, 32);
+  while ((p.lp + parts - 1) / parts > kWsMaxPart - kWsChunk) parts *= 2;
+  p.k_per_part = (int)align_up((p.lp + parts - 1) / parts, kWsChunk);
   p.kparts = (int)((p.lp + p.k_per_part - 1) / p.k_per_part);
   // scores: with few 128-token tiles, K is split by whole 512-element chunks into as many parts as still give
   // at most one workgroup per CU (one round of long-lived workgroups streams fastest)
@@ -531,12 +868,14 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   int64_t o = 0;
   p.off_qt = o; o += align_up(n_seqs * heads * hidden * 2, 256);
   p.off_s = o; o += align_up(n_seqs * heads * p.lp * 4, 256) * p.score_parts;
-  p.off_p = o; o += align_up(n_seqs * heads * p.lp * 2, 256);
   p.off_ctx = o; o += align_up(n_seqs * heads * hidden * 2, 256);
   p.off_tiles = o; o += align_up((n_seqs + 1) * 4, 256);
   p.off_order = o; o += align_up(n_seqs * 4, 256);
+  p.off_zero = o; o += align_up(hidden * 2, 256);
   p.off_partial = o;
   if (p.kparts > 1) o += align_up((int64_t)p.kparts * n_seqs * heads * hidden * 4, 256);
+  p.off_ml = o;
+  if (p.kparts > 1) o += align_up((int64_t)p.kparts * n_seqs * heads * 2 * 4, 256);
   p.total = o;
   return p;
 }
@@ -577,7 +916,8 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
                         (uint64_t)q_stride * 2, (uint64_t)slot_stride * 2, (uint64_t)w_stride * 2,
                         (uint64_t)out_stride * 2}) != 16)
     return APS_ERR_UNSUPPORTED;
-  if (n_seqs > 65535 || max_len > ((int64_t)1 << 24)) return APS_ERR_UNSUPPORTED;
+  if (n_seqs > 65535 / ((num_heads + 47) / 48) || max_len > ((int64_t)1 << 24) || num_slots > 0x7fffffff)
+    return APS_ERR_UNSUPPORTED;
   const Plan p = make_plan(n_seqs, max_len, num_heads, hidden);
   if (workspace_bytes < p.total) return APS_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
@@ -586,23 +926,51 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
   char* qt = ws + p.off_qt;
   float* sc = (float*)(ws + p.off_s);
   const int64_t s_part_stride = align_up(n_seqs * num_heads * p.lp * 4, 256) / 4;  // elements between K parts
-  char* pr = ws + p.off_p;
   char* ctx = ws + p.off_ctx;
   float* partial = (float*)(ws + p.off_partial);
 
-  // 1. qt[s][h][:] = scale*log2(e) * W_k[h]^T q[seq_rows[s]][h]: batch = head, K = head_size, B = rows of W_k
-  {
+  int32_t* tiles = (int32_t*)(ws + p.off_tiles);
+  int32_t* order = n_seqs > 1 && n_seqs <= kMaxOrderedSeqs ? (int32_t*)(ws + p.off_order) : nullptr;
+  // 1. qt[s][h][:] = scale*log2(e) * W_k[h]^T q[seq_rows[s]][h], and the plan of the ragged batch (tile list of
+  //    the scores kernel, longest-first order of the weighted sum) in the same launch
+  if (head_size <= 128) {
+    QImageArgs g{};
+    g.q = (const char*)q; g.q_stride_b = q_stride * 2; g.seq_rows = seq_rows; g.num_q_rows = num_q_rows;
+    g.n_seqs = (int)n_seqs;
+    g.w = (const char*)w_k; g.w_stride_b = w_stride * 2;
+    g.heads = num_heads; g.hidden = hidden;
+    g.qt = qt;
+    g.alpha = softmax_scale * 1.4426950408889634f;
+    g.row_start = seq_start; g.tile_tokens = kScTokens; g.tile_start = tiles; g.order = order;
+    g.zero_row = (u32x4*)(ws + p.off_zero); g.zero_vecs = (int)(hidden * 2 / 16);
+    const dim3 grid((unsigned)((hidden + 511) / 512), (unsigned)num_heads + 1);
+#define APS_LAUNCH_QI(B)                                                                     \
+  switch (head_size / 32) {                                                                  \
+    case 1: APS_LAUNCH((query_image_kernel<B, 1>), grid, dim3(256), 0, s, g); break;         \
+    case 2: APS_LAUNCH((query_image_kernel<B, 2>), grid, dim3(256), 0, s, g); break;         \
+    case 3: APS_LAUNCH((query_image_kernel<B, 3>), grid, dim3(256), 0, s, g); break;         \
+    default: APS_LAUNCH((query_image_kernel<B, 4>), grid, dim3(256), 0, s, g); break;        \
+  }
+    if (bf16) { APS_LAUNCH_QI(true) } else { APS_LAUNCH_QI(false) }
+#undef APS_LAUNCH_QI
+    const int st = launch_status();
+    if (st != APS_OK) return st;
+  } else {  // heads wider than 128: the generic few-row product (batch = head, K = head_size, B = rows of W_k)
     NnArgs g{};
     g.a = (const char*)q; g.a_batch_stride_b = (int64_t)head_size * 2; g.lda_b = q_stride * 2;
     g.m_rows = (int)n_seqs; g.a_row_ids = seq_rows; g.num_a_rows = num_q_rows;
     g.b = (const char*)w_k; g.b_row_stride_b = w_stride * 2; g.num_b_rows = hidden;
-    g.row_ids = nullptr; g.row_start = nullptr; g.k_fixed = head_size;
+    g.k_fixed = head_size;
     g.n = hidden;
     g.out = qt; g.out_batch_stride = hidden; g.out_row_stride = (int64_t)num_heads * hidden;
-    g.partial = nullptr; g.batches = num_heads; g.k_per_part = head_size;
+    g.batches = num_heads;
     g.m_tiles = (int)((n_seqs + 47) / 48);
     g.alpha = softmax_scale * 1.4426950408889634f;
-    const int st = bf16 ? launch_nn<true>(g, 1, s) : launch_nn<false>(g, 1, s);
+    int st = bf16 ? launch_nn<true>(g, s) : launch_nn<false>(g, s);
+    if (st != APS_OK) return st;
+    APS_LAUNCH(seq_plan_kernel, dim3(1), dim3(256), 0, s, seq_start, (int)n_seqs, kScTokens, tiles, order,
+               (u32x4*)(ws + p.off_zero), (int)(hidden * 2 / 16));
+    st = launch_status();
     if (st != APS_OK) return st;
   }
   // 2. S[s][h][t] = <qt[s][h], hidden row t of sequence s>
@@ -614,9 +982,6 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     g.heads = num_heads;
     g.s = sc; g.s_batch_stride = (int64_t)num_heads * p.lp; g.s_row_stride = p.lp;
     g.k = hidden;
-    int32_t* tiles = (int32_t*)(ws + p.off_tiles);
-    int32_t* order = n_seqs > 1 && n_seqs <= kMaxOrderedSeqs ? (int32_t*)(ws + p.off_order) : nullptr;
-    APS_LAUNCH(seq_plan_kernel, dim3(1), dim3(256), 0, s, seq_start, (int)n_seqs, kScTokens, tiles, order);
     g.tile_start = tiles; g.n_seqs = (int)n_seqs;
     g.k_per_part = p.score_k_per_part; g.s_part_stride = s_part_stride;
     // upper bound of the tile count that the host can know: every sequence at max_len
@@ -647,43 +1012,46 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     const int st = launch_status();
     if (st != APS_OK) return st;
   }
-  // 3. P = softmax over the tokens, zero padded to whole groups of 32 tokens
+  // 3. ctx[s][h][:] = sum_t softmax_t(S[s][h])[t] * hidden row t: online softmax inside the pass over the rows
   {
-    const dim3 grid((unsigned)num_heads, (unsigned)n_seqs);
-    if (bf16)
-      APS_LAUNCH(softmax_rows_kernel<true>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp,
-                         p.score_parts, s_part_stride);
-    else
-      APS_LAUNCH(softmax_rows_kernel<false>, grid, dim3(256), 0, s, sc, (uint16_t*)pr, seq_start, num_heads, p.lp,
-                         p.score_parts, s_part_stride);
-    const int st = launch_status();
-    if (st != APS_OK) return st;
-  }
-  // 4. ctx[s][h][:] = sum_t P[s][h][t] * hidden row t: batch = sequence, K = its length, B = paged rows
-  {
-    NnArgs g{};
-    g.a = pr; g.a_batch_stride_b = (int64_t)num_heads * p.lp * 2; g.lda_b = p.lp * 2;
-    g.m_rows = num_heads; g.a_row_ids = nullptr; g.num_a_rows = num_heads;
-    g.b = (const char*)paged_cache; g.b_row_stride_b = slot_stride * 2; g.num_b_rows = num_slots;
-    g.row_ids = hidden_slots; g.row_start = seq_start; g.k_fixed = 0;
+    WsumArgs g{};
+    g.s = sc; g.s_batch_stride = (int64_t)num_heads * p.lp; g.s_row_stride = p.lp; g.s_part_stride = s_part_stride;
+    g.score_parts = p.score_parts;
+    g.cache = (const char*)paged_cache; g.slot_stride_b = slot_stride * 2; g.num_slots = num_slots;
+    g.row_ids = hidden_slots; g.row_start = seq_start;
+    g.zero_row = ws + p.off_zero;
+    g.heads = num_heads; g.m_tiles = (num_heads + 47) / 48; g.n_seqs = (int)n_seqs; g.k_per_part = p.k_per_part;
     g.n = hidden;
     g.out = ctx; g.out_batch_stride = (int64_t)num_heads * hidden; g.out_row_stride = hidden;
     g.partial = p.kparts > 1 ? partial : nullptr;
-    g.batches = (int)n_seqs; g.k_per_part = p.k_per_part;
-    g.m_tiles = (num_heads + 47) / 48;
-    g.alpha = 1.f;
-    if (n_seqs > 1 && n_seqs <= kMaxOrderedSeqs) g.batch_order = (const int32_t*)(ws + p.off_order);  // from step 2
-    int st = bf16 ? launch_nn<true>(g, p.kparts, s) : launch_nn<false>(g, p.kparts, s);
+    g.partial_ml = p.kparts > 1 ? (float*)(ws + p.off_ml) : nullptr;
+    g.order = order;
+    const int mt = g.m_tiles > 1 ? 3 : (num_heads + 15) / 16;
+    const dim3 grid((unsigned)((hidden + kWsWaves * 128 - 1) / (kWsWaves * 128)), (unsigned)(n_seqs * g.m_tiles),
+                    (unsigned)p.kparts);
+#define APS_LAUNCH_WSUM(B, P)                                                                         \
+  switch (mt) {                                                                                       \
+    case 1: APS_LAUNCH((hidden_wsum_kernel<B, 1, P>), grid, dim3(kWsThreads), 0, s, g); break;        \
+    case 2: APS_LAUNCH((hidden_wsum_kernel<B, 2, P>), grid, dim3(kWsThreads), 0, s, g); break;        \
+    default: APS_LAUNCH((hidden_wsum_kernel<B, 3, P>), grid, dim3(kWsThreads), 0, s, g); break;       \
+  }
+    if (p.score_parts > 1) {
+      if (bf16) { APS_LAUNCH_WSUM(true, true) } else { APS_LAUNCH_WSUM(false, true) }
+    } else {
+      if (bf16) { APS_LAUNCH_WSUM(true, false) } else { APS_LAUNCH_WSUM(false, false) }
+    }
+#undef APS_LAUNCH_WSUM
+    int st = launch_status();
     if (st != APS_OK) return st;
     if (p.kparts > 1) {
       const int64_t quads = n_seqs * num_heads * hidden / 4;
       const dim3 rgrid((unsigned)((quads + 255) / 256));
       if (bf16)
-        APS_LAUNCH(nn_reduce_kernel<true>, rgrid, dim3(256), 0, s, partial, ctx, p.kparts, (int)n_seqs,
-                           num_heads, hidden, g.out_batch_stride, g.out_row_stride, 1.f);
+        APS_LAUNCH(wsum_combine_kernel<true>, rgrid, dim3(256), 0, s, partial, g.partial_ml, ctx, p.kparts, (int)n_seqs,
+                   num_heads, hidden, g.out_batch_stride, g.out_row_stride);
       else
-        APS_LAUNCH(nn_reduce_kernel<false>, rgrid, dim3(256), 0, s, partial, ctx, p.kparts, (int)n_seqs,
-                           num_heads, hidden, g.out_batch_stride, g.out_row_stride, 1.f);
+        APS_LAUNCH(wsum_combine_kernel<false>, rgrid, dim3(256), 0, s, partial, g.partial_ml, ctx, p.kparts,
+                   (int)n_seqs, num_heads, hidden, g.out_batch_stride, g.out_row_stride);
       st = launch_status();
       if (st != APS_OK) return st;
     }
