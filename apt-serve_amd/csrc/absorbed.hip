@@ -392,6 +392,30 @@ __global__ __launch_bounds__(kScThreads) void hidden_scores_kernel(const ScoreAr
     }
 }
 
+// S[0] += S[1] + ... + S[parts-1]: the partial scores of a K-split scores pass (few tiles: small batches) made
+// whole before the softmax reads them, 4 scores per thread, every part's load independent of the others, added in
+// part order.
+__global__ __launch_bounds__(256) void score_parts_sum_kernel(float* __restrict__ s, int64_t n, int parts,
+                                                              int64_t part_stride) {
+  const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (idx >= n) return;
+  float4v acc = *(const float4v*)(s + idx);
+  int p = 1;
+  for (; p + 3 < parts; p += 4) {
+    const float4v v0 = *(const float4v*)(s + p * part_stride + idx);
+    const float4v v1 = *(const float4v*)(s + (p + 1) * part_stride + idx);
+    const float4v v2 = *(const float4v*)(s + (p + 2) * part_stride + idx);
+    const float4v v3 = *(const float4v*)(s + (p + 3) * part_stride + idx);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = (((acc[i] + v0[i]) + v1[i]) + v2[i]) + v3[i];
+  }
+  for (; p < parts; ++p) {
+    const float4v v = *(const float4v*)(s + p * part_stride + idx);
+    acc[0] += v[0]; acc[1] += v[1]; acc[2] += v[2]; acc[3] += v[3];
+  }
+  *(float4v*)(s + idx) = acc;
+}
+
 // ------------------------------------------------------------------ per-head projection of many rows
 // out[map(m)][h*head_rows + d] = <W[h*head_rows + d], x[m][h]> + bias, for m < m_rows: the per-head value
 // projection of the context rows of many sequences.  The same streaming core as the scores: the streamed rows
@@ -451,8 +475,8 @@ __global__ __launch_bounds__(kScThreads) void head_proj_kernel(const HeadProjArg
 // columns; a wavefront owns 128 columns and walks the rows 32 tokens at a time: a lane loads an 8x8 block (8
 // rows, 16 bytes = 8 columns each; 16 lanes read 256 contiguous bytes of a row), transposes it in registers with
 // v_perm_b32 and feeds 8 MFMAs per 16 heads.  The softmax is an online one, 96 tokens (a chunk = 3 steps) at a
-// time: the threads of the workgroup read the fp32 scores of the next chunk of all heads once (adding the partial
-// scores of a K-split scores pass), keep a running maximum and sum per head, and leave p = exp2(s - max) as
+// time: the threads of the workgroup read the fp32 scores of the next chunk of all heads once, keep a running
+// maximum and sum per head, and leave p = exp2(s - max) as
 // 16-bit values in LDS, where every wavefront fetches its MFMA operand — the scores are read once per workgroup
 // instead of the probabilities once per 128 columns (those redundant reads were a quarter of the traffic of the
 // kernel this replaces), and no softmax pass or probability buffer exists.  When a chunk moves a head's maximum
@@ -495,7 +519,7 @@ __device__ __forceinline__ float half_wave_max(float x) {
 }
 
 struct WsumArgs {
-  const float* s; int64_t s_batch_stride, s_row_stride, s_part_stride; int score_parts;  // S[part][z][h][t]
+  const float* s; int64_t s_batch_stride, s_row_stride;  // S[z][h][t], complete scores
   const char* cache; int64_t slot_stride_b, num_slots;
   const int64_t* row_ids; const int64_t* row_start;
   const char* zero_row;                                   // n zeros (what a token without a cached row reads)
@@ -506,7 +530,7 @@ struct WsumArgs {
   const int32_t* order;                                   // nullable: the y-th sequence dispatched (longest first)
 };
 
-template <bool BF16, int MT, bool PARTS>
+template <bool BF16, int MT>
 __global__ __launch_bounds__(kWsThreads) __attribute__((amdgpu_waves_per_eu(APS_WS_OCC, APS_WS_OCC))) void hidden_wsum_kernel(
     const WsumArgs g) {
   constexpr int NJ = 16 * MT / kWsHeadsPerPass;   // score quads per thread and chunk
@@ -580,23 +604,6 @@ __global__ __launch_bounds__(kWsThreads) __attribute__((amdgpu_waves_per_eu(APS_
       for (int qq = 0; qq < QJ; ++qq) {
         const int t = quad_t(chunk, qq);
         const int ts = (quad_ok(qq) && t < kend) ? t : 0;
-        if constexpr (PARTS) {  // the partial scores of a K-split scores pass (few tiles: small batches)
-          const char* sp = s_base + s_off(j, ts);
-          const int64_t stride_b = g.s_part_stride * 4;
-          int part = 1;
-          for (; part + 3 < g.score_parts; part += 4) {  // four independent loads in flight, added in part order
-            const float4v o0 = *(const float4v*)(sp + part * stride_b);
-            const float4v o1 = *(const float4v*)(sp + (part + 1) * stride_b);
-            const float4v o2 = *(const float4v*)(sp + (part + 2) * stride_b);
-            const float4v o3 = *(const float4v*)(sp + (part + 3) * stride_b);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) sv[j][qq][i] = (((sv[j][qq][i] + o0[i]) + o1[i]) + o2[i]) + o3[i];
-          }
-          for (; part < g.score_parts; ++part) {
-            const float4v o = *(const float4v*)(sp + part * stride_b);
-            sv[j][qq][0] += o[0]; sv[j][qq][1] += o[1]; sv[j][qq][2] += o[2]; sv[j][qq][3] += o[3];
-          }
-        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           ok[qq][i] = head_ok && quad_ok(qq) && t + i < kend;
@@ -824,7 +831,7 @@ inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 struct Plan {
   int64_t lp;        // padded row length of S
   int kparts;        // token partitions of the weighted sum
-  int score_parts;   // parts of K in the scores kernel (partial scores, added by the weighted sum as it reads them)
+  int score_parts;   // parts of K in the scores kernel (partial scores, made whole by score_parts_sum_kernel)
   int64_t score_k_per_part;
   int k_per_part;
   int64_t off_qt, off_s, off_ctx, off_tiles, off_order, off_zero, off_partial, off_ml, total;
@@ -1012,11 +1019,17 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     const int st = launch_status();
     if (st != APS_OK) return st;
   }
+  if (p.score_parts > 1) {
+    const int64_t n = n_seqs * num_heads * p.lp;   // a multiple of 32
+    APS_LAUNCH(score_parts_sum_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, s, sc, n, p.score_parts,
+               s_part_stride);
+    const int st = launch_status();
+    if (st != APS_OK) return st;
+  }
   // 3. ctx[s][h][:] = sum_t softmax_t(S[s][h])[t] * hidden row t: online softmax inside the pass over the rows
   {
     WsumArgs g{};
-    g.s = sc; g.s_batch_stride = (int64_t)num_heads * p.lp; g.s_row_stride = p.lp; g.s_part_stride = s_part_stride;
-    g.score_parts = p.score_parts;
+    g.s = sc; g.s_batch_stride = (int64_t)num_heads * p.lp; g.s_row_stride = p.lp;
     g.cache = (const char*)paged_cache; g.slot_stride_b = slot_stride * 2; g.num_slots = num_slots;
     g.row_ids = hidden_slots; g.row_start = seq_start;
     g.zero_row = ws + p.off_zero;
@@ -1029,17 +1042,13 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     const int mt = g.m_tiles > 1 ? 3 : (num_heads + 15) / 16;
     const dim3 grid((unsigned)((hidden + kWsWaves * 128 - 1) / (kWsWaves * 128)), (unsigned)(n_seqs * g.m_tiles),
                     (unsigned)p.kparts);
-#define APS_LAUNCH_WSUM(B, P)                                                                         \
-  switch (mt) {                                                                                       \
-    case 1: APS_LAUNCH((hidden_wsum_kernel<B, 1, P>), grid, dim3(kWsThreads), 0, s, g); break;        \
-    case 2: APS_LAUNCH((hidden_wsum_kernel<B, 2, P>), grid, dim3(kWsThreads), 0, s, g); break;        \
-    default: APS_LAUNCH((hidden_wsum_kernel<B, 3, P>), grid, dim3(kWsThreads), 0, s, g); break;       \
+#define APS_LAUNCH_WSUM(B)                                                                          \
+  switch (mt) {                                                                                     \
+    case 1: APS_LAUNCH((hidden_wsum_kernel<B, 1>), grid, dim3(kWsThreads), 0, s, g); break;         \
+    case 2: APS_LAUNCH((hidden_wsum_kernel<B, 2>), grid, dim3(kWsThreads), 0, s, g); break;         \
+    default: APS_LAUNCH((hidden_wsum_kernel<B, 3>), grid, dim3(kWsThreads), 0, s, g); break;        \
   }
-    if (p.score_parts > 1) {
-      if (bf16) { APS_LAUNCH_WSUM(true, true) } else { APS_LAUNCH_WSUM(false, true) }
-    } else {
-      if (bf16) { APS_LAUNCH_WSUM(true, false) } else { APS_LAUNCH_WSUM(false, false) }
-    }
+    if (bf16) { APS_LAUNCH_WSUM(true) } else { APS_LAUNCH_WSUM(false) }
 #undef APS_LAUNCH_WSUM
     int st = launch_status();
     if (st != APS_OK) return st;
