@@ -786,6 +786,44 @@ def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, se
     return out
 
 
+# ------------------------------------------------------------------ residual add + LayerNorm
+
+def add_layer_norm(x, residual, weight, bias, eps: float = 1e-5, out=None, sum_out=None):
+    """``s = x + residual`` (rounded to the activation dtype; ``residual`` may be ``None``) and
+    ``LayerNorm(s) * weight + bias`` in one launch: the residual add and the LayerNorm that follows it in
+    ``OPTDecoderLayer.forward`` (additional_designs/model_executor/models/aptserve_opt.py:186-211).
+    Returns ``(normed, s)``; ``s`` is ``x`` itself when there is no residual."""
+    dev = x.device
+    _check_data("x", x, dev)
+    _need(x.dim() == 2 and x.dtype in (torch.float16, torch.bfloat16), "x must be a 2-D f16 or bf16 tensor")
+    rows, width = x.shape
+    for n, t in (("weight", weight), ("bias", bias)):
+        if t is not None:
+            _check_data(n, t, dev)
+            _need(t.dim() == 1 and t.numel() == width and t.dtype == x.dtype and t.is_contiguous(),
+                  f"{n} must be a contiguous [width] vector of x's dtype")
+    _need(weight is not None, "weight is required")
+    if residual is not None:
+        _check_data("residual", residual, dev)
+        _need(residual.shape == x.shape and residual.dtype == x.dtype, "residual must look like x")
+    if out is None:
+        out = torch.empty(rows, width, dtype=x.dtype, device=dev)
+    if residual is not None and sum_out is None:
+        sum_out = torch.empty(rows, width, dtype=x.dtype, device=dev)
+    for n, t in (("out", out), ("sum_out", sum_out)):
+        if t is not None:
+            _check_data(n, t, dev)
+            _need(t.shape == x.shape and t.dtype == x.dtype, f"{n} must look like x")
+    with _on(dev):
+        st = _lib.load().aps_add_layer_norm(
+            _ptr(out), None if residual is None else _ptr(sum_out), _ptr(x), _ptr(residual), _ptr(weight), _ptr(bias),
+            rows, width, x.stride(0), 0 if residual is None else residual.stride(0), out.stride(0),
+            0 if residual is None or sum_out is None else sum_out.stride(0), float(eps), _DTYPE_CODE[x.dtype],
+            _stream(x))
+    _lib.check(st, "add_layer_norm")
+    return out, (x if residual is None else sum_out)
+
+
 # ------------------------------------------------------------------ block maintenance
 
 _LAYER_BASES = {}

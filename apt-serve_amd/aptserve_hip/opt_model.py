@@ -6,8 +6,9 @@ pre-LayerNorm OPT variants (``do_layer_norm_before=True``: 125m, 1.3b ... 175b):
 state cached for a hidden-cached sequence is the output of ``self_attn_layer_norm``, i.e.
 the input of ``qkv_proj``.  Weights are random-initialised from a locally built config
 (no checkpoint, no tokenizer).  Attention, the q/kv projections, the cache traffic, fc1 and
-fc2 run on this library's kernels; LayerNorm, ReLU, the residual adds and the embedding
-lookup are plain PyTorch-ROCm element-wise ops.
+fc2 run on this library's kernels, and so does every (residual add, LayerNorm) pair
+(``ops.add_layer_norm``: one launch instead of two element-wise ones; ``fused_norm=False``
+keeps the plain PyTorch-ROCm ops); ReLU and the embedding lookup are PyTorch-ROCm ops.
 """
 
 from __future__ import annotations
@@ -67,7 +68,15 @@ class HybridOPTDecoderLayer:
         self.self_attn = HybridOPTAttention(cfg.hidden_size, cfg.num_attention_heads, w[prefix + "qkv_w"],
                                             w[prefix + "qkv_b"], w[prefix + "out_w"], w[prefix + "out_b"], **attn_kw)
 
+    def _mlp(self, x):
+        w, p = self.w, self.p
+        with phase("projections"):
+            x = ops.linear_nt(x, w[p + "fc1_w"], w[p + "fc1_b"])
+            x = torch.relu_(x)
+            return ops.linear_nt(x, w[p + "fc2_w"], w[p + "fc2_b"])
+
     def forward(self, hidden_states, kv_cache, shared_cache, md: HybridAttentionMetadata):
+        """additional_designs/model_executor/models/aptserve_opt.py:179-212 with plain element-wise ops."""
         w, p, Hd = self.w, self.p, self.cfg.hidden_size
         residual = hidden_states
         hidden_states = F.layer_norm(hidden_states, (Hd,), w[p + "attn_ln_w"], w[p + "attn_ln_b"])
@@ -75,19 +84,27 @@ class HybridOPTDecoderLayer:
         hidden_states = residual + hidden_states
         residual = hidden_states
         hidden_states = F.layer_norm(hidden_states, (Hd,), w[p + "final_ln_w"], w[p + "final_ln_b"])
-        with phase("projections"):
-            hidden_states = ops.linear_nt(hidden_states, w[p + "fc1_w"], w[p + "fc1_b"])
-            hidden_states = torch.relu_(hidden_states)
-            hidden_states = ops.linear_nt(hidden_states, w[p + "fc2_w"], w[p + "fc2_b"])
-        return residual + hidden_states
+        return residual + self._mlp(hidden_states)
+
+    def forward_fused_norm(self, residual, normed, kv_cache, shared_cache, md, next_ln_w, next_ln_b):
+        """The same layer with every (residual add, LayerNorm) pair in one launch.  ``normed`` is this layer's
+        ``self_attn_layer_norm`` of ``residual`` (computed by the previous layer's last launch); returns the
+        layer's output and the NEXT norm of it (the next layer's ``self_attn_layer_norm``, or the decoder's
+        final one)."""
+        w, p = self.w, self.p
+        attn = self.self_attn(normed, kv_cache, shared_cache, md)
+        normed, residual = ops.add_layer_norm(attn, residual, w[p + "final_ln_w"], w[p + "final_ln_b"])
+        mlp = self._mlp(normed)
+        normed, residual = ops.add_layer_norm(mlp, residual, next_ln_w, next_ln_b)
+        return residual, normed
 
     __call__ = forward
 
 
 class HybridOPTModel:
     def __init__(self, cfg: OPTConfig, weights: Dict[str, torch.Tensor], num_layers: Optional[int] = None,
-                 **attn_kw) -> None:
-        self.cfg, self.w = cfg, weights
+                 fused_norm: bool = True, **attn_kw) -> None:
+        self.cfg, self.w, self.fused_norm = cfg, weights, fused_norm
         n = cfg.num_hidden_layers if num_layers is None else num_layers
         self.layers = [HybridOPTDecoderLayer(cfg, weights, f"layers.{i}.", **attn_kw) for i in range(n)]
 
@@ -95,9 +112,16 @@ class HybridOPTModel:
                 md: HybridAttentionMetadata) -> torch.Tensor:
         w = self.w
         hidden_states = F.embedding(input_ids, w["embed_tokens"]) + F.embedding(positions + 2, w["embed_positions"])
-        for layer, kv in zip(self.layers, kv_caches):
-            hidden_states = layer(hidden_states, kv, shared_cache, md)
-        return F.layer_norm(hidden_states, (self.cfg.hidden_size,), w["final_ln_w"], w["final_ln_b"])
+        if not self.fused_norm or not self.layers:
+            for layer, kv in zip(self.layers, kv_caches):
+                hidden_states = layer(hidden_states, kv, shared_cache, md)
+            return F.layer_norm(hidden_states, (self.cfg.hidden_size,), w["final_ln_w"], w["final_ln_b"])
+        normed, _ = ops.add_layer_norm(hidden_states, None, w["layers.0.attn_ln_w"], w["layers.0.attn_ln_b"])
+        for i, (layer, kv) in enumerate(zip(self.layers, kv_caches)):
+            nxt = f"layers.{i + 1}.attn_ln_" if i + 1 < len(self.layers) else "final_ln_"
+            hidden_states, normed = layer.forward_fused_norm(hidden_states, normed, kv, shared_cache, md,
+                                                             w[nxt + "w"], w[nxt + "b"])
+        return normed
 
     __call__ = forward
 

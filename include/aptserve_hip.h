@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define APS_ABI_VERSION 6
+#define APS_ABI_VERSION 7
 
 typedef void* aps_stream_t; /* a hipStream_t; NULL = the null stream */
 
@@ -489,7 +489,7 @@ int aps_kv_reproject_gathered(
  *     slices of the fused QKV weight); b_v nullable.
  *   max_len >= the longest sequence.  f16 / bf16; head_size % 32 == 0.
  * workspace: aps_absorbed_attention_workspace_bytes(...) bytes, 16-byte
- * aligned, owned by the caller (query images, fp32 scores, probabilities,
+ * aligned, owned by the caller (query images, fp32 scores,
  * per-head context vectors). */
 int64_t aps_absorbed_attention_workspace_bytes(int64_t n_seqs, int64_t max_len,
                                                int num_heads, int head_size);
@@ -501,6 +501,21 @@ int aps_absorbed_attention(
     const void* b_v, int64_t w_stride, int num_heads, int head_size,
     float softmax_scale, void* out, int64_t out_stride, int64_t out_rows,
     int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream);
+
+/* Residual add and LayerNorm of a decoder layer in one launch.
+ * ref: model_executor/models/aptserve_opt.py:186-211 (OPTDecoderLayer.forward:
+ * `hidden_states = residual + hidden_states` followed by the next nn.LayerNorm,
+ * which at :189-190 produces the rows a hidden-cached sequence caches).
+ *   s[r, :]      = round16(x[r, :] + residual[r, :])        (residual nullable: s = x)
+ *   normed[r, :] = LayerNorm(s[r, :]) * gamma + beta        (fp32 statistics over the rounded sum, eps as given)
+ * sum (nullable) receives s, the next residual.  f16 / bf16; width a multiple
+ * of 8, at most 16384; strides in elements; all pointers 16-byte aligned. */
+int aps_add_layer_norm(void* normed, void* sum, const void* x,
+                       const void* residual, const void* gamma,
+                       const void* beta, int64_t rows, int64_t width,
+                       int64_t x_stride, int64_t residual_stride,
+                       int64_t normed_stride, int64_t sum_stride, float eps,
+                       int dtype, aps_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Block maintenance, aware of hidden blocks.

@@ -109,8 +109,8 @@ def test_linear_workspace_planning_is_host_only_and_consistent():
 
 def test_absorbed_attention_workspace_planning_is_host_only():
     """The workspace of the attention on hidden rows covers at least its named buffers (query image and context
-    rows: n*H*Hd 16-bit each; scores fp32 and probabilities 16-bit over the padded longest sequence), grows with
-    the batch, and degenerate arguments plan nothing."""
+    rows: n*H*Hd 16-bit each; fp32 scores over the padded longest sequence; a row of zeros), grows with the
+    batch, and degenerate arguments plan nothing."""
     lib = _lib.load()
     f = lib.aps_absorbed_attention_workspace_bytes
     for heads, d in ((12, 64), (40, 128)):
@@ -119,11 +119,14 @@ def test_absorbed_attention_workspace_planning_is_host_only():
         for n in (1, 2, 8, 16, 17, 128, 300, 5000):
             for max_len in (1, 33, 700, 2048):
                 lp = -(-max_len // 32) * 32
-                need = 2 * n * heads * hd * 2 + n * heads * lp * 4 + n * heads * lp * 2
+                need = 2 * n * heads * hd * 2 + n * heads * lp * 4 + hd * 2
                 got = f(n, max_len, heads, d)
                 assert got >= need and got % 256 == 0, (n, max_len, heads, d, got, need)
-            assert f(n, 2048, heads, d) > prev
-            prev = f(n, 2048, heads, d)
+            # small batches carry the partial sums of their token partitions as well: growth is only monotonic
+            # once no sequence is split
+            if n >= 300:
+                assert f(n, 2048, heads, d) > prev
+                prev = f(n, 2048, heads, d)
     assert f(0, 100, 40, 128) == 0 and f(4, 0, 40, 128) == 0
 
 
