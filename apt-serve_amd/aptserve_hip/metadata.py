@@ -161,6 +161,54 @@ class _Staging:
         return dev
 
 
+    def upload_into(self, i: int, host: torch.Tensor, dst: torch.Tensor, stream) -> torch.Tensor:
+        """Like ``upload`` into device memory the caller keeps (same address in every step)."""
+        dst.copy_(host, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record(stream)
+        self.events[i] = ev
+        return dst
+
+
+class StaticDecodeBuffers:
+    """Device storage for the metadata of decode steps of one shape class: ``batch`` sequences of which
+    ``n_hidden`` are hidden-cached, none longer than ``cap_len`` tokens.  ``build_metadata(..., static=this)``
+    writes every step's metadata to the same addresses, which is what lets a step that was recorded into a HIP
+    graph be replayed on the next step's batch."""
+
+    def __init__(self, batch: int, n_hidden: int, cap_len: int, block_size: int, device) -> None:
+        if cap_len % block_size:
+            raise ValueError("cap_len must be a whole number of blocks")
+        self.batch, self.n_hidden, self.cap_len, self.block_size = batch, n_hidden, cap_len, block_size
+        self.device = torch.device(device)
+        self.width = cap_len // block_size
+        self.cap_hidden_rows = n_hidden * cap_len
+        self.cap_rows = self.cap_hidden_rows + (batch - n_hidden)
+        self.packed = torch.zeros(2 * batch + 2 * batch * self.width, dtype=torch.int32, device=self.device)
+        self._b64 = self._b32 = None
+
+    def check(self, batch: int, n_hidden: int, max_len: int, block_size: int, device) -> None:
+        if (batch, n_hidden, block_size) != (self.batch, self.n_hidden, self.block_size) or max_len > self.cap_len \
+                or torch.device(device) != self.device:
+            raise ValueError("this batch does not fit the static metadata buffers (batch size, number of "
+                             "hidden-cached sequences, block size and device must match; lengths must not exceed "
+                             f"{self.cap_len})")
+
+    def take64(self, n: int) -> torch.Tensor:
+        if self._b64 is None:
+            self._b64 = torch.zeros(n, dtype=torch.int64, device=self.device)
+        if self._b64.numel() != n:
+            raise RuntimeError("static metadata layout changed")
+        return self._b64
+
+    def take32(self, n: int) -> torch.Tensor:
+        if self._b32 is None:
+            self._b32 = torch.zeros(n, dtype=torch.int32, device=self.device)
+        if self._b32.numel() != n:
+            raise RuntimeError("static metadata layout changed")
+        return self._b32
+
+
 _staging = {}
 
 
@@ -192,7 +240,9 @@ def _pack_tables(tables, lens: np.ndarray, out: np.ndarray, rows: Optional[np.nd
     ``[B, >=W]`` int array is copied as it is (``rows``: boolean mask of the tables that count, the others are
     left empty)."""
     if isinstance(tables, np.ndarray):       # 0-padded by contract: one block copy
-        out[:, :] = tables[:, :out.shape[1]]
+        w = min(out.shape[1], tables.shape[1])
+        out[:, :w] = tables[:, :w]
+        out[:, w:] = 0
         if rows is not None:
             out[~rows] = 0
         return
@@ -209,7 +259,8 @@ def _pack_tables(tables, lens: np.ndarray, out: np.ndarray, rows: Optional[np.nd
 def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequence[bool],
                    block_tables: Sequence[Sequence[int]], block_tables_4_shared: Sequence[Sequence[int]],
                    block_size: int, device, context_lens: Optional[Sequence[int]] = None,
-                   check_totals: bool = False) -> HybridAttentionMetadata:
+                   check_totals: bool = False, static: Optional["StaticDecodeBuffers"] = None
+                   ) -> HybridAttentionMetadata:
     """Build the metadata of one homogeneous batch (all prompts or all decodes, as the
     reference's scheduler emits them, additional_designs/core/aptserve_scheduler.py:1613-1625).
 
@@ -220,6 +271,11 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
     Tables may be lists of lists (what the reference's scheduler hands over) or packed, 0-padded
     ``[batch, width]`` int arrays that the caller keeps up to date between steps: flattening ~10 k Python
     integers of a 256-sequence batch costs more host time than everything else in this function together.
+
+    ``static`` (decode steps only): persistent device buffers of fixed capacity (:class:`StaticDecodeBuffers`).
+    The metadata is built into them, at the same addresses in every step, and the row-indexed fields come back
+    at their capacity instead of the step's own length (entries past the step's rows are never referenced) —
+    what a step recorded into a HIP graph needs.
     """
     device = torch.device(device)
     B = len(seq_lens)
@@ -277,8 +333,14 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
             Ws = int(bts_lens.max()) if (have_tables and n_hs) else 0
             # width of the table handed to attention: the longest *selected* table (:601-609)
             Wo = int(np.where(hid, bts_lens, bt_lens).max()) if have_tables else 0
+        if static is not None:
+            static.check(B, n_hs, max_len, block_size, device)
+            if have_tables:
+                W = Wo = static.width
+                Ws = static.width if n_hs else 0
         # one packed upload: lens | flags | private tables | shared tables
-        stg, slot, host = _stage(device, 2 * B + B * W + B * Ws, zero=not (arrays and (Ws == 0 or shared_arrays)))
+        stg, slot, host = _stage(device, 2 * B + B * W + B * Ws,
+                                 zero=static is not None or not (arrays and (Ws == 0 or shared_arrays)))
         hv = host.numpy()
         hv[:B] = lens
         hv[B:2 * B] = hid
@@ -290,20 +352,25 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
             else:
                 shared = [t if h else () for t, h in zip(block_tables_4_shared, hid)]
                 _pack_tables(shared, bts_lens, hv[2 * B + B * W:].reshape(B, Ws))
-        packed = stg.upload(slot, host, device, stream)
+        if static is None:
+            packed = stg.upload(slot, host, device, stream)
+        else:
+            packed = stg.upload_into(slot, host, static.packed[:host.numel()], stream)
+            # capacities in place of this step's row counts: same buffer layout in every step
+            num_tot_step, num_tot, n_hr = num_tot, static.cap_rows, static.cap_hidden_rows
         d_lens, d_hid = packed[:B], packed[B:2 * B]
         d_bt = packed[2 * B:2 * B + B * W].view(B, W)
         d_bts = packed[2 * B + B * W:].view(B, Ws)
         # one allocation per output dtype
         sizes64 = [num_tot, n_hr, n_hr, n_kv, n_hs, n_hs, B, num_tot - B, B, 4, num_tot, num_tot, n_hr, n_hs + 1,
                    n_kv, B]
-        buf64 = torch.empty(sum(sizes64), **i64)
+        buf64 = torch.empty(sum(sizes64), **i64) if static is None else static.take64(sum(sizes64))
         (slot_mapping, slot_mapping_shared, use_tot, kv_use, use_input, store_tot, upd, pull, positions,
          totals, holder_src, kv_dest, hidden_slots, hidden_seq_start, kv_use_input,
          new_token_slot) = torch.split(buf64, sizes64)
         n_types = (B * Wo + 3) // 4 if (n_hs and Wo) else 0          # uint8 [B, Wo] carried in the int32 buffer
         sizes32 = [B * Wo, B + 1, B + 1, B, B, n_types]
-        buf32 = torch.empty(sum(sizes32), **i32)
+        buf32 = torch.empty(sum(sizes32), **i32) if static is None else static.take32(sum(sizes32))
         bt_out, seq_start, query_start, ctx, kv_seq_lens, types32 = torch.split(buf32, sizes32)
         bt_out = bt_out.view(B, Wo)
         # per-block source for the hybrid attention: every block of a hidden sequence is a workspace block
@@ -323,6 +390,9 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
                 query_start.data_ptr(), ctx.data_ptr(), positions.data_ptr(), totals.data_ptr(),
                 stream.cuda_stream)
         _lib.check(st, "build_decode_metadata")
+        if static is not None:
+            num_tot, n_hr = num_tot_step, int(hid_lens.sum())
+            max_len = max_hid_len = static.cap_len      # host-side bounds that stay put while the bucket lasts
         if check_totals:
             got = totals.tolist()
             if got != [num_tot, n_hr, n_hs, n_kv]:
@@ -338,7 +408,8 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
             block_types=block_types, holder_src=holder_src, kv_dest=kv_dest, hidden_slots=hidden_slots,
             hidden_seq_start=hidden_seq_start, max_hidden_seq_len=max_hid_len,
             kv_cache_use_input=kv_use_input, new_token_slot=new_token_slot, kv_seq_lens=kv_seq_lens,
-            max_kv_seq_len=int(lens[~hid].max()) if n_kv else 0, private_block_tables=d_bt)
+            max_kv_seq_len=(max_len if static is not None else int(lens[~hid].max())) if n_kv else 0,
+            private_block_tables=d_bt)
 
     # ------------------------------------------------------------------ prompts
     ctxs = np.zeros(B, dtype=np.int64) if context_lens is None else np.asarray(context_lens, dtype=np.int64)

@@ -123,11 +123,15 @@ class StepLoop:
 
     def __init__(self, forward: Callable, pick: Callable, requests: List[Request], num_blocks: int, block_size: int,
                  device, max_prompt_tokens: int = 4096, max_seqs: int = 256,
-                 on_step: Optional[Callable] = None, step_cost: Optional[Callable[[Dict], float]] = None) -> None:
+                 on_step: Optional[Callable] = None, step_cost: Optional[Callable[[Dict], float]] = None,
+                 decode_runner=None) -> None:
         """``step_cost(entry) -> seconds`` drives the simulated clock from a fixed cost model (same arrivals,
         admissions and batches whatever the measured speed, so two data flows can be compared step by step);
-        ``None`` advances it by the measured wall time of every step."""
+        ``None`` advances it by the measured wall time of every step.  ``decode_runner``
+        (:class:`aptserve_hip.graph_step.DecodeGraphRunner`): decode steps are replayed from its HIP graphs
+        instead of being issued through ``forward``."""
         self.forward, self.pick = forward, pick
+        self.decode_runner = decode_runner
         self.waiting = sorted(requests, key=lambda r: r.arrival)
         self.running: List[Request] = []
         self.finished: List[Request] = []
@@ -197,17 +201,27 @@ class StepLoop:
                 self.pool.grow(r, r.seq_len, self.block_size)
         seq_lens = [r.seq_len for r in batch]
         t0 = time.perf_counter()
-        md = metadata.build_metadata(is_prompt, seq_lens, [r.use_hidden for r in batch],
-                                     [r.block_table for r in batch], [r.shared_table for r in batch],
-                                     self.block_size, self.device)
         if is_prompt:
             ids = np.concatenate([r.token_ids for r in batch])
         else:
             ids = np.fromiter((r.generated[-1] for r in batch), dtype=np.int64, count=len(batch))
         input_ids = torch.from_numpy(ids).to(self.device, non_blocking=True)
+        graphed = self.decode_runner is not None and not is_prompt
+        captures = self.decode_runner.captures if graphed else 0
+        if graphed:
+            rec = self.decode_runner.prepare(seq_lens, [r.use_hidden for r in batch], [r.block_table for r in batch],
+                                             [r.shared_table for r in batch], input_ids)
+            md = rec.md
+        else:
+            md = metadata.build_metadata(is_prompt, seq_lens, [r.use_hidden for r in batch],
+                                         [r.block_table for r in batch], [r.shared_table for r in batch],
+                                         self.block_size, self.device)
         torch.cuda.synchronize(self.device)
         t1 = time.perf_counter()
-        hidden = self.forward(input_ids, md.input_positions, md)
+        if graphed:
+            hidden, md = self.decode_runner.run(rec)
+        else:
+            hidden = self.forward(input_ids, md.input_positions, md)
         nxt = self.pick(hidden, md)
         t_enq = time.perf_counter()              # everything is enqueued: host time of the step
         torch.cuda.synchronize(self.device)
@@ -216,7 +230,8 @@ class StepLoop:
         entry = dict(kind="prefill" if is_prompt else "decode", seqs=len(batch), tokens=int(len(ids)),
                      rows=md.num_tot_tokens, hidden_seqs=sum(r.use_hidden for r in batch),
                      metadata_ms=(t1 - t0) * 1e3, model_ms=(t2 - t1) * 1e3, host_enqueue_ms=(t_enq - t1) * 1e3,
-                     now=self.now)
+                     now=self.now, graph=graphed,
+                     recorded=graphed and self.decode_runner.captures != captures)  # this step recorded its graph
         if self.on_step is not None:
             self.on_step(dict(is_prompt=is_prompt, seq_lens=seq_lens, use_hidden=[r.use_hidden for r in batch],
                               block_tables=[list(r.block_table) for r in batch],

@@ -292,11 +292,15 @@ def main():
             torch.cuda.empty_cache()
             extras["opt13b_step_loop_reference_sequence"] = step_loop_figures(
                 torch, dev, args.seed, weights=w13, reference_sequence=True, profile_steps=0)
+            torch.cuda.empty_cache()
+            extras["opt13b_step_loop_absorbed_graphs"] = step_loop_figures(
+                torch, dev, args.seed, absorbed=True, weights=w13, graph=True, profile_steps=0)
+            d_ = extras["opt13b_step_loop_absorbed_graphs"].pop("schedule")
             del w13
             # all flows ran the same schedule (fixed-cost clock): keep no copy, only the comparison
             a_, b_ = extras["opt13b_step_loop"].pop("schedule"), extras["opt13b_step_loop_absorbed"].pop("schedule")
             c_ = extras["opt13b_step_loop_reference_sequence"].pop("schedule")
-            extras["opt13b_step_loop_same_schedule"] = a_ == b_ == c_
+            extras["opt13b_step_loop_same_schedule"] = a_ == b_ == c_ == d_
         if "cost" in want:
             extras["cost_coef"] = cost_coef_figures(torch, dev)
         if not args.no_cpu and "cpu" in want:
@@ -446,7 +450,7 @@ def mfma_ceiling_figures(torch, dev):
 
 
 def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile_steps=12, absorbed=False,
-                      weights=None, reference_sequence=False):
+                      weights=None, reference_sequence=False, graph=False):
     """BASELINE configs[4]: OPT-13B (random-init fp16, 40 layers) serving steps on the hybrid cache with
     synthetic arrivals (3 req/s, CV 1) and lognormal prompt/output lengths; half of the requests hidden-cached.
     The simulated clock runs on a fixed cost per step, so every data flow sees the same arrivals, admissions and
@@ -469,11 +473,16 @@ def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile
 
     def on_step(info):
         seq_len_sum.append((sum(info["seq_lens"]), sum(l for l, h in zip(info["seq_lens"], info["use_hidden"]) if h)))
+    runner = None
+    if graph:      # decode steps replayed from one HIP graph per shape class (absorbed flow only)
+        from aptserve_hip import graph_step
+        runner = graph_step.DecodeGraphRunner(model, kv, shared, BS, dev, max_graphs=96)
     loop = step_loop.StepLoop(lambda ids, pos, md: model(ids, pos, kv, shared, md), model.next_tokens, reqs, N, BS, dev,
-                              step_cost=step_loop.fixed_step_cost(), on_step=on_step)
+                              step_cost=step_loop.fixed_step_cost(), on_step=on_step, decode_runner=runner)
     loop.run(warm_steps)
     log = loop.run(warm_steps + timed_steps)[warm_steps:]
-    dec = [e for e in log if e["kind"] == "decode"]
+    dec_all = [e for e in log if e["kind"] == "decode"]
+    dec = [e for e in dec_all if not e.get("recorded")]      # steps that recorded a graph ran twice: counted apart
     pre = [e for e in log if e["kind"] == "prefill"]
     mean = lambda xs: sum(xs) / len(xs) if xs else None
     # ---- split of a decode step: per-phase GPU time and what each phase achieves
@@ -528,6 +537,7 @@ def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile
     return {"workload": "OPT-13B 40 layers fp16 random-init, eager; gamma arrivals 3 req/s cv 1; prompts "
                         "lognormal(5.5,1.0) in [4,2048]; outputs lognormal(5.0,0.9) in [4,1024]; 50% hidden-cached; "
                         "simulated clock on a fixed cost per step (12.5 ms decode, 10 ms + 20 us/token prompt); "
+                        + ("decode steps replayed from one HIP graph per shape class; " if graph else "")
                         + ("the reference's operator sequence, call for call, on this library's kernels"
                            if reference_sequence else
                            "hidden-cached sequences attend on their hidden rows (absorbed projections)" if absorbed
@@ -536,6 +546,8 @@ def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile
             "warm_steps": warm_steps, "steps": len(log), "decode_steps": len(dec), "prefill_steps": len(pre),
             "schedule": [(e["kind"][0], e["seqs"], e["rows"]) for e in log],
             "preemptions": loop.preemptions,
+            "decode_steps_that_recorded_a_graph": len(dec_all) - len(dec),
+            "decode_ms_per_recording_step": mean([e["model_ms"] + e["metadata_ms"] for e in dec_all if e.get("recorded")]),
             "decode_ms_per_step": mean([e["model_ms"] for e in dec]),
             "decode_seqs_per_step": mean([e["seqs"] for e in dec]),
             "decode_rows_per_step": mean([e["rows"] for e in dec]),

@@ -91,3 +91,43 @@ def test_gather_write_and_attention_replay_from_a_graph(dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(holder, want_holder) and torch.equal(out, want_out)
+
+
+def test_whole_decode_steps_replay_from_graphs_of_their_shape_class(dev):
+    """A two-layer decoder in the serving loop, once issued launch by launch and once with every decode step
+    replayed from the HIP graph of its shape class (batch size, hidden-cached sequences, bucketed length): the
+    same requests, the same schedule, and hidden states, chosen tokens and caches that are equal bit for bit.
+    Graphs are recorded when a shape class first appears and replayed for the steps that follow (new metadata in
+    the same buffers, eager prompt steps and synchronisations in between)."""
+    from aptserve_hip import graph_step, opt_model, step_loop
+    cfg = opt_model.OPTConfig(hidden_size=768, num_attention_heads=12, num_hidden_layers=2, ffn_dim=1024,
+                              vocab_size=1000, max_position_embeddings=2048)
+    N2, w = 96, opt_model.random_weights(cfg, 0, dev)
+
+    def run(graphed):
+        model = opt_model.HybridOPTModel(cfg, w, absorbed=True)
+        kv, shared = backend.allocate_caches(cfg.num_hidden_layers, N2, BS, 12, 64, torch.float16, dev)
+        reqs = step_loop.synth_requests(3, 7, rate=2000.0, hidden_fraction=0.5, vocab=1000, prompt_mu=3.3,
+                                        prompt_sigma=0.6, out_mu=1.6, out_sigma=0.3)
+        steps = []
+        runner = graph_step.DecodeGraphRunner(model, kv, shared, BS, dev, len_bucket=64) if graphed else None
+        loop = step_loop.StepLoop(lambda ids, pos, md: model(ids, pos, kv, shared, md), model.next_tokens, reqs, N2,
+                                  BS, dev, max_prompt_tokens=120, decode_runner=runner,
+                                  step_cost=step_loop.fixed_step_cost(),   # same schedule in both runs
+                                  on_step=lambda s: steps.append((s["is_prompt"], s["hidden"].clone(),
+                                                                  list(s["next_tokens"]))))
+        loop.run(40)
+        torch.cuda.synchronize()
+        return steps, kv, runner
+
+    eager, e_kv, _ = run(False)
+    graph, g_kv, runner = run(True)
+    assert len(eager) == len(graph) and any(not p for p, _, _ in eager)
+    for i, ((p0, h0, t0), (p1, h1, t1)) in enumerate(zip(eager, graph)):
+        assert p0 == p1 and t0 == t1, f"step {i}: schedule or tokens differ"
+        assert torch.equal(h0, h1), f"step {i} ({'prompt' if p0 else 'decode'}) differs from the eager loop"
+    for a, b in zip(e_kv, g_kv):
+        assert torch.equal(a, b)
+    n_decode = sum(1 for p, _, _ in eager if not p)
+    replays = sum(r.replays for r in runner.recorded.values())
+    assert replays == n_decode and 1 <= runner.captures < n_decode, (runner.captures, n_decode)
