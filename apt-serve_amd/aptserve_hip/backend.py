@@ -107,11 +107,15 @@ class HybridAttentionImpl:
         assert self.fp8 or kv_scale == 1.0, "kv_scale needs an fp8 K/V cache"            # :312
         ks, vs = self.k_scale * kv_scale, self.v_scale * kv_scale
         md = attn_metadata
-        if md.num_prefills and md.max_prompt_context_len > 0:
-            # the reference's prefix branch (aptserve_flash_attn.py:431-447) attends over the cache through the
-            # block table; the prompt attention here reads only this step's q/k/v
-            raise ValueError("prompt steps with an already-cached prefix (context_lens != 0) are not supported: "
-                             "prefix / chunked-prompt attention over the cache is not built")
+        # a prompt step that continues a cached prefix (chunked prompts, prefix caching): the reference's prefix
+        # branch (aptserve_flash_attn.py:431-447) attends over the K/V cache through the block table
+        prefix = bool(md.num_prefills and md.max_prompt_context_len > 0)
+        if prefix:
+            if md.num_hidden_cache_tokens != 0:
+                raise ValueError("a prompt step that continues a cached prefix cannot hold hidden-cached sequences: "
+                                 "their prefix is cached as hidden rows, not as K/V")
+            if kv_cache is None or self.fp8 or md.block_tables.numel() == 0:
+                raise ValueError("the prefix branch needs a K/V cache in the activation dtype and block tables")
         num_tokens, hidden_size = query.shape
         H, D = self.num_heads, self.head_size
         query = query.view(-1, H, D)
@@ -163,7 +167,13 @@ class HybridAttentionImpl:
         decode_query = query[n_prefill:]
         if md.prefill_metadata is not None:
             pm = md.prefill_metadata
-            if self.prefill_attention is not None:       # caller-supplied prompt attention
+            if prefix:                                   # aptserve_flash_attn.py:431-447
+                ops.flash_attn_varlen_func(
+                    q=query[:n_prefill], k=key_cache, v=value_cache, cu_seqlens_q=pm.query_start_loc,
+                    max_seqlen_q=pm.max_query_len, cu_seqlens_k=pm.seq_start_loc,
+                    max_seqlen_k=pm.max_prefill_seq_len, softmax_scale=self.scale, causal=True,
+                    block_table=pm.block_tables, out=output[:n_prefill])
+            elif self.prefill_attention is not None:     # caller-supplied prompt attention
                 output[:n_prefill] = self.prefill_attention(query[:n_prefill], key[:n_prefill], value[:n_prefill],
                                                             pm.seq_start_loc, pm.max_prefill_seq_len, self.scale)
             else:                                        # aptserve_flash_attn.py:414-426

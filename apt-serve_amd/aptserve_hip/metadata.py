@@ -457,7 +457,10 @@ def build_metadata(is_prompt: bool, seq_lens: Sequence[int], use_hidden: Sequenc
         seq_lens=lens.tolist(), seq_lens_tensor=d_lens, max_query_len=int(qlens.max()),
         max_prefill_seq_len=int(lens.max()), max_decode_seq_len=0, query_start_loc=query_start,
         seq_start_loc=seq_start, context_lens_tensor=ctx,
-        block_tables=torch.empty(B, 0, **i32), use_cuda_graph=False, input_positions=positions, block_types=None,
+        # the tables travel with a prompt step only when it continues a cached prefix (the reference fills them for
+        # prefix hits and chunked prompts: aptserve_model_runner.py:410-437)
+        block_tables=d_bt if (W and int(ctxs.max()) > 0) else torch.empty(B, 0, **i32), use_cuda_graph=False,
+        input_positions=positions, block_types=None,
         token_is_hidden=token_is_hidden, max_prompt_context_len=int(ctxs.max()))
 
 

@@ -690,23 +690,23 @@ def kv_reproject_gathered(hidden_states, paged_cache, holder_src, w_kv, b_kv, ws
 # ------------------------------------------------------------------ prompt attention
 
 def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=None, max_seqlen_k=None,
-                           softmax_scale=None, causal: bool = True, window_size=None, alibi_slopes=None, out=None):
-    """Prompt-step case of the third-party function with the keywords used at
-    additional_designs/attention/backends/aptserve_flash_attn.py:414-426: q, k and v are the
-    packed, freshly projected ``[tokens, H, D]`` tensors of the same sequences
-    (``cu_seqlens_q is cu_seqlens_k``), causal.  Returns ``[tokens, H, D]``."""
+                           softmax_scale=None, causal: bool = True, window_size=None, alibi_slopes=None, out=None,
+                           block_table=None):
+    """Prompt-step cases of the third-party function with the keywords used at
+    additional_designs/attention/backends/aptserve_flash_attn.py:414-426 and :435-447.
+
+    Without ``block_table``: q, k and v are the packed, freshly projected ``[tokens, H, D]`` tensors of the
+    same sequences (``cu_seqlens_q is cu_seqlens_k``), causal.  With ``block_table`` (int32 ``[seqs, W]``, the
+    prefix branch): ``k`` / ``v`` are the ``[blocks, BS, H, D]`` K/V caches, ``cu_seqlens_k`` delimits the
+    sequences' total lengths (cached prefix + this step's tokens, all of them already in the cache) and query
+    ``j`` of a sequence attends to keys ``0 .. j + klen - qlen``.  Returns ``[tokens, H, D]``."""
     dev = q.device
     _need(causal, "only causal attention is provided")
     _need(alibi_slopes is None, "alibi_slopes is not supported")
     _need(window_size in (None, (-1, -1)), "sliding windows are not supported")
     _need(cu_seqlens_q is not None, "cu_seqlens_q is required")
-    _need(cu_seqlens_k is None or cu_seqlens_k is cu_seqlens_q or torch.equal(cu_seqlens_k, cu_seqlens_q),
-          "prompt attention needs identical query and key sequence boundaries")
-    for n, t in (("q", q), ("k", k), ("v", v)):
-        _check_data(n, t, dev)
-        _need(t.dim() == 3 and t.shape == q.shape, f"{n} must be [tokens, heads, head_dim] like q")
-        _need(t.stride(2) == 1 and t.stride(1) == t.size(2), f"{n}: heads of one token must be contiguous")
-        _need(t.dtype == q.dtype, "q, k, v dtypes differ")
+    _check_data("q", q, dev)
+    _need(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.size(2), "q must be [tokens, heads, head_dim]")
     _need(q.dtype in (torch.float16, torch.bfloat16), "f16 or bf16 expected")
     _check_index("cu_seqlens_q", cu_seqlens_q, dev, torch.int32)
     T, H, D = q.shape
@@ -722,6 +722,33 @@ def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_se
         _check_data("out", out, dev)
         _need(out.shape == q.shape and out.dtype == q.dtype and out.stride(2) == 1 and out.stride(1) == D,
               "out must look like q")
+    if block_table is not None:
+        for n, c in (("k", k), ("v", v)):
+            _check_data(n, c, dev)
+            _check_kv_cache(n, c, H, D)
+            _need(c.dtype == q.dtype, "the prefix branch reads caches of the query dtype")
+        _need(k.shape == v.shape and k.stride(0) == v.stride(0), "key and value cache layouts differ")
+        _need(cu_seqlens_k is not None, "the prefix branch needs cu_seqlens_k")
+        _check_index("cu_seqlens_k", cu_seqlens_k, dev, torch.int32)
+        _need(cu_seqlens_k.numel() == n_seq + 1, "cu_seqlens_q and cu_seqlens_k must delimit the same sequences")
+        _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.size(0) == n_seq and
+              block_table.device == dev and (block_table.size(1) <= 1 or block_table.stride(1) == 1),
+              "block_table must be int32 [seqs, width] with contiguous rows on the same GPU")
+        with _on(dev):
+            st = _lib.load().aps_paged_prefill_attention(
+                out.data_ptr() if T else None, q.data_ptr() if T else None, k.data_ptr(), v.data_ptr(),
+                _ptr(block_table), _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), n_seq if T else 0, T, max_len, H, D,
+                k.size(1), block_table.stride(0), block_table.size(1), q.stride(0), out.stride(0), k.stride(0),
+                k.size(0), float(softmax_scale), _DTYPE_CODE[q.dtype], _stream(q))
+        _lib.check(st, "flash_attn_varlen_func (prefix branch)")
+        return out
+    _need(cu_seqlens_k is None or cu_seqlens_k is cu_seqlens_q or torch.equal(cu_seqlens_k, cu_seqlens_q),
+          "prompt attention needs identical query and key sequence boundaries")
+    for n, t in (("k", k), ("v", v)):
+        _check_data(n, t, dev)
+        _need(t.dim() == 3 and t.shape == q.shape, f"{n} must be [tokens, heads, head_dim] like q")
+        _need(t.stride(2) == 1 and t.stride(1) == t.size(2), f"{n}: heads of one token must be contiguous")
+        _need(t.dtype == q.dtype, "q, k, v dtypes differ")
     with _on(dev):
         st = _lib.load().aps_varlen_prefill_attention(
             out.data_ptr() if T else None, q.data_ptr() if T else None, k.data_ptr() if T else None,

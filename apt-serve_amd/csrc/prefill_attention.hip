@@ -13,6 +13,11 @@
 // positions, 8 consecutive d), transposes it in registers and stores 8 rows of V^T; K is staged row-major
 // with its 16-byte chunks XOR-swizzled by key%16 so the fragment reads do not collide in the 64 banks.
 // The next tile's pieces travel global -> registers while the current tile is multiplied.
+//
+// PAGED variant (a prompt step that continues a cached prefix: chunked prompts, prefix caching): the queries are
+// the step's new tokens, the keys and values the whole sequence so far — prefix and new tokens alike — read from
+// the paged K/V cache through the sequence's block table; query i of a sequence with qlen new tokens and klen
+// tokens in all attends to keys 0 .. i + (klen - qlen).  Everything after the address of a key row is shared.
 #include "aps_common.h"
 
 #include <math.h>
@@ -37,6 +42,10 @@ struct PrefillArgs {
   int num_heads;
   int64_t num_tokens;  // rows of q / k / v / out: sequence boundaries outside [0, num_tokens] are not followed
   float scale_log2;
+  // PAGED: k / v are [blocks, block_size, heads, D] caches, k_stride_b / v_stride_b their token row strides
+  const int32_t* cu_seqlens_k; const int32_t* block_tables;
+  int64_t table_stride, table_width, block_stride_b, num_blocks;
+  int block_size;
 };
 
 template <bool BF16>
@@ -65,7 +74,7 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
   }
 }
 
-template <bool BF16, int D>
+template <bool BF16, int D, bool PAGED>
 // Two wavefronts per SIMD: the kernel needs ~244 registers, and left to itself the compiler splits them into
 // 244 + 64 accumulation registers, which leaves room for one.
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void prefill_attention_kernel(
@@ -91,18 +100,24 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int seq = blockIdx.y, head = blockIdx.x;
   const int s0 = a.cu_seqlens[seq], s1 = a.cu_seqlens[seq + 1];
   if (s0 < 0 || s1 < s0 || s1 > a.num_tokens) return;  // boundaries come from device memory: never follow bad ones
-  const int len = s1 - s0;
+  const int qlen = s1 - s0;          // queries of this sequence in this step
+  int len = qlen;                    // keys: the same tokens, or (PAGED) everything cached so far
+  if constexpr (PAGED) {
+    len = a.cu_seqlens_k[seq + 1] - a.cu_seqlens_k[seq];
+    if (len < qlen || (int64_t)(len + a.block_size - 1) / a.block_size > a.table_width) return;
+  }
+  const int off = len - qlen;        // query i sees keys 0 .. i + off
   const int q0 = (int)(gridDim.z - 1 - blockIdx.z) * BQ;
-  if (q0 >= len) return;
+  if (q0 >= qlen) return;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int qcol = lane & 31, half = lane >> 5;
-  const int my_q = q0 + wave * 32 + qcol;      // query index inside the sequence (may be >= len)
-  const bool q_live = my_q < len;
+  const int my_q = q0 + wave * 32 + qcol;      // query index inside the sequence's new tokens (may be >= qlen)
+  const bool q_live = my_q < qlen;
 
   // Q^T fragments: B operand, lane = (query, 8 consecutive d of each 16-wide k-step)
   u32x4 qf[KS];
   {
-    const char* qp = a.q + (int64_t)(s0 + (q_live ? my_q : len - 1)) * a.q_stride_b + (int64_t)head * D * 2;
+    const char* qp = a.q + (int64_t)(s0 + (q_live ? my_q : qlen - 1)) * a.q_stride_b + (int64_t)head * D * 2;
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = *(const u32x4*)(qp + (16 * s + 8 * half) * 2);
   }
@@ -122,8 +137,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   constexpr int PER_K = BKV * KCH / kThreads;
   const bool v_thread = tid < 8 * KCH;           // whole wavefronts
   const int vo = tid / KCH, vch = tid % KCH;
-  const char* k_base = a.k + (int64_t)s0 * a.k_stride_b + (int64_t)head * D * 2;
-  const char* v_base = a.v + (int64_t)s0 * a.v_stride_b + (int64_t)head * D * 2 + vch * 16;
+  const char* k_base = a.k + (PAGED ? 0 : (int64_t)s0 * a.k_stride_b) + (int64_t)head * D * 2;
+  const char* v_base = a.v + (PAGED ? 0 : (int64_t)s0 * a.v_stride_b) + (int64_t)head * D * 2 + vch * 16;
+  // byte offset of key gk of the sequence from k_base / v_base (`stride_b`: the operand's token row stride)
+  auto key_off = [&](int gk, int64_t stride_b) -> int64_t {
+    if constexpr (PAGED) {
+      const int bi = gk / a.block_size;
+      int64_t blk = a.block_tables[(int64_t)seq * a.table_stride + bi];
+      blk = blk < 0 ? 0 : (blk >= a.num_blocks ? a.num_blocks - 1 : blk);  // a bad table: wrong numbers, no fault
+      return blk * a.block_stride_b + (int64_t)(gk - bi * a.block_size) * stride_b;
+    } else {
+      return (int64_t)gk * stride_b;
+    }
+  };
   u32x4 kreg[PER_K], vreg[8];
   auto fetch_tile = [&](int kv0) {
 #pragma unroll
@@ -131,14 +157,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
       const int c = tid + j * kThreads;
       const int key = c / KCH, ch = c % KCH;
       const int gk = min(kv0 + key, len - 1);
-      kreg[j] = *(const u32x4*)(k_base + (int64_t)gk * a.k_stride_b + ch * 16);
+      kreg[j] = *(const u32x4*)(k_base + key_off(gk, a.k_stride_b) + ch * 16);
     }
     if (v_thread) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {  // stored position 8*vo + j holds this key (see the file comment)
         const int key = (vo >> 1) * 16 + (vo & 1) * 4 + (j & 3) + (j >> 2) * 8;
         const int gk = min(kv0 + key, len - 1);
-        vreg[j] = *(const u32x4*)(v_base + (int64_t)gk * a.v_stride_b);
+        vreg[j] = *(const u32x4*)(v_base + key_off(gk, a.v_stride_b));
       }
     }
   };
@@ -162,8 +188,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
   };
 
-  const int kv_end = min(len, q0 + BQ);  // causal: keys beyond the tile's last query are never needed
-  const int wave_q0 = q0 + wave * 32;    // first query of this wavefront
+  const int kv_end = min(len, q0 + BQ + off);  // causal: keys beyond the tile's last query are never needed
+  const int wave_q0 = q0 + wave * 32 + off;    // last key the first query of this wavefront sees
   fetch_tile(0);
   for (int kv0 = 0; kv0 < kv_end; kv0 += BKV) {
     __syncthreads();  // previous tile fully consumed
@@ -198,7 +224,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int key = kv0 + t * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
-          if (!(key <= my_q && key < len)) st[t][e] = -INFINITY;
+          if (!(key <= my_q + off && key < len)) st[t][e] = -INFINITY;
         }
     }
 #pragma unroll
@@ -269,6 +295,29 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
 using namespace aps;
 
+namespace {
+int launch_prefill(PrefillArgs& a, bool paged, int64_t num_seqs, int64_t max_seqlen_q, int num_heads, int head_size,
+                   int dtype, aps_stream_t stream) {
+  const int64_t q_tiles = (max_seqlen_q + BQ - 1) / BQ;
+  if (q_tiles > 65535 || num_seqs > 65535 || num_heads > 65535) return APS_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)num_heads, (unsigned)num_seqs, (unsigned)q_tiles);
+  hipStream_t s = (hipStream_t)stream;
+#define APS_LAUNCH_PF(B, D_, P) APS_LAUNCH((prefill_attention_kernel<B, D_, P>), grid, dim3(kThreads), 0, s, a)
+#define APS_LAUNCH_PF_D(B, P)                                        \
+  do {                                                               \
+    if (head_size == 64) APS_LAUNCH_PF(B, 64, P); else APS_LAUNCH_PF(B, 128, P); \
+  } while (0)
+  if (paged) {
+    if (dtype == APS_F16) APS_LAUNCH_PF_D(false, true); else APS_LAUNCH_PF_D(true, true);
+  } else {
+    if (dtype == APS_F16) APS_LAUNCH_PF_D(false, false); else APS_LAUNCH_PF_D(true, false);
+  }
+#undef APS_LAUNCH_PF_D
+#undef APS_LAUNCH_PF
+  return launch_status();
+}
+}  // namespace
+
 extern "C" {
 
 int aps_varlen_prefill_attention(void* out, const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
@@ -288,26 +337,49 @@ int aps_varlen_prefill_attention(void* out, const void* q, const void* k, const 
                         (uint64_t)v_stride * 2}) != 16 ||
       common_vec_bytes({addr(out), (uint64_t)out_stride * 2}) < 8)
     return APS_ERR_UNSUPPORTED;
-  if (num_seqs > 65535 || num_heads > 65535) return APS_ERR_UNSUPPORTED;
-  PrefillArgs a;
+  PrefillArgs a{};
   a.q = (const char*)q; a.k = (const char*)k; a.v = (const char*)v; a.out = (char*)out;
   a.cu_seqlens = cu_seqlens;
   a.q_stride_b = q_stride * 2; a.k_stride_b = k_stride * 2; a.v_stride_b = v_stride * 2; a.out_stride_b = out_stride * 2;
   a.num_heads = num_heads;
   a.num_tokens = num_tokens;
   a.scale_log2 = softmax_scale * kLog2e;
-  const int64_t q_tiles = (max_seqlen + BQ - 1) / BQ;
-  if (q_tiles > 65535) return APS_ERR_UNSUPPORTED;
-  const dim3 grid((unsigned)num_heads, (unsigned)num_seqs, (unsigned)q_tiles);
-  hipStream_t s = (hipStream_t)stream;
-  if (dtype == APS_F16) {
-    if (head_size == 64) APS_LAUNCH((prefill_attention_kernel<false, 64>), grid, dim3(kThreads), 0, s, a);
-    else APS_LAUNCH((prefill_attention_kernel<false, 128>), grid, dim3(kThreads), 0, s, a);
-  } else {
-    if (head_size == 64) APS_LAUNCH((prefill_attention_kernel<true, 64>), grid, dim3(kThreads), 0, s, a);
-    else APS_LAUNCH((prefill_attention_kernel<true, 128>), grid, dim3(kThreads), 0, s, a);
-  }
-  return launch_status();
+  return launch_prefill(a, false, num_seqs, max_seqlen, num_heads, head_size, dtype, stream);
+}
+
+int aps_paged_prefill_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                const int32_t* block_tables, const int32_t* cu_seqlens_q,
+                                const int32_t* cu_seqlens_k, int64_t num_seqs, int64_t num_q_tokens,
+                                int64_t max_seqlen_q, int num_heads, int head_size, int block_size,
+                                int64_t table_stride, int64_t table_width, int64_t q_stride, int64_t out_stride,
+                                int64_t cache_block_stride, int64_t num_cache_blocks, float softmax_scale, int dtype,
+                                aps_stream_t stream) {
+  if (num_seqs < 0 || num_q_tokens < 0 || max_seqlen_q < 0 || num_heads <= 0 || head_size <= 0 || block_size <= 0 ||
+      table_width < 0 || num_cache_blocks < 0)
+    return APS_ERR_INVALID_ARG;
+  if (!(softmax_scale > 0.f) || softmax_scale > 3.0e38f) return APS_ERR_INVALID_ARG;
+  if (num_seqs == 0 || num_q_tokens == 0 || max_seqlen_q == 0) return APS_OK;
+  if (!out || !q || !k_cache || !v_cache || !block_tables || !cu_seqlens_q || !cu_seqlens_k || num_cache_blocks == 0)
+    return APS_ERR_INVALID_ARG;
+  if (dtype != APS_F16 && dtype != APS_BF16) return APS_ERR_UNSUPPORTED;
+  if (head_size != 64 && head_size != 128) return APS_ERR_UNSUPPORTED;
+  const int64_t row = (int64_t)num_heads * head_size;
+  if (q_stride < row || out_stride < row || cache_block_stride < row * block_size || table_stride < table_width)
+    return APS_ERR_INVALID_ARG;
+  if (common_vec_bytes({addr(q), addr(k_cache), addr(v_cache), (uint64_t)q_stride * 2,
+                        (uint64_t)cache_block_stride * 2}) != 16 ||
+      common_vec_bytes({addr(out), (uint64_t)out_stride * 2}) < 8)
+    return APS_ERR_UNSUPPORTED;
+  PrefillArgs a{};
+  a.q = (const char*)q; a.k = (const char*)k_cache; a.v = (const char*)v_cache; a.out = (char*)out;
+  a.cu_seqlens = cu_seqlens_q; a.cu_seqlens_k = cu_seqlens_k; a.block_tables = block_tables;
+  a.q_stride_b = q_stride * 2; a.k_stride_b = row * 2; a.v_stride_b = row * 2; a.out_stride_b = out_stride * 2;
+  a.table_stride = table_stride; a.table_width = table_width;
+  a.block_stride_b = cache_block_stride * 2; a.num_blocks = num_cache_blocks; a.block_size = block_size;
+  a.num_heads = num_heads;
+  a.num_tokens = num_q_tokens;
+  a.scale_log2 = softmax_scale * kLog2e;
+  return launch_prefill(a, true, num_seqs, max_seqlen_q, num_heads, head_size, dtype, stream);
 }
 
 }  // extern "C"

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define APS_ABI_VERSION 7
+#define APS_ABI_VERSION 8
 
 typedef void* aps_stream_t; /* a hipStream_t; NULL = the null stream */
 
@@ -317,6 +317,29 @@ int aps_varlen_prefill_attention(void* out, const void* q, const void* k,
                                  int64_t v_stride, int64_t out_stride,
                                  float softmax_scale, int dtype,
                                  aps_stream_t stream);
+
+/* Prompt-step attention that continues a cached prefix (chunked prompts, prefix
+ * caching).  ref: third-party vllm_flash_attn.flash_attn_varlen_func with
+ * block_table=, as called at attention/backends/aptserve_flash_attn.py:431-447
+ * (k=key_cache, v=value_cache, cu_seqlens_q=query_start_loc,
+ * cu_seqlens_k=seq_start_loc, causal=True).  The queries are the step's new
+ * tokens, packed and delimited by cu_seqlens_q; sequence i has
+ * klen = cu_seqlens_k[i+1] - cu_seqlens_k[i] tokens in all (prefix + new), whose
+ * K / V rows are read from the [blocks, block_size, H, D] caches through
+ * block_tables[i, j / block_size] (the new tokens' rows must have been written
+ * already); query j of its qlen new tokens attends to keys 0 .. j + klen - qlen
+ * (bottom-right aligned causal mask).  A sequence with klen < qlen, with more
+ * blocks than table_width or with bad boundaries is skipped; block ids are
+ * clamped into [0, num_cache_blocks).  Otherwise as aps_varlen_prefill_attention
+ * (dtypes, head sizes, softmax_scale > 0, max_seqlen_q bounds the qlen). */
+int aps_paged_prefill_attention(
+    void* out, const void* q, const void* k_cache, const void* v_cache,
+    const int32_t* block_tables, const int32_t* cu_seqlens_q,
+    const int32_t* cu_seqlens_k, int64_t num_seqs, int64_t num_q_tokens,
+    int64_t max_seqlen_q, int num_heads, int head_size, int block_size,
+    int64_t table_stride, int64_t table_width, int64_t q_stride,
+    int64_t out_stride, int64_t cache_block_stride, int64_t num_cache_blocks,
+    float softmax_scale, int dtype, aps_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Ragged-batch metadata, built on the GPU from a per-sequence description.

@@ -107,6 +107,29 @@ def varlen_causal_attention(q, k, v, cu_seqlens, softmax_scale):
     return out
 
 
+def paged_prefix_attention(q, k_cache, v_cache, block_tables, cu_seqlens_q, cu_seqlens_k, softmax_scale):
+    """``flash_attn_varlen_func(q, k=key_cache, v=value_cache, cu_seqlens_q=, cu_seqlens_k=, causal=True,
+    block_table=)`` as called at additional_designs/attention/backends/aptserve_flash_attn.py:431-447 (the
+    prefix branch), restated from the third-party function's published definition: the queries of sequence
+    ``b`` are rows ``cu_seqlens_q[b]:cu_seqlens_q[b+1]`` of ``q``, its keys and values the first
+    ``klen = cu_seqlens_k[b+1] - cu_seqlens_k[b]`` tokens read through ``block_tables[b]``, and with fewer
+    queries than keys the causal mask is aligned to the bottom right: query ``j`` sees keys
+    ``0 .. j + klen - qlen``.  fp32 result ``[tokens, H, D]``."""
+    out = torch.zeros(q.shape, dtype=torch.float32)
+    for b in range(len(cu_seqlens_q) - 1):
+        q0, q1 = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1])
+        klen = int(cu_seqlens_k[b + 1]) - int(cu_seqlens_k[b])
+        qlen = q1 - q0
+        if qlen == 0:
+            continue
+        k, v = materialize_kv(k_cache, v_cache, block_tables[b], klen)          # [klen, H, D] fp32
+        s = torch.einsum("qhd,khd->hqk", q[q0:q1].float(), k) * softmax_scale
+        visible = torch.arange(klen)[None, :] <= (torch.arange(qlen)[:, None] + (klen - qlen))
+        s = s.masked_fill(~visible[None], float("-inf"))
+        out[q0:q1] = torch.einsum("hqk,khd->qhd", torch.softmax(s, dim=-1), v)
+    return out
+
+
 def absorbed_hidden_attention(q, hidden_rows, w_k, w_v, b_v, softmax_scale):
     """Decode attention of ONE hidden-cached sequence computed on its cached hidden rows,
     without materialising K and V ("absorbed" projection weights).

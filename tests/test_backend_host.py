@@ -22,15 +22,23 @@ def _prompt_metadata(context_len):
         block_tables=torch.empty(1, 0, dtype=torch.int32), max_prompt_context_len=context_len)
 
 
-def test_prompt_step_with_cached_prefix_is_rejected_before_any_launch():
-    """seq_start_loc counts whole sequences while q/k/v hold only the new tokens: handing that to the prompt
-    attention would read past the step's rows, so the dispatcher refuses (the reference's prefix branch,
-    additional_designs/attention/backends/aptserve_flash_attn.py:431-447, has no counterpart here)."""
+def test_prefix_branch_without_a_cache_or_with_hidden_sequences_is_rejected_before_any_launch():
+    """A prompt step that continues a cached prefix takes the prefix branch
+    (additional_designs/attention/backends/aptserve_flash_attn.py:431-447), which reads K/V through the block
+    tables: without a K/V cache and tables there is nothing to read (seq_start_loc counts whole sequences while
+    q/k/v hold only the new tokens, so the plain prompt attention must not be used either), and a hidden-cached
+    sequence keeps no K/V of its prefix."""
     impl = HybridAttentionImpl(2, 64, 0.125)
     md = _prompt_metadata(context_len=3)
     q = torch.zeros(5, 128, dtype=torch.float16)
-    with pytest.raises(ValueError, match="context_lens"):
-        impl.forward(q, q, q, None, None, md)
+    with pytest.raises(ValueError, match="prefix branch"):
+        impl.forward(q, q, q, None, None, md)                       # no cache
+    cache = torch.zeros(2, 4, 16, 2, 64, dtype=torch.float16)
+    with pytest.raises(ValueError, match="prefix branch"):
+        impl.forward(q, q, q, cache, None, md)                      # no block tables
+    md.num_hidden_cache_tokens = 5
+    with pytest.raises(ValueError, match="hidden-cached"):
+        impl.forward(q, q, q, cache, None, md)
 
 
 def test_constructor_rejects_what_the_reference_rejects():

@@ -226,3 +226,51 @@ def test_absorbed_attention_equals_attention_over_reprojected_kv(L):
     assert not torch.allclose(OA.absorbed_hidden_attention(q, x, wk, wv, None, scale), ref, atol=1e-3)
     if L > 1:
         assert not torch.allclose(OA.absorbed_hidden_attention(q, x, wk.t().contiguous(), wv, bv, scale), ref, atol=1e-3)
+
+
+def test_prefix_attention_pinned_by_dense_softmax_and_its_two_limits():
+    """``paged_prefix_attention`` (the prefix branch's flash_attn_varlen_func call): (a) every query row against a
+    float64 softmax over the keys it may see, written from the definition; (b) with no prefix it is the plain
+    causal prompt attention; (c) with one new token per sequence it is the decode attention."""
+    B, H, D, BS = 3, 2, 8, 16
+    klens, qlens = [37, 16, 50], [5, 16, 1]
+    kc, vc, bt, k_dense, v_dense = build_paged(B, H, D, BS, klens, 11)
+    q = randn((sum(qlens), H, D), 12)
+    cu_q = torch.tensor([0] + list(np.cumsum(qlens)), dtype=torch.int32)
+    cu_k = torch.tensor([0] + list(np.cumsum(klens)), dtype=torch.int32)
+    out = OA.paged_prefix_attention(q, kc, vc, bt, cu_q, cu_k, 0.3)
+    row = 0
+    for b in range(B):
+        for j in range(qlens[b]):
+            n_vis = j + klens[b] - qlens[b] + 1                       # keys 0 .. j + klen - qlen
+            for h in range(H):
+                s = (k_dense[b][:n_vis, h].double() @ q[row, h].double()) * 0.3
+                p = torch.softmax(s, 0)
+                assert torch.allclose(out[row, h].double(), p @ v_dense[b][:n_vis, h].double(), atol=1e-5)
+            row += 1
+    # (b) no prefix: klen == qlen
+    q2 = randn((sum(klens), H, D), 13)
+    k2, v2 = torch.cat(k_dense), torch.cat(v_dense)
+    full = OA.paged_prefix_attention(q2, kc, vc, bt, cu_k, cu_k, 0.3)
+    assert torch.allclose(full, OA.varlen_causal_attention(q2, k2, v2, cu_k, 0.3), atol=1e-5)
+    # (c) one query per sequence
+    q3 = randn((B, H, D), 14)
+    one = OA.paged_prefix_attention(q3, kc, vc, bt, torch.arange(B + 1, dtype=torch.int32), cu_k, 0.3)
+    dec = OA.paged_decode_attention(q3, kc, vc, bt, torch.tensor(klens, dtype=torch.int32), 0.3)
+    assert torch.allclose(one, dec, atol=1e-5)
+
+
+def test_chunked_prompt_equals_one_shot_prompt():
+    """The rows a prompt's second chunk produces through the prefix branch are the rows the whole prompt
+    produces in one step."""
+    H, D, BS = 2, 8, 16
+    klens, ctx = [45, 20], [30, 7]
+    kc, vc, bt, k_dense, v_dense = build_paged(2, H, D, BS, klens, 21)
+    q_full = randn((sum(klens), H, D), 22)
+    cu_k = torch.tensor([0] + list(np.cumsum(klens)), dtype=torch.int32)
+    one_shot = OA.varlen_causal_attention(q_full, torch.cat(k_dense), torch.cat(v_dense), cu_k, 0.25)
+    new = [torch.arange(int(cu_k[b]) + ctx[b], int(cu_k[b + 1])) for b in range(2)]
+    idx = torch.cat(new)
+    cu_q = torch.tensor([0] + list(np.cumsum([len(n) for n in new])), dtype=torch.int32)
+    chunk = OA.paged_prefix_attention(q_full[idx], kc, vc, bt, cu_q, cu_k, 0.25)
+    assert torch.allclose(chunk, one_shot[idx], atol=1e-5)

@@ -72,3 +72,83 @@ def test_argument_validation(dev):
             ops.flash_attn_varlen_func(q, q, q, cu_seqlens_q=cu, max_seqlen_q=8, softmax_scale=bad)
     e = torch.zeros(0, 2, 64, dtype=torch.float16, device=dev)
     assert ops.flash_attn_varlen_func(e, e, e, cu_seqlens_q=cu[:1], max_seqlen_q=0).shape == (0, 2, 64)
+
+
+# ------------------------------------------------------------------ prefix branch (keys from the paged cache)
+
+def run_prefix(dev, klens, qlens, H, D, dtype=torch.float16, seed=0, BS=16):
+    from test_oracle_attention import build_paged
+    B = len(klens)
+    kc, vc, bt, _, _ = build_paged(B, H, D, BS, klens, seed, dtype=dtype)
+    q = randn((sum(qlens), H, D), seed + 5, dtype)
+    cu_q = torch.tensor([0] + list(np.cumsum(qlens)), dtype=torch.int32)
+    cu_k = torch.tensor([0] + list(np.cumsum(klens)), dtype=torch.int32)
+    ref = OA.paged_prefix_attention(q, kc, vc, bt, cu_q, cu_k, D ** -0.5)
+    out = ops.flash_attn_varlen_func(q=q.to(dev), k=kc.to(dev), v=vc.to(dev), cu_seqlens_q=cu_q.to(dev),
+                                     cu_seqlens_k=cu_k.to(dev), max_seqlen_q=max(qlens), max_seqlen_k=max(klens),
+                                     softmax_scale=D ** -0.5, causal=True, block_table=bt.to(dev))
+    out = out.float().cpu()
+    tol = 5e-3 if dtype == torch.float16 else 2e-2
+    assert torch.allclose(out, ref, atol=tol, rtol=tol), (out - ref).abs().max().item()
+    return out
+
+
+@pytest.mark.parametrize("H,D,dtype", [(3, 64, torch.float16), (2, 128, torch.bfloat16), (40, 128, torch.float16)])
+def test_prefix_attention_over_the_paged_cache(dev, H, D, dtype):
+    """New tokens of a prompt attend over the whole sequence in the cache (aptserve_flash_attn.py:431-447):
+    prefixes of 0 .. several tiles, chunks of 1 .. several query tiles, prefix lengths that are no multiple of the
+    block or tile size."""
+    klens = [37, 16, 300, 129, 64, 700, 1]
+    qlens = [5, 16, 130, 1, 64, 257, 1]
+    run_prefix(dev, klens, qlens, H, D, dtype)
+
+
+def test_prefix_attention_block_size_32_and_argument_errors(dev):
+    run_prefix(dev, [100, 45], [33, 45], 4, 64, BS=32, seed=3)
+    from test_oracle_attention import build_paged
+    kc, vc, bt, _, _ = build_paged(1, 2, 64, 16, [20], 1)
+    q = randn((4, 2, 64), 2).to(dev)
+    cu_q, cu_k = torch.tensor([0, 4], dtype=torch.int32, device=dev), torch.tensor([0, 20], dtype=torch.int32, device=dev)
+    with pytest.raises(ValueError):        # no key boundaries
+        ops.flash_attn_varlen_func(q, kc.to(dev), vc.to(dev), cu_seqlens_q=cu_q, max_seqlen_q=4, block_table=bt.to(dev))
+    with pytest.raises(ValueError):        # int64 table
+        ops.flash_attn_varlen_func(q, kc.to(dev), vc.to(dev), cu_seqlens_q=cu_q, cu_seqlens_k=cu_k, max_seqlen_q=4,
+                                   block_table=bt.long().to(dev))
+    # a sequence with more new tokens than tokens in all is skipped, not read out of bounds
+    out = torch.full_like(q, 7.0)
+    bad_k = torch.tensor([0, 2], dtype=torch.int32, device=dev)
+    ops.flash_attn_varlen_func(q, kc.to(dev), vc.to(dev), cu_seqlens_q=cu_q, cu_seqlens_k=bad_k, max_seqlen_q=4,
+                               block_table=bt.to(dev), out=out)
+    torch.cuda.synchronize()
+    assert (out == 7).all()
+
+
+def test_chunked_prompt_through_the_dispatcher_equals_one_shot(dev):
+    """A prompt step over 2 K/V-cached prompts, then the same prompts in two chunks (the second chunk takes the
+    dispatcher's prefix branch over the cache the first chunk filled): same attention output rows, same cache."""
+    from aptserve_hip import backend, metadata
+    H, D, BS, N = 12, 64, 16, 32
+    lens, ctx = [45, 20], [30, 7]
+    tables = [[3, 9, 1], [7, 4]]
+    T = sum(lens)
+    q, k, v = (randn((T, H * D), 30 + i).to(dev) for i in range(3))
+    impl = backend.HybridAttentionImpl(H, D, D ** -0.5)
+    kv1 = torch.zeros(2, N, BS, H, D, dtype=torch.float16, device=dev)
+    md = metadata.build_metadata(True, lens, [False, False], tables, [[], []], BS, dev)
+    one_shot = impl.forward(q, k, v, kv1, None, md)
+    # chunk 1: the first ctx tokens of each prompt; chunk 2: the rest, with context_lens = ctx
+    starts = np.cumsum([0] + lens)
+    first = torch.cat([torch.arange(starts[b], starts[b] + ctx[b]) for b in range(2)]).to(dev)
+    rest = torch.cat([torch.arange(starts[b] + ctx[b], starts[b + 1]) for b in range(2)]).to(dev)
+    kv2 = torch.zeros_like(kv1)
+    md_a = metadata.build_metadata(True, ctx, [False, False], tables, [[], []], BS, dev)
+    impl.forward(q[first], k[first], v[first], kv2, None, md_a)
+    md_b = metadata.build_metadata(True, lens, [False, False], tables, [[], []], BS, dev, context_lens=ctx)
+    assert md_b.max_prompt_context_len == 30 and md_b.block_tables.shape == (2, 3)
+    second = impl.forward(q[rest], k[rest], v[rest], kv2, None, md_b)
+    assert torch.equal(kv1, kv2)
+    assert torch.allclose(second.float(), one_shot[rest].float(), atol=5e-3, rtol=5e-3)
+    # hidden-cached prompts cannot continue a prefix: their prefix holds no K/V
+    md_h = metadata.build_metadata(True, lens, [True, False], tables, [[], []], BS, dev, context_lens=ctx)
+    with pytest.raises(ValueError):
+        impl.forward(q[rest], k[rest], v[rest], kv2, None, md_h)
