@@ -288,20 +288,26 @@ class HybridOPTAttention:
         w, b = self.qkv_proj.weight, self.qkv_proj.bias
         s = w.shape[0] // 3
         H, D = self.num_heads, self.head_dim
-        # the newest hidden row of every hidden-cached sequence joins its cache first
         a = self.attn
-        with phase("write"):
-            ops.hidden_to_cache(hidden_states, hidden_cache, md.slot_mapping, md.hidden_cache_use_input,
-                                md.hidden_cache_store_tot)
         n_kv = md.num_decode_tokens - md.num_hidden_cache_tokens
         attn_output = torch.empty_like(hidden_states)
+        one_write = n_kv and not a.fp8 and md.kv_cache_use_input is not None and md.new_token_slot is not None
+        if not one_write:      # the newest hidden row of every hidden-cached sequence joins its cache
+            with phase("write"):
+                ops.hidden_to_cache(hidden_states, hidden_cache, md.slot_mapping, md.hidden_cache_use_input,
+                                    md.hidden_cache_store_tot)
         if n_kv:
             with phase("projections"):
                 qkv, _ = self.qkv_proj(hidden_states)
                 q, k, v = qkv.chunk(chunks=3, dim=-1)
             with phase("write"):
-                ops.reshape_and_cache_flash(k, v, kv_cache[0], kv_cache[1], md.new_token_slot, a.kv_cache_dtype,
-                                            a.k_scale, a.v_scale, token_idx=md.kv_cache_use_input)
+                if one_write:  # ... in the same launch as the newest K/V rows of the K/V-cached sequences
+                    ops.decode_step_cache_ops(None, hidden_states, hidden_cache, None, md.slot_mapping,
+                                              md.hidden_cache_use_input, md.hidden_cache_store_tot, k, v,
+                                              md.kv_cache_use_input, md.new_token_slot, kv_cache=kv_cache)
+                else:
+                    ops.reshape_and_cache_flash(k, v, kv_cache[0], kv_cache[1], md.new_token_slot, a.kv_cache_dtype,
+                                                a.k_scale, a.v_scale, token_idx=md.kv_cache_use_input)
             with phase("attention"):
                 ops.paged_decode_attention(q.view(-1, H, D), kv_cache[0], kv_cache[1], md.private_block_tables,
                                            md.kv_seq_lens, self.scaling, max_seq_len=md.max_kv_seq_len or None,

@@ -189,47 +189,57 @@ def gather_hidden_rows(holder, hidden_states, paged_cache, holder_src, slot_mapp
 
 
 def decode_step_cache_ops(holder, hidden_states, paged_cache, holder_src, slot_mapping, hidden_cache_use_input,
-                          hidden_cache_store_tot, key, value, kv_cache_use_input, new_token_slot) -> None:
+                          hidden_cache_store_tot, key, value, kv_cache_use_input, new_token_slot,
+                          kv_cache=None) -> None:
     """The cache traffic of one decode layer in one launch: ``gather_hidden_rows`` (store of the newest hidden
     rows, holder assembly: additional_designs/model_executor/models/aptserve_opt.py:108-121) and the write of
     the newest K/V rows of the K/V-cached sequences into the two planes of ``paged_cache``
     (``reshape_and_cache_flash``, additional_designs/attention/backends/aptserve_flash_attn.py:338-345).
     ``key`` / ``value`` ``[batch, H*D]`` or ``[batch, H, D]``; ``kv_cache_use_input`` and ``new_token_slot``
-    from the metadata builder.  Same bytes in the cache and the holder as the two separate calls."""
-    dev = holder.device
-    for n, t in (("holder", holder), ("hidden_states", hidden_states), ("paged_cache", paged_cache),
-                 ("key", key), ("value", value)):
+    from the metadata builder.  Same bytes in the cache and the holder as the two separate calls.
+    ``holder`` (and ``holder_src``) may be ``None``: the stores alone, for a data flow that assembles no holder.
+    ``kv_cache``: the K/V planes when they are not ``paged_cache`` (a separate hidden-row cache)."""
+    dev = hidden_states.device
+    for n, t in (("hidden_states", hidden_states), ("paged_cache", paged_cache), ("key", key), ("value", value)):
         _check_data(n, t, dev)
-    _need(holder.dim() == 2 and hidden_states.dim() == 2, "holder and hidden_states must be 2-D")
+    _need(hidden_states.dim() == 2, "hidden_states must be 2-D")
     width = hidden_states.size(1)
-    _need(holder.size(1) == width, "holder and hidden_states widths differ")
-    _need(holder.dtype == hidden_states.dtype == paged_cache.dtype == key.dtype == value.dtype, "dtypes differ")
-    _check_paged(paged_cache, width)
-    _need(paged_cache.size(0) == 2 and paged_cache.size(3) * paged_cache.size(4) == width,
-          "paged_cache must be (2, num_blocks, block_size, heads, head_dim) with heads*head_dim == hidden width")
-    key = _as_thd("key", key, paged_cache.size(3), paged_cache.size(4))
-    value = _as_thd("value", value, paged_cache.size(3), paged_cache.size(4))
+    n_rows = slot_mapping.numel()
+    if holder is not None:
+        _check_data("holder", holder, dev)
+        _need(holder.dim() == 2 and holder.size(1) == width and holder.dtype == hidden_states.dtype,
+              "holder must be 2-D, as wide as hidden_states and of its dtype")
+        _need(holder.size(0) == n_rows, "slot_mapping must have one entry per holder row")
+        _check_index("holder_src", holder_src, dev)
+        _need(holder_src.numel() == n_rows, "holder_src must have one entry per holder row")
+    kvc = paged_cache if kv_cache is None else kv_cache
+    _check_data("kv_cache", kvc, dev)
+    _need(hidden_states.dtype == paged_cache.dtype == kvc.dtype == key.dtype == value.dtype, "dtypes differ")
+    for c in (paged_cache, kvc):
+        _check_paged(c, width)
+        _need(c.size(0) == 2 and c.size(3) * c.size(4) == width,
+              "a cache must be (2, num_blocks, block_size, heads, head_dim) with heads*head_dim == hidden width")
+    key = _as_thd("key", key, kvc.size(3), kvc.size(4))
+    value = _as_thd("value", value, kvc.size(3), kvc.size(4))
     B = hidden_states.size(0)
     _need(key.size(0) == B and value.size(0) == B, "one key / value row per sequence expected")
-    for n, t in (("holder_src", holder_src), ("slot_mapping", slot_mapping),
-                 ("hidden_cache_use_input", hidden_cache_use_input),
+    for n, t in (("slot_mapping", slot_mapping), ("hidden_cache_use_input", hidden_cache_use_input),
                  ("hidden_cache_store_tot", hidden_cache_store_tot), ("kv_cache_use_input", kv_cache_use_input),
                  ("new_token_slot", new_token_slot)):
         _check_index(n, t, dev)
-    _need(holder_src.numel() == holder.size(0), "holder_src must have one entry per holder row")
-    _need(slot_mapping.numel() == holder.size(0), "slot_mapping must have one entry per holder row")
     _need(hidden_cache_use_input.numel() == hidden_cache_store_tot.numel(), "store index lengths differ")
     _need(new_token_slot.numel() == B, "new_token_slot must have one entry per sequence")
     slot_stride = paged_cache.stride(2)
     with _on(dev):
         st = _lib.load().aps_decode_step_cache_ops(
-            holder.data_ptr(), hidden_states.data_ptr(), paged_cache.data_ptr(), _ptr(holder_src), holder.size(0),
+            None if holder is None else _ptr(holder), hidden_states.data_ptr(), paged_cache.data_ptr(),
+            None if holder is None else _ptr(holder_src), n_rows,
             _ptr(slot_mapping), _ptr(hidden_cache_use_input), _ptr(hidden_cache_store_tot),
-            hidden_cache_store_tot.numel(), B, width, holder.stride(0), hidden_states.stride(0), slot_stride,
-            paged_cache.numel() // slot_stride, key.data_ptr(), value.data_ptr(), paged_cache[0].data_ptr(),
-            paged_cache[1].data_ptr(), _ptr(kv_cache_use_input), _ptr(new_token_slot), kv_cache_use_input.numel(),
-            key.stride(0), value.stride(0), paged_cache.size(2), paged_cache.stride(1), paged_cache.size(1),
-            holder.element_size(), _stream(holder))
+            hidden_cache_store_tot.numel(), B, width, 0 if holder is None else holder.stride(0), hidden_states.stride(0),
+            slot_stride, paged_cache.numel() // slot_stride, key.data_ptr(), value.data_ptr(), kvc[0].data_ptr(),
+            kvc[1].data_ptr(), _ptr(kv_cache_use_input), _ptr(new_token_slot), kv_cache_use_input.numel(),
+            key.stride(0), value.stride(0), kvc.size(2), kvc.stride(1), kvc.size(1),
+            hidden_states.element_size(), _stream(hidden_states))
     _lib.check(st, "decode_step_cache_ops")
 
 
@@ -526,7 +536,25 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, block_table=None, cache_seqlens
 
 # --------------------------------------------------------------------- a5 / a6
 
-def linear_nt(x, weight, bias=None, out=None, out_row_map=None, workspace=None, split_k: bool = True):
+_TILE_COUNTERS = {}
+
+
+def _tile_counters(dev) -> torch.Tensor:
+    """The zero-initialised tile counters of ``aps_linear_nt`` for the current stream of ``dev``: every call
+    leaves them zero again, and calls on one stream run one after the other, so one array per (device, stream)
+    serves them all.  Under stream capture the array of the capturing stream is the one a replay uses."""
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    t = _TILE_COUNTERS.get(key)
+    if t is None:
+        with torch.cuda.stream(torch.cuda.default_stream(dev)):     # allocated and cleared outside any capture
+            t = torch.zeros(256, dtype=torch.int32, device=dev)
+        torch.cuda.default_stream(dev).synchronize()
+        _TILE_COUNTERS[key] = t
+    return t
+
+
+def linear_nt(x, weight, bias=None, out=None, out_row_map=None, workspace=None, split_k: bool = True,
+              relu: bool = False):
     """``out = x @ weight.T + bias`` on the matrix cores (f16/bf16, fp32 accumulation).
 
     ``x [M, K]`` and ``weight [N, K]`` may be row-strided views (a row slice of the fused
@@ -534,6 +562,10 @@ def linear_nt(x, weight, bias=None, out=None, out_row_map=None, workspace=None, 
     ``out_row_map`` (int64 ``[M]``) scatters result row ``m`` to ``out[out_row_map[m]]``.
     With ``split_k`` (default) a problem of few output tiles is split along K through an fp32
     ``workspace`` (allocated here when not given) so that enough workgroups stream the weights.
+    ``relu``: negative results are stored as zero (``fc1`` with the activation that follows it,
+    additional_designs/model_executor/models/aptserve_opt.py:205-206).
+    The K split of a decode step's few rows is summed inside the same launch (by the workgroup that finishes a
+    tile last) with the help of a small array of counters kept per device and stream (:func:`_tile_counters`).
     """
     dev = x.device
     _check_data("x", x, dev)
@@ -565,8 +597,10 @@ def linear_nt(x, weight, bias=None, out=None, out_row_map=None, workspace=None, 
         st = lib.aps_linear_nt(
             x.data_ptr() if M else None, weight.data_ptr(), None if bias is None else bias.data_ptr(),
             out.data_ptr() if out.numel() else None, M, N, K, x.stride(0), weight.stride(0), out.stride(0),
-            None if out_row_map is None else _ptr(out_row_map), out.size(0), _DTYPE_CODE[x.dtype], ws_ptr,
-            workspace.numel() * workspace.element_size() if need else 0, _stream(x))
+            None if out_row_map is None else _ptr(out_row_map), out.size(0), _DTYPE_CODE[x.dtype],
+            1 if relu else 0, ws_ptr,
+            workspace.numel() * workspace.element_size() if need else 0,
+            _tile_counters(dev).data_ptr() if need else None, _stream(x))
     _lib.check(st, "linear_nt")
     return out
 

@@ -69,10 +69,10 @@ class HybridOPTDecoderLayer:
                                             w[prefix + "qkv_b"], w[prefix + "out_w"], w[prefix + "out_b"], **attn_kw)
 
     def _mlp(self, x):
+        """fc1 with its ReLU (stored by fc1's own epilogue), then fc2."""
         w, p = self.w, self.p
         with phase("projections"):
-            x = ops.linear_nt(x, w[p + "fc1_w"], w[p + "fc1_b"])
-            x = torch.relu_(x)
+            x = ops.linear_nt(x, w[p + "fc1_w"], w[p + "fc1_b"], relu=True)
             return ops.linear_nt(x, w[p + "fc2_w"], w[p + "fc2_b"])
 
     def forward(self, hidden_states, kv_cache, shared_cache, md: HybridAttentionMetadata):

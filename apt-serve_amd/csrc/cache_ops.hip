@@ -168,6 +168,7 @@ struct ResolvedGatherOp {
   const int64_t* use_input; const int64_t* store_tot;
   int64_t n_rows, n_store, n_inputs;
   int64_t holder_stride_b, hidden_stride_b, slot_stride_b, num_slots;
+  int64_t n_map;  // entries of slot_mapping (= n_rows unless no holder is assembled)
   __device__ RowDesc operator()(int64_t i) const {
     RowDesc r{nullptr, nullptr};
     if (i < n_rows) {
@@ -182,7 +183,7 @@ struct ResolvedGatherOp {
       const int64_t j = i - n_rows;
       const int64_t b = use_input[j];
       const int64_t t = store_tot[j];
-      if (b < 0 || b >= n_inputs || t < 0 || t >= n_rows) return r;
+      if (b < 0 || b >= n_inputs || t < 0 || t >= n_map) return r;
       const int64_t slot = slot_mapping[t];
       if (slot < 0 || slot >= num_slots) return r;
       r.src = hidden_states + b * hidden_stride_b;
@@ -612,7 +613,7 @@ int aps_gather_hidden_rows(void* holder, const void* hidden_states, void* paged_
   const int64_t e = elem_size;
   ResolvedGatherOp op{(char*)holder, (const char*)hidden_states, (char*)paged_cache, holder_src, slot_mapping,
                       hidden_cache_use_input, hidden_cache_store_tot, n_rows, n_store, num_inputs,
-                      holder_stride * e, hidden_stride * e, slot_stride * e, num_slots};
+                      holder_stride * e, hidden_stride * e, slot_stride * e, num_slots, n_rows};
   const int vb = common_vec_bytes({addr(holder), addr(hidden_states), addr(paged_cache),
                                    (uint64_t)(holder_stride * e), (uint64_t)(hidden_stride * e),
                                    (uint64_t)(slot_stride * e), (uint64_t)(hidden_size * e)});
@@ -630,12 +631,11 @@ int aps_decode_step_cache_ops(void* holder, const void* hidden_states, void* pag
   if (n_rows < 0 || n_store < 0 || n_kv < 0 || num_inputs < 0 || hidden_size < 0 || !valid_elem(elem_size))
     return APS_ERR_INVALID_ARG;
   if (n_rows + n_store + n_kv == 0 || hidden_size == 0) return APS_OK;
-  if ((n_rows || n_store) && (!holder || !hidden_states || !paged_cache)) return APS_ERR_INVALID_ARG;
-  if (n_rows && !holder_src) return APS_ERR_INVALID_ARG;
+  if ((n_rows || n_store) && (!hidden_states || !paged_cache)) return APS_ERR_INVALID_ARG;
+  if (n_rows && holder && !holder_src) return APS_ERR_INVALID_ARG;
   if (n_store && (!slot_mapping || !hidden_cache_use_input || !hidden_cache_store_tot)) return APS_ERR_INVALID_ARG;
-  if ((n_rows || n_store) &&
-      (holder_stride < hidden_size || hidden_stride < hidden_size || slot_stride < hidden_size))
-    return APS_ERR_INVALID_ARG;
+  if ((n_rows || n_store) && (hidden_stride < hidden_size || slot_stride < hidden_size)) return APS_ERR_INVALID_ARG;
+  if (n_rows && holder && holder_stride < hidden_size) return APS_ERR_INVALID_ARG;
   if (n_kv) {
     if (!key || !value || !key_cache || !value_cache || !kv_cache_use_input || !new_token_slot || block_size <= 0)
       return APS_ERR_INVALID_ARG;
@@ -643,16 +643,19 @@ int aps_decode_step_cache_ops(void* holder, const void* hidden_states, void* pag
       return APS_ERR_INVALID_ARG;
   }
   const int64_t e = elem_size;
+  const int64_t n_map = n_rows;   // slot_mapping always has n_rows entries; without a holder no row is gathered
+  if (!holder) n_rows = 0;
   DecodeStepOp op{ResolvedGatherOp{(char*)holder, (const char*)hidden_states, (char*)paged_cache, holder_src,
                                    slot_mapping, hidden_cache_use_input, hidden_cache_store_tot, n_rows, n_store,
-                                   num_inputs, holder_stride * e, hidden_stride * e, slot_stride * e, num_slots},
+                                   num_inputs, holder_stride * e, hidden_stride * e, slot_stride * e, num_slots,
+                                   n_map},
                   (const char*)key, (const char*)value, (char*)key_cache, (char*)value_cache, kv_cache_use_input,
                   new_token_slot, n_kv, key_stride * e, value_stride * e, block_stride * e, hidden_size * e,
                   num_blocks, BlockSplit(block_size > 0 ? block_size : 1)};
   uint64_t bits = (uint64_t)(hidden_size * e);
   if (n_rows || n_store)
-    bits |= addr(holder) | addr(hidden_states) | addr(paged_cache) | (uint64_t)(holder_stride * e) |
-            (uint64_t)(hidden_stride * e) | (uint64_t)(slot_stride * e);
+    bits |= addr(hidden_states) | addr(paged_cache) | (uint64_t)(hidden_stride * e) | (uint64_t)(slot_stride * e);
+  if (n_rows) bits |= addr(holder) | (uint64_t)(holder_stride * e);
   if (n_kv)
     bits |= addr(key) | addr(value) | addr(key_cache) | addr(value_cache) | (uint64_t)(key_stride * e) |
             (uint64_t)(value_stride * e) | (uint64_t)(block_stride * e);

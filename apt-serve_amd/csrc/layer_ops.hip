@@ -41,17 +41,17 @@ __device__ __forceinline__ uint32_t to16(float v) {
   return BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
 }
 
-template <bool BF16>
+template <bool BF16, int VECS>
 __global__ __launch_bounds__(kLnThreads) void add_layer_norm_kernel(const AddLnArgs g) {
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
   const int nvec = g.width >> 3;  // 8 elements (16 bytes) per vector
   const char* x = g.x + row * g.x_stride_b;
   const char* r = g.residual ? g.residual + row * g.res_stride_b : nullptr;
-  float v[kLnVecs][8];
+  float v[VECS][8];
   float total = 0.f;
 #pragma unroll
-  for (int j = 0; j < kLnVecs; ++j) {
+  for (int j = 0; j < VECS; ++j) {
     const int i = threadIdx.x + j * kLnThreads;
     if (i < nvec) {
       const u32x4 a = *(const u32x4*)(x + (int64_t)i * 16);
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kLnThreads) void add_layer_norm_kernel(const AddLnA
   const float mean = block_sum(total, red) / (float)g.width;
   float sq = 0.f;
 #pragma unroll
-  for (int j = 0; j < kLnVecs; ++j) {
+  for (int j = 0; j < VECS; ++j) {
     if (threadIdx.x + j * kLnThreads < nvec) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(kLnThreads) void add_layer_norm_kernel(const AddLnA
   }
   const float rstd = rsqrtf(block_sum(sq, red) / (float)g.width + g.eps);
 #pragma unroll
-  for (int j = 0; j < kLnVecs; ++j) {
+  for (int j = 0; j < VECS; ++j) {
     const int i = threadIdx.x + j * kLnThreads;
     if (i < nvec) {
       const u32x4 w = *(const u32x4*)(g.gamma + (int64_t)i * 16);
@@ -129,7 +129,15 @@ extern "C" int aps_add_layer_norm(void* normed, void* sum, const void* x, const 
   AddLnArgs g{(char*)normed, (char*)sum, (const char*)x, (const char*)residual, (const char*)gamma,
               (const char*)beta, x_stride * 2, residual_stride * 2, normed_stride * 2, sum_stride * 2, (int)width, eps};
   const dim3 grid((unsigned)rows);
-  if (dtype == APS_BF16) APS_LAUNCH(add_layer_norm_kernel<true>, grid, dim3(kLnThreads), 0, (hipStream_t)stream, g);
-  else APS_LAUNCH(add_layer_norm_kernel<false>, grid, dim3(kLnThreads), 0, (hipStream_t)stream, g);
+  // rows of up to 3 * 256 * 8 = 6144 elements (every OPT up to 13B) keep 3 vectors per thread, wider ones 8
+  const bool narrow = width <= 3 * kLnThreads * 8;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == APS_BF16) {
+    if (narrow) APS_LAUNCH((add_layer_norm_kernel<true, 3>), grid, dim3(kLnThreads), 0, s, g);
+    else APS_LAUNCH((add_layer_norm_kernel<true, kLnVecs>), grid, dim3(kLnThreads), 0, s, g);
+  } else {
+    if (narrow) APS_LAUNCH((add_layer_norm_kernel<false, 3>), grid, dim3(kLnThreads), 0, s, g);
+    else APS_LAUNCH((add_layer_norm_kernel<false, kLnVecs>), grid, dim3(kLnThreads), 0, s, g);
+  }
   return launch_status();
 }

@@ -82,7 +82,11 @@ struct OutMap {
   const int64_t* map;
   int64_t limit0, limit1;  // rows (plain) or workspace slots; private slots
   int aligned16;           // every base and the pitch allow 128-bit stores
+  int relu;                // negative results are stored as zero (the activation between fc1 and fc2)
 };
+
+// max(v, 0) that keeps a NaN, as the element-wise activation on the rounded result would
+__device__ __forceinline__ float act(const OutMap& o, float v) { return (o.relu && v < 0.f) ? 0.f : v; }
 
 // Start of result row `row` for the column half `half`; nullptr when the row is skipped.
 __device__ __forceinline__ uint16_t* out_row(const OutMap& o, int64_t row, int half) {
@@ -115,6 +119,10 @@ struct GemmArgs {
   // partial tile to partial[z][m][n]; a second kernel adds the splits and the bias
   float* partial;
   int kt_per_split;
+  // weight_stream_kernel only: one zero-initialised counter per output tile.  With it the workgroup that
+  // stores a tile's last partial product adds the parts itself (and puts the counter back to zero) instead of
+  // leaving them to a second launch.
+  int* tile_counters;
   // tail split (large M): logical tiles from tail_from on are cut into tail_ways parts of tail_kt k-tiles each;
   // part p of tail tile i stores its fp32 result tile at tail_partial[(i * tail_ways + p)][256][256]
   float* tail_partial;
@@ -363,7 +371,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int i = 0; i < RT; ++i) {
 #pragma unroll
       for (int e = 0; e < 4; e += 2) {
-        const float v0 = acc[i][j][e] + bv, v1 = acc[i][j][e + 1] + bv;
+        const float v0 = act(g.out, acc[i][j][e] + bv), v1 = act(g.out, acc[i][j][e + 1] + bv);
         const uint32_t h0 = BF16 ? f32_to_bf16_bits(v0) : f32_to_f16_bits(v0);
         const uint32_t h1 = BF16 ? f32_to_bf16_bits(v1) : f32_to_f16_bits(v1);
         // even lanes keep row e and receive the neighbour's row-e value; odd lanes keep row e+1
@@ -503,6 +511,7 @@ __global__ __launch_bounds__(kSkWaves * 64) void skinny_nt_kernel(const GemmArgs
       const uint16_t bb = ((const uint16_t*)g.bias)[n + i];
       v += BF16 ? __uint_as_float((uint32_t)bb << 16) : (float)__builtin_bit_cast(_Float16, bb);
     }
+    v = act(g.out, v);
     h[i] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
   }
   if (g.out.aligned16) {  // 8-byte store
@@ -642,6 +651,7 @@ __global__ __launch_bounds__(kRsWaves * 64) void rowstream_nt_kernel(const GemmA
         const uint16_t bb = ((const uint16_t*)g.bias)[n];
         v += BF16 ? __uint_as_float((uint32_t)bb << 16) : (float)__builtin_bit_cast(_Float16, bb);
       }
+      v = act(g.out, v);
       dst[n - (half ? g.out.n_split : 0)] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
     }
 }
@@ -695,9 +705,77 @@ __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArg
                                      g.lda_b, (int)min((int64_t)(16 * NHT), g.m - m0), klen, lds, acc);
   // lane (g4, c) holds activation rows m0 + 16*ht + 4*g4 + i and weight row n0 + 16*wave + c
   const int64_t n = n0 + wave * 16 + c;
-  if (n >= g.n) return;
+  const bool own = g.partial && g.tile_counters;   // the last workgroup of a tile adds the parts
+  if (n >= g.n && !own) return;
+  if (g.partial && n < g.n) {
+#pragma unroll
+    for (int ht = 0; ht < NHT; ++ht)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int64_t row = m0 + 16 * ht + 4 * g4 + i;
+        if (row >= g.m) continue;
+        float* dst = g.partial + ((int64_t)blockIdx.y * g.m + row) * g.n + n;
+        // read by another workgroup of this launch: stored through to device-coherent memory
+        if (own) __hip_atomic_store(dst, acc[ht][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else *dst = acc[ht][i];
+      }
+  }
+  if (g.partial) {
+    if (!own) return;
+    // The parts cross between workgroups through device-coherent stores and loads (they go past the L2 of the
+    // compute die, which is not coherent with the other dies' inside a launch) and a counter per tile: a
+    // workgroup waits until its own stores are acknowledged, counts itself in, and the one that finds every
+    // other workgroup of the tile counted adds the parts.  No workgroup waits for another, whichever arrives
+    // last does the sum in part order, so the result does not depend on which; and no device-scope fence is
+    // used (a release writes the whole L2 back: measured 8-10 us per launch, more than the second launch cost).
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    int* flag = (int*)lds;
+    if (tid == 0) {
+      int* counter = g.tile_counters + blockIdx.z * gridDim.x + blockIdx.x;
+      const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int last = before == (int)gridDim.y - 1;
+      // nobody else touches the counter any more in this launch; zero for the next one
+      if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *flag = last;
+    }
+    __syncthreads();
+    if (!*flag || n >= g.n) return;
+    // parts 0, 1, 2, ... added in that order (what splitk_reduce_kernel does), eight loads per value in flight
+    const int parts = (int)gridDim.y;
+    const int64_t plane = g.m * g.n;
+    const float* pp[NHT][4];
+#pragma unroll
+    for (int ht = 0; ht < NHT; ++ht)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int64_t row = min(m0 + 16 * ht + 4 * g4 + i, g.m - 1);   // rows past the end: a valid address, not stored
+        pp[ht][i] = g.partial + row * g.n + n;
+        acc[ht][i] = __hip_atomic_load(pp[ht][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    for (int z0 = 1; z0 < parts; z0 += 8) {
+      float t[NHT][4][8];
+#pragma unroll
+      for (int ht = 0; ht < NHT; ++ht)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int zb = 0; zb < 8; ++zb)
+            t[ht][i][zb] = __hip_atomic_load(pp[ht][i] + (int64_t)min(z0 + zb, parts - 1) * plane, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int zb = 0; zb < 8; ++zb)
+        if (z0 + zb < parts) {
+#pragma unroll
+          for (int ht = 0; ht < NHT; ++ht)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[ht][i] += t[ht][i][zb];
+        }
+    }
+  }
   float b = 0.f;
-  if (!g.partial && g.bias) b = load_16bit_as_f32<BF16>(g.bias, n);
+  if (g.bias) b = load_16bit_as_f32<BF16>(g.bias, n);
   const int half = (g.out.n_split && n >= g.out.n_split) ? 1 : 0;
 #pragma unroll
   for (int ht = 0; ht < NHT; ++ht)
@@ -705,12 +783,10 @@ __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArg
     for (int i = 0; i < 4; ++i) {
       const int64_t row = m0 + 16 * ht + 4 * g4 + i;
       if (row >= g.m) continue;
-      if (g.partial) {
-        g.partial[((int64_t)blockIdx.y * g.m + row) * g.n + n] = acc[ht][i];
-      } else {
+      {
         uint16_t* dst = out_row(g.out, row, half);
         if (!dst) continue;
-        const float v = acc[ht][i] + b;
+        const float v = act(g.out, acc[ht][i] + b);
         dst[n - (half ? g.out.n_split : 0)] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
       }
     }
@@ -787,6 +863,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     auto cv = [](uint16_t v) { return BF16 ? __uint_as_float((uint32_t)v << 16) : (float)__builtin_bit_cast(_Float16, v); };
     s.x += cv(b[0]); s.y += cv(b[1]); s.z += cv(b[2]); s.w += cv(b[3]);
   }
+  s.x = act(out, s.x); s.y = act(out, s.y); s.z = act(out, s.z); s.w = act(out, s.w);
   const int half = (out.n_split && col >= out.n_split) ? 1 : 0;
   uint16_t* o = out_row(out, row, half);
   if (!o) return;
@@ -816,6 +893,7 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const GemmArgs g) {
     s.x += load_16bit_as_f32<BF16>(g.bias, col); s.y += load_16bit_as_f32<BF16>(g.bias, col + 1);
     s.z += load_16bit_as_f32<BF16>(g.bias, col + 2); s.w += load_16bit_as_f32<BF16>(g.bias, col + 3);
   }
+  s.x = act(g.out, s.x); s.y = act(g.out, s.y); s.z = act(g.out, s.z); s.w = act(g.out, s.w);
   const int half = (g.out.n_split && col >= g.out.n_split) ? 1 : 0;
   uint16_t* o = out_row(g.out, row, half);
   if (!o) return;
@@ -908,7 +986,8 @@ struct GatherSrc {
 
 static int launch_gemm(const void* x, const void* weight, const void* bias, const OutMap& om, int64_t m, int64_t n,
                        int64_t k, int64_t x_stride, int64_t w_stride, int dtype, void* workspace,
-                       int64_t workspace_bytes, aps_stream_t stream, const GatherSrc* gs = nullptr) {
+                       int64_t workspace_bytes, aps_stream_t stream, const GatherSrc* gs = nullptr,
+                       int32_t* tile_counters = nullptr) {
   if (dtype != APS_F16 && dtype != APS_BF16) return APS_ERR_UNSUPPORTED;
   if (n % BN != 0 || k % BK != 0) return APS_ERR_UNSUPPORTED;
   if (x_stride < k || w_stride < k) return APS_ERR_INVALID_ARG;
@@ -942,9 +1021,10 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
     const int parts = weight_stream_parts(m, n, k, &k_per_part);
     if (parts == 1 || (workspace && workspace_bytes >= (int64_t)parts * m * n * 4 && !(addr(workspace) & 15))) {
       g.partial = parts > 1 ? (float*)workspace : nullptr;
+      g.tile_counters = parts > 1 ? (int*)tile_counters : nullptr;   // (at most kNumCus tiles are split)
       int st = dtype == APS_BF16 ? launch_weight_stream<true>(g, parts, k_per_part, s)
                                  : launch_weight_stream<false>(g, parts, k_per_part, s);
-      if (st != APS_OK || parts == 1) return st;
+      if (st != APS_OK || parts == 1 || g.tile_counters) return st;
       const int64_t quads = m * n / 4;
       const dim3 rgrid((unsigned)((quads + 255) / 256));
       if (dtype == APS_BF16)
@@ -1071,8 +1151,9 @@ extern "C" {
 
 int aps_linear_nt(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n, int64_t k,
                   int64_t x_stride, int64_t w_stride, int64_t out_stride, const int64_t* out_row_map,
-                  int64_t out_rows, int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream) {
-  if (m < 0 || n <= 0 || k <= 0) return APS_ERR_INVALID_ARG;
+                  int64_t out_rows, int dtype, int flags, void* workspace, int64_t workspace_bytes,
+                  int32_t* tile_counters, aps_stream_t stream) {
+  if (m < 0 || n <= 0 || k <= 0 || (flags & ~APS_LINEAR_RELU)) return APS_ERR_INVALID_ARG;
   if (m == 0) return APS_OK;
   if (!x || !weight || !out) return APS_ERR_INVALID_ARG;
   if (out_stride < n) return APS_ERR_INVALID_ARG;
@@ -1081,7 +1162,10 @@ int aps_linear_nt(const void* x, const void* weight, const void* bias, void* out
   OutMap om{};
   om.base[0] = (char*)out; om.ld = out_stride; om.n_split = 0;
   om.map = out_row_map; om.limit0 = out_rows; om.aligned16 = align == 16;
-  return launch_gemm(x, weight, bias, om, m, n, k, x_stride, w_stride, dtype, workspace, workspace_bytes, stream);
+  om.relu = (flags & APS_LINEAR_RELU) ? 1 : 0;
+  if (addr(tile_counters) & 3) return APS_ERR_INVALID_ARG;
+  return launch_gemm(x, weight, bias, om, m, n, k, x_stride, w_stride, dtype, workspace, workspace_bytes, stream,
+                     nullptr, tile_counters);
 }
 
 int aps_kv_reproject_to_cache(const void* x, const void* w_kv, const void* b_kv, void* ws_k_cache, void* ws_v_cache,

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define APS_ABI_VERSION 8
+#define APS_ABI_VERSION 9
 
 typedef void* aps_stream_t; /* a hipStream_t; NULL = the null stream */
 
@@ -49,6 +49,9 @@ enum aps_dtype {
 /* flags of aps_mixed_kv_to_cache */
 #define APS_MIXED_LITERAL_MODULO 1u /* reproduce `blk % (2*nkv)` of mixed_cache.cu:88 */
 #define APS_MIXED_SKIP_MIRROR 2u    /* do not write range B (the shared mirror) */
+
+/* aps_linear_nt flags */
+#define APS_LINEAR_RELU 1 /* store max(result, 0): fc1 with its activation */
 
 int aps_abi_version(void);
 const char* aps_status_string(int status);
@@ -138,7 +141,10 @@ int aps_gather_hidden_rows(void* holder, const void* hidden_states,
  * width of a hidden row (hidden_size = heads * head_size) and the dtype of the
  * hidden rows.  Bit-identical to aps_reshape_and_cache_flash (token_idx =
  * kv_cache_use_input) followed by aps_gather_hidden_rows; the destinations of
- * the three kinds of rows are disjoint, so no order between them is needed. */
+ * the three kinds of rows are disjoint, so no order between them is needed.
+ * holder may be NULL (then holder_src too): no holder is assembled, n_rows is
+ * only the length of slot_mapping, and the launch is the two kinds of stores —
+ * what a flow that attends on the cached hidden rows themselves needs. */
 int aps_decode_step_cache_ops(
     void* holder, const void* hidden_states, void* paged_cache,
     const int64_t* holder_src, int64_t n_rows, const int64_t* slot_mapping,
@@ -435,15 +441,26 @@ int aps_build_prefill_metadata(
  * that a second kernel adds (in fp32, then bias, then one rounding); without it
  * a single-launch kernel runs.  A workspace that is passed but too small or
  * misaligned is an error (APS_ERR_WORKSPACE), never a silent fallback.
+ * flags: APS_LINEAR_RELU stores max(result, 0) — the ReLU between fc1 and fc2
+ * of the decoder's MLP (model_executor/models/aptserve_opt.py:205-207:
+ * `fc1`, `activation_fn`, `fc2`) without an element-wise launch of its own; the
+ * rounded values are those of "linear, then relu" on 16-bit tensors.
+ * tile_counters (nullable): APS_LINEAR_TILE_COUNTERS int32 that are zero on
+ * entry and zero again when the call's work is done, owned by the caller (one
+ * array per stream that calls concurrently).  With them the K split of a decode
+ * step's few rows (3..48) needs no second launch: the workgroup that stores the
+ * last partial product of an output tile adds the tile's parts itself (in part
+ * order: the result is bit for bit the two-launch one).
  * ------------------------------------------------------------------------ */
+#define APS_LINEAR_TILE_COUNTERS 256
 int aps_linear_nt_splits(int64_t m, int64_t n, int64_t k);
 int64_t aps_linear_nt_workspace_bytes(int64_t m, int64_t n, int64_t k);
 int aps_linear_nt(const void* x, const void* weight, const void* bias,
                   void* out, int64_t m, int64_t n, int64_t k, int64_t x_stride,
                   int64_t w_stride, int64_t out_stride,
                   const int64_t* out_row_map, int64_t out_rows, int dtype,
-                  void* workspace, int64_t workspace_bytes,
-                  aps_stream_t stream);
+                  int flags, void* workspace, int64_t workspace_bytes,
+                  int32_t* tile_counters, aps_stream_t stream);
 
 /* K/V re-projection with the cache write fused into the epilogue: one pass that
  * replaces the kv_only projection (model_executor/models/aptserve_opt.py:123-124),

@@ -313,6 +313,37 @@ def test_decode_step_cache_ops_one_launch(dev, seed, frac, H, D, dtype):
     assert bits_equal(g, ref)
 
 
+def test_decode_step_cache_ops_without_a_holder_stores_only(dev):
+    """No holder (the flow that attends on the cached hidden rows assembles none): the launch is the hidden-row
+    stores and the K/V-row writes, the hidden rows into one cache and the K/V rows into another."""
+    from aptserve_hip import metadata
+    N, BS, H, D = 64, 16, 4, 32
+    b = workloads.small_decode_batch(3, 9, 90, 0.5, N)
+    md, gmd = oracle_metadata(b), metadata.build_from_batch(b, dev)
+    B, Hd = len(b.seq_lens), H * D
+    hs, kv = randn((B, Hd), 3), randn((B, 2 * Hd), 10)
+    k, v = kv.chunk(2, -1)
+    sm = t64(md["slot_mapping"])
+    seq_idx = torch.tensor([i for i, h in enumerate(b.use_hidden) if not h], dtype=torch.int64)
+    for separate in (False, True):
+        hidden_cache, kv_cache = sentinel_cache((2, N, BS, H, D)), sentinel_cache((2, N, BS, H, D), seed=9)
+        ref_h, ref_kv = hidden_cache.clone(), (kv_cache.clone() if separate else None)
+        if not separate:
+            ref_kv = ref_h
+        O.hidden_to_cache(hs, ref_h, sm, t64(md["hidden_cache_use_input"]), t64(md["hidden_cache_store_tot"]))
+        O.reshape_and_cache_flash(k[seq_idx].view(-1, H, D), v[seq_idx].view(-1, H, D), ref_kv[0], ref_kv[1],
+                                  sm[t64(md["kv_cache_use_tot"])], "auto")
+        gh, gkv = hidden_cache.to(dev), kv_cache.to(dev)
+        dk, dv = kv.to(dev).chunk(2, -1)
+        ops.decode_step_cache_ops(None, hs.to(dev), gh, None, gmd.slot_mapping, gmd.hidden_cache_use_input,
+                                  gmd.hidden_cache_store_tot, dk, dv, gmd.kv_cache_use_input, gmd.new_token_slot,
+                                  kv_cache=gkv if separate else None)
+        assert bits_equal(gh, ref_h)
+        if separate:
+            assert bits_equal(gkv, ref_kv)
+    assert md["num_hidden_cache_tokens"] > 0 and len(seq_idx) > 0
+
+
 def test_decode_step_cache_ops_skips_bad_rows(dev):
     """Padding slots, out-of-range sequence positions and slots past the cache are skipped, not written."""
     H, D, N, BS = 1, 8, 4, 16

@@ -85,10 +85,48 @@ def test_few_rows_weight_stream_strides_row_map_and_workspace(dev):
     small = torch.empty(1024, dtype=torch.uint8, device=dev)
     out = torch.empty(M, N, dtype=torch.float16, device=dev)
     st = ops._lib.load().aps_linear_nt(xd.data_ptr(), wd.data_ptr(), bd.data_ptr(), out.data_ptr(), M, N, K,
-                                       xd.stride(0), wd.stride(0), out.stride(0), None, M, 0, small.data_ptr(),
-                                       small.numel(), None)
+                                       xd.stride(0), wd.stride(0), out.stride(0), None, M, 0, 0, small.data_ptr(),
+                                       small.numel(), None, None)
     torch.cuda.synchronize()
     assert st == -3
+
+
+@pytest.mark.parametrize("M", [1, 2, 5, 16, 30, 48, 49, 100, 300, 3328])   # every kernel family and the tail split
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_relu_epilogue_equals_relu_of_the_rounded_product(dev, M, dtype):
+    """fc1 with its activation (aptserve_opt.py:205-206): negative results are stored as zero, everything else
+    bit for bit as without the flag — in the epilogue of every kernel of the family and in the kernels that add
+    K-split partial products."""
+    N, K = (512, 192) if M < 1000 else (5120, 1024)
+    x, w, b = randn((M, K), M, dtype).to(dev), (randn((N, K), 1) * 0.05).to(dtype).to(dev), randn((N,), 3, dtype).to(dev)
+    for split_k in (True, False):
+        plain = ops.linear_nt(x, w, b, split_k=split_k)
+        act = ops.linear_nt(x, w, b, split_k=split_k, relu=True)
+        assert (plain < 0).any() and torch.equal(act, torch.relu(plain))
+
+
+@pytest.mark.parametrize("M,N,K", [(3, 768, 768), (5, 5120, 5120), (5, 5120, 20480), (17, 1536, 768), (48, 5120, 5120),
+                                   (33, 15360, 5120), (7, 256, 2048)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_k_split_summed_inside_the_launch_equals_the_two_launch_sum(dev, M, N, K, dtype):
+    """The K split of a decode step's few rows with tile counters (the workgroup that stores a tile's last
+    partial product adds the parts, in part order) against the same split summed by the second kernel: the same
+    bits, the counters zero again afterwards, call after call on the same counters."""
+    lib = ops._lib.load()
+    x, w, b = randn((M, K), M, dtype).to(dev), (randn((N, K), 1) * 0.05).to(dtype).to(dev), randn((N,), 3, dtype).to(dev)
+    assert lib.aps_linear_nt_splits(M, N, K) > 1
+    ws = torch.empty(lib.aps_linear_nt_workspace_bytes(M, N, K), dtype=torch.uint8, device=dev)
+    code = 0 if dtype == torch.float16 else 1
+    two = torch.empty(M, N, dtype=dtype, device=dev)
+    st = lib.aps_linear_nt(x.data_ptr(), w.data_ptr(), b.data_ptr(), two.data_ptr(), M, N, K, K, K, N, None, M, code, 0,
+                           ws.data_ptr(), ws.numel(), None, None)
+    assert st == 0
+    counters = ops._tile_counters(dev)
+    for rep in range(30):          # the parts cross between workgroups inside the launch: every repetition must agree
+        relu = rep % 3 == 1
+        one = ops.linear_nt(x, w, b, relu=relu)
+        assert torch.equal(one, torch.relu(two) if relu else two), rep
+    assert int(counters.abs().sum()) == 0
 
 
 def test_identity_and_one_hot_weights_are_exact(dev):
