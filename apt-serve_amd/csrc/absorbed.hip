@@ -23,6 +23,15 @@
 #include "mfma_common.h"
 #include "row_stream_core.h"
 
+// the per-head value projection lives with the other weight-streaming kernels
+__attribute__((visibility("hidden"))) int aps_internal_headwise_linear(
+    const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n, int64_t k, int64_t x_stride,
+    int64_t x_head_stride, int head_rows, int64_t w_stride, int64_t out_stride, const int64_t* out_row_map,
+    int64_t out_rows, int dtype, void* workspace, int64_t workspace_bytes, int32_t* tile_counters, hipStream_t stream);
+// bytes of fp32 partial products that call uses for m rows (0: it runs a kernel that needs none)
+__attribute__((visibility("hidden"))) int64_t aps_internal_headwise_workspace_bytes(int64_t m, int64_t n, int64_t k,
+                                                                                   int head_rows);
+
 namespace aps {
 namespace {
 
@@ -187,7 +196,8 @@ constexpr int kMaxOrderedSeqs = 4096;  // lengths are ranked out of LDS, quadrat
 __device__ __forceinline__ void plan_ragged_batch(const int64_t* __restrict__ row_start, int n_seqs, int tile_tokens,
                                                   int32_t* __restrict__ tile_start, int32_t* __restrict__ order,
                                                   u32x4* __restrict__ zero_row, int zero_vecs) {
-  // the row of zeros that tokens without a cached row read in the weighted sum
+  // the row of zeros that tokens without a cached row read in the weighted sum; behind it (same region of the
+  // workspace, counted in zero_vecs) the arrival counters of the value projection's K split
   for (int i = threadIdx.x; i < zero_vecs; i += 256) zero_row[i] = u32x4{0u, 0u, 0u, 0u};
   __shared__ int32_t part[256];
   __shared__ int32_t carry;
@@ -834,7 +844,9 @@ struct Plan {
   int score_parts;   // parts of K in the scores kernel (partial scores, made whole by score_parts_sum_kernel)
   int64_t score_k_per_part;
   int k_per_part;
-  int64_t off_qt, off_s, off_ctx, off_tiles, off_order, off_zero, off_partial, off_ml, total;
+  int64_t off_qt, off_s, off_ctx, off_tiles, off_order, off_zero, off_partial, off_ml, off_vp, total;
+  int64_t zero_bytes;      // the row of zeros and, behind it, the arrival counters: cleared by the planning workgroup
+  int64_t off_vp_counters;
 };
 
 Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
@@ -879,10 +891,14 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   p.off_tiles = o; o += align_up((n_seqs + 1) * 4, 256);
   p.off_order = o; o += align_up(n_seqs * 4, 256);
   p.off_zero = o; o += align_up(hidden * 2, 256);
+  p.off_vp_counters = o; o += APS_LINEAR_TILE_COUNTERS * 4;
+  p.zero_bytes = o - p.off_zero;
   p.off_partial = o;
   if (p.kparts > 1) o += align_up((int64_t)p.kparts * n_seqs * heads * hidden * 4, 256);
   p.off_ml = o;
   if (p.kparts > 1) o += align_up((int64_t)p.kparts * n_seqs * heads * 2 * 4, 256);
+  p.off_vp = o;   // fp32 partial products of the value projection's K split (few sequences)
+  if (n_seqs <= 16) o += align_up(aps_internal_headwise_workspace_bytes(n_seqs, hidden, hidden, (int)(hidden / heads)), 256);
   p.total = o;
   return p;
 }
@@ -891,12 +907,6 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
 }  // namespace aps
 
 using namespace aps;
-
-// the per-head value projection lives with the other weight-streaming kernels
-__attribute__((visibility("hidden"))) int aps_internal_headwise_linear(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n,
-                                 int64_t k, int64_t x_stride, int64_t x_head_stride, int head_rows, int64_t w_stride,
-                                 int64_t out_stride, const int64_t* out_row_map, int64_t out_rows, int dtype,
-                                 hipStream_t stream);
 
 extern "C" {
 
@@ -949,7 +959,7 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     g.qt = qt;
     g.alpha = softmax_scale * 1.4426950408889634f;
     g.row_start = seq_start; g.tile_tokens = kScTokens; g.tile_start = tiles; g.order = order;
-    g.zero_row = (u32x4*)(ws + p.off_zero); g.zero_vecs = (int)(hidden * 2 / 16);
+    g.zero_row = (u32x4*)(ws + p.off_zero); g.zero_vecs = (int)(p.zero_bytes / 16);
     const dim3 grid((unsigned)((hidden + 511) / 512), (unsigned)num_heads + 1);
 #define APS_LAUNCH_QI(B)                                                                     \
   switch (head_size / 32) {                                                                  \
@@ -976,7 +986,7 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     int st = bf16 ? launch_nn<true>(g, s) : launch_nn<false>(g, s);
     if (st != APS_OK) return st;
     APS_LAUNCH(seq_plan_kernel, dim3(1), dim3(256), 0, s, seq_start, (int)n_seqs, kScTokens, tiles, order,
-               (u32x4*)(ws + p.off_zero), (int)(hidden * 2 / 16));
+               (u32x4*)(ws + p.off_zero), (int)(p.zero_bytes / 16));
     st = launch_status();
     if (st != APS_OK) return st;
   }
@@ -1068,7 +1078,8 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
   // 5. out[seq_rows[s]][h*D + d] = <W_v[h*D + d], ctx[s][h]> + b_v
   if (n_seqs <= 16)  // few sequences: the weight-streaming kernels read W_v once
     return aps_internal_headwise_linear(ctx, w_v, b_v, out, n_seqs, hidden, hidden, (int64_t)num_heads * hidden,
-                                        hidden, head_size, w_stride, out_stride, seq_rows, out_rows, dtype, s);
+                                        hidden, head_size, w_stride, out_stride, seq_rows, out_rows, dtype,
+                                        ws + p.off_vp, p.total - p.off_vp, (int32_t*)(ws + p.off_vp_counters), s);
   {
     HeadProjArgs g{};
     g.w = (const char*)w_v; g.w_stride_b = w_stride * 2; g.head_rows = head_size; g.heads = num_heads;

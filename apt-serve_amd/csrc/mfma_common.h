@@ -56,6 +56,38 @@ __device__ __forceinline__ float4v mfma16(const u32x4& a, const u32x4& b, const 
                                                   0);
 }
 
+// ---- results handed from workgroup to workgroup inside one launch
+// The partial results of a split reduction cross between workgroups through device-coherent stores and loads
+// (they go past the L2 of the compute die, which is not coherent with the other dies' inside a launch) and one
+// counter per output tile: a workgroup waits until its own stores are acknowledged, counts itself in, and the
+// one that finds every other workgroup of the tile counted does the sum.  No workgroup waits for another;
+// whichever arrives last adds the parts in part order, so the result does not depend on which.  No device-scope
+// fence is used: a release writes the whole L2 back (measured: 8-10 us per launch of 240 workgroups, more than a
+// second launch for the sum costs).
+__device__ __forceinline__ void coherent_store(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float coherent_load(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// True in every thread of the workgroup that arrives last of `count` at `counter` (zero before the first arrival;
+// the last arrival puts it back to zero).  Called by all threads of the workgroup after their coherent_store()s;
+// `flag` is a word of LDS that no wavefront still uses.
+__device__ __forceinline__ bool last_arrival(int* counter, int count, int* flag) {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);   // every store of this wavefront acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int last = before == count - 1;
+    // nobody else touches the counter any more in this launch: zero for the next one
+    if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *flag = last;
+  }
+  __syncthreads();
+  return *flag != 0;
+}
+
 template <bool BF16>
 __device__ __forceinline__ float load_16bit_as_f32(const void* p, int64_t i) {
   const uint16_t v = ((const uint16_t*)p)[i];

@@ -700,8 +700,11 @@ __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArg
     return g.w + (n < g.n ? n : 0) * g.ldw_b + (lane & 7) * 16 + k0 * 2;
   };
   float4v acc[NHT];
+  // (head-wise x: the 128 weight rows of a workgroup lie inside one head, whose x is the image)
+  const int64_t head_off = g.head_rows ? (n0 / g.head_rows) * g.x_head_stride_b : 0;
   stream_rows_times_image<BF16, NHT>(weight_row(n0 + wave * 16 + (lane >> 3)),
-                                     weight_row(n0 + wave * 16 + 8 + (lane >> 3)), g.a + m0 * g.lda_b + k0 * 2,
+                                     weight_row(n0 + wave * 16 + 8 + (lane >> 3)),
+                                     g.a + head_off + m0 * g.lda_b + k0 * 2,
                                      g.lda_b, (int)min((int64_t)(16 * NHT), g.m - m0), klen, lds, acc);
   // lane (g4, c) holds activation rows m0 + 16*ht + 4*g4 + i and weight row n0 + 16*wave + c
   const int64_t n = n0 + wave * 16 + c;
@@ -715,33 +718,14 @@ __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArg
         const int64_t row = m0 + 16 * ht + 4 * g4 + i;
         if (row >= g.m) continue;
         float* dst = g.partial + ((int64_t)blockIdx.y * g.m + row) * g.n + n;
-        // read by another workgroup of this launch: stored through to device-coherent memory
-        if (own) __hip_atomic_store(dst, acc[ht][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (own) coherent_store(dst, acc[ht][i]);   // read by another workgroup of this launch
         else *dst = acc[ht][i];
       }
   }
   if (g.partial) {
     if (!own) return;
-    // The parts cross between workgroups through device-coherent stores and loads (they go past the L2 of the
-    // compute die, which is not coherent with the other dies' inside a launch) and a counter per tile: a
-    // workgroup waits until its own stores are acknowledged, counts itself in, and the one that finds every
-    // other workgroup of the tile counted adds the parts.  No workgroup waits for another, whichever arrives
-    // last does the sum in part order, so the result does not depend on which; and no device-scope fence is
-    // used (a release writes the whole L2 back: measured 8-10 us per launch, more than the second launch cost).
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    int* flag = (int*)lds;
-    if (tid == 0) {
-      int* counter = g.tile_counters + blockIdx.z * gridDim.x + blockIdx.x;
-      const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const int last = before == (int)gridDim.y - 1;
-      // nobody else touches the counter any more in this launch; zero for the next one
-      if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      *flag = last;
-    }
-    __syncthreads();
-    if (!*flag || n >= g.n) return;
+    if (!last_arrival(g.tile_counters + blockIdx.z * gridDim.x + blockIdx.x, (int)gridDim.y, (int*)lds) || n >= g.n)
+      return;
     // parts 0, 1, 2, ... added in that order (what splitk_reduce_kernel does), eight loads per value in flight
     const int parts = (int)gridDim.y;
     const int64_t plane = g.m * g.n;
@@ -752,7 +736,7 @@ __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArg
       for (int i = 0; i < 4; ++i) {
         const int64_t row = min(m0 + 16 * ht + 4 * g4 + i, g.m - 1);   // rows past the end: a valid address, not stored
         pp[ht][i] = g.partial + row * g.n + n;
-        acc[ht][i] = __hip_atomic_load(pp[ht][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        acc[ht][i] = coherent_load(pp[ht][i]);
       }
     for (int z0 = 1; z0 < parts; z0 += 8) {
       float t[NHT][4][8];
@@ -762,8 +746,7 @@ __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArg
         for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int zb = 0; zb < 8; ++zb)
-            t[ht][i][zb] = __hip_atomic_load(pp[ht][i] + (int64_t)min(z0 + zb, parts - 1) * plane, __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT);
+            t[ht][i][zb] = coherent_load(pp[ht][i] + (int64_t)min(z0 + zb, parts - 1) * plane);
 #pragma unroll
       for (int zb = 0; zb < 8; ++zb)
         if (z0 + zb < parts) {
@@ -1117,13 +1100,21 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
 
 }  // extern "C"
 
+__attribute__((visibility("hidden"))) int64_t aps_internal_headwise_workspace_bytes(int64_t m, int64_t n, int64_t k,
+                                                                                   int head_rows) {
+  if (m < 3 || m > kWsMaxRows || head_rows <= 0 || head_rows % kScTokens != 0 || n % kScTokens != 0 || k % BK != 0)
+    return 0;
+  const int parts = weight_stream_parts(m, n, k, nullptr);
+  return parts > 1 ? (int64_t)parts * m * n * 4 : 16;   // (a nonzero size says "this shape is covered")
+}
+
 // out[map[m]][n] = <weight[n], x[m] + (n / head_rows) * x_head_stride> + bias[n]: the value projection of the
 // absorbed attention, where the rows of head h multiply that head's context vector.  Any m: at most 8 rows
 // stream the weights through the dot kernel, more go through the MFMA kernel in tiles of 16 rows.
 __attribute__((visibility("hidden"))) int aps_internal_headwise_linear(const void* x, const void* weight, const void* bias, void* out, int64_t m, int64_t n,
                                  int64_t k, int64_t x_stride, int64_t x_head_stride, int head_rows, int64_t w_stride,
                                  int64_t out_stride, const int64_t* out_row_map, int64_t out_rows, int dtype,
-                                 hipStream_t s) {
+                                 void* workspace, int64_t workspace_bytes, int32_t* tile_counters, hipStream_t s) {
   if (m <= 0) return APS_OK;
   if (n % 16 != 0 || k % 64 != 0 || head_rows % 16 != 0) return APS_ERR_UNSUPPORTED;
   if (x_stride * 2 * 16 >= ((int64_t)1 << 31) || w_stride * 2 * 16 >= ((int64_t)1 << 31)) return APS_ERR_UNSUPPORTED;
@@ -1135,6 +1126,19 @@ __attribute__((visibility("hidden"))) int aps_internal_headwise_linear(const voi
   g.out.map = out_row_map; g.out.limit0 = out_rows;
   g.out.aligned16 = common_vec_bytes({addr(out), (uint64_t)out_stride * 2}) == 16;
   g.x_head_stride_b = x_head_stride * 2; g.head_rows = head_rows;
+  // 3..48 rows and heads of whole 128-row tiles: the weight rows through the streaming core, K split over
+  // enough workgroups to fill the chip, the parts added by the last workgroup of each tile
+  const int64_t need = aps_internal_headwise_workspace_bytes(m, n, k, head_rows);
+  if (need > 0 && workspace && tile_counters && workspace_bytes >= need && !(addr(workspace) & 15) &&
+      common_vec_bytes({addr(x), addr(weight), (uint64_t)x_stride * 2, (uint64_t)x_head_stride * 2,
+                        (uint64_t)w_stride * 2}) == 16) {
+    int64_t k_per_part = 0;
+    const int parts = weight_stream_parts(m, n, k, &k_per_part);
+    g.partial = parts > 1 ? (float*)workspace : nullptr;
+    g.tile_counters = parts > 1 ? (int*)tile_counters : nullptr;
+    return dtype == APS_BF16 ? launch_weight_stream<true>(g, parts, k_per_part, s)
+                             : launch_weight_stream<false>(g, parts, k_per_part, s);
+  }
   if (m <= 8 && n % (kRsWaves * kRsRows) == 0)
     return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
   const int pairs = (int)((k / 32 + 1) / 2);
