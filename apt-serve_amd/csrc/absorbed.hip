@@ -793,6 +793,160 @@ __global__ __launch_bounds__(kWsThreads) __attribute__((amdgpu_waves_per_eu(APS_
     }
 }
 
+// ------------------------------------------------------------------ few cached rows: one chunk per workgroup
+// The same sum for a batch with few cached rows in all (a serving step's handful of sequences).  There the pass
+// above is not a stream but a chain of memory latencies - slots, scores, rows, chunk after chunk, with a handful
+// of workgroups - and lasts 17-20 us for 6 MB.  Here a workgroup owns ONE chunk of kWsChunk tokens of one sequence
+// (and kWsWaves * 128 columns), requests everything it needs at once - its scores and, behind the slots, all rows
+// of the chunk - does the chunk's softmax while the rows are on their way, multiplies, and leaves unnormalised
+// sums with the chunk's (max, sum) for wsum_combine_kernel: two memory round trips deep whatever the lengths.
+// The price is the fp32 sums of every chunk (heads x hidden values: about as many bytes as the chunk's rows),
+// which is why only small batches come here.
+template <bool BF16, int MT>
+__global__ __launch_bounds__(kWsThreads) void hidden_wsum_chunk_kernel(const WsumArgs g) {
+  constexpr int NJ = 16 * MT / kWsHeadsPerPass;
+  __shared__ __attribute__((aligned(16))) char p_lds[16 * MT * kWsPStride];
+  __shared__ __attribute__((aligned(16))) float fin_s[2][16 * MT];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int g4 = lane >> 4, c = lane & 15;
+  const int z = blockIdx.y / g.m_tiles;
+  const int m0 = (blockIdx.y % g.m_tiles) * (16 * MT);
+  const int64_t rs = g.row_start[z];
+  const int K = (int)min(g.row_start[z + 1] - rs, g.s_row_stride);
+  const int kbeg = blockIdx.z * kWsChunk;
+  const int n_tok = min(K - kbeg, kWsChunk);
+  const float kNegInf = -INFINITY;
+  if (n_tok <= 0 && g.partial) {  // a chunk past the end of its sequence: the combining kernel skips it
+    if (blockIdx.x == 0 && tid < 16 * MT && m0 + tid < g.heads) {
+      float* ml = g.partial_ml + (((int64_t)blockIdx.z * g.n_seqs + z) * g.heads + m0 + tid) * 2;
+      ml[0] = kNegInf;
+      ml[1] = 0.f;
+    }
+    return;
+  }
+  // ---- requests: the chunk's scores (thread (hl, tq): heads hl + HP*j, tokens 4*tq .. 4*tq+3) ...
+  const int hl = tid >> 5, tq = tid & 31;
+  const bool quad_ok = tq < kWsChunk / 4 && 4 * tq < n_tok;
+  float4v sv[NJ];
+  {
+    const char* s_base = (const char*)(g.s + (int64_t)z * g.s_batch_stride);
+    const int ts = quad_ok ? kbeg + 4 * tq : 0;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int head = m0 + hl + kWsHeadsPerPass * j;
+      sv[j] = *(const float4v*)(s_base + ((int64_t)(head < g.heads ? head : 0) * g.s_row_stride + ts) * 4);
+    }
+  }
+  // ... and the rows: lane (g4, c) reads tokens 32*st + 8*g4 + i, columns col0 .. col0+7 (a token past the chunk's
+  // end or without a cached row reads the row of zeros, a column past the row column 0)
+  const int64_t col0 = (int64_t)blockIdx.x * (kWsWaves * 128) + wave * 128 + 8 * c;
+  const bool col_ok = col0 < g.n;
+  const char* b_col = g.cache + (col_ok ? col0 : 0) * 2;
+  const char* z_col = g.zero_row + (col_ok ? col0 : 0) * 2;
+  int64_t slot[kWsRing][8];
+#pragma unroll
+  for (int st = 0; st < kWsRing; ++st)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int t = 32 * st + 8 * g4 + i;
+      slot[st][i] = g.row_ids[rs + kbeg + (t < n_tok ? t : 0)];
+      if (t >= n_tok) slot[st][i] = -1;
+    }
+  u32x4 r[kWsRing][8];
+#pragma unroll
+  for (int st = 0; st < kWsRing; ++st)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const bool ok = slot[st][i] >= 0 && slot[st][i] < g.num_slots;
+      r[st][i] = __builtin_nontemporal_load((const u32x4*)(ok ? b_col + slot[st][i] * g.slot_stride_b : z_col));
+    }
+  // ---- softmax of the chunk, 16-bit probabilities into LDS
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    const bool head_ok = m0 + hl + kWsHeadsPerPass * j < g.heads;
+    bool ok[4];
+    float cmax = kNegInf;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ok[i] = head_ok && quad_ok && 4 * tq + i < n_tok;
+      cmax = fmaxf(cmax, ok[i] ? sv[j][i] : kNegInf);
+    }
+    cmax = half_wave_max(cmax);
+    float sum = 0.f;
+    uint16_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float e = ok[i] ? __builtin_amdgcn_exp2f(sv[j][i] - cmax) : 0.f;
+      sum += e;
+      o[i] = BF16 ? f32_to_bf16_bits(e) : f32_to_f16_bits(e);
+    }
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+    const int q_dst = tq < kWsChunk / 4 ? tq : kWsChunk / 4;  // lanes past the chunk: the spare slot behind the row
+    *(uint2*)(p_lds + (hl + kWsHeadsPerPass * j) * kWsPStride + q_dst * 8) =
+        uint2{(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
+    if (tq == 0) {
+      fin_s[0][hl + kWsHeadsPerPass * j] = cmax;
+      fin_s[1][hl + kWsHeadsPerPass * j] = sum;
+    }
+  }
+  __syncthreads();
+  // ---- products: heads x tokens (LDS) times tokens x columns (registers, 8x8 blocks transposed)
+  float4v acc[MT][8];
+#pragma unroll
+  for (int ht = 0; ht < MT; ++ht)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[ht][j] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int st = 0; st < kWsRing; ++st) {
+    const char* prow = p_lds + c * kWsPStride + (32 * st + 8 * g4) * 2;
+    u32x4 pf[MT];
+#pragma unroll
+    for (int ht = 0; ht < MT; ++ht) pf[ht] = *(const u32x4*)(prow + ht * 16 * kWsPStride);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      u32x4 tcol;  // column j of the 8x8 block: dword p = (row 2p, row 2p+1)
+      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) tcol[p] = __builtin_amdgcn_perm(r[st][2 * p + 1][j >> 1], r[st][2 * p][j >> 1], sel);
+#pragma unroll
+      for (int ht = 0; ht < MT; ++ht) acc[ht][j] = mfma16<BF16>(pf[ht], tcol, acc[ht][j]);
+    }
+  }
+  if (g.partial_ml && blockIdx.x == 0 && tid < 16 * MT && m0 + tid < g.heads) {
+    float* ml = g.partial_ml + (((int64_t)blockIdx.z * g.n_seqs + z) * g.heads + m0 + tid) * 2;
+    ml[0] = fin_s[0][tid];
+    ml[1] = fin_s[1][tid];
+  }
+  if (!col_ok) return;
+#pragma unroll
+  for (int ht = 0; ht < MT; ++ht)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + 16 * ht + 4 * g4 + i;
+      if (m >= g.heads) continue;
+      if (g.partial) {
+        float* dst = g.partial + (((int64_t)blockIdx.z * g.n_seqs + z) * g.heads + m) * g.n + col0;
+        *(float4v*)dst = float4v{acc[ht][0][i], acc[ht][1][i], acc[ht][2][i], acc[ht][3][i]};
+        *(float4v*)(dst + 4) = float4v{acc[ht][4][i], acc[ht][5][i], acc[ht][6][i], acc[ht][7][i]};
+      } else {  // the sequence's only chunk: the context row itself
+        const float l = fin_s[1][16 * ht + 4 * g4 + i];
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+        uint16_t h[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float v = acc[ht][j][i] * inv;
+          h[j] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+        }
+        u32x4 o;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) o[p] = (uint32_t)h[2 * p] | ((uint32_t)h[2 * p + 1] << 16);
+        *(u32x4*)(g.out + ((int64_t)z * g.out_batch_stride + (int64_t)m * g.out_row_stride + col0) * 2) = o;
+      }
+    }
+}
+
 // ctx[z][h][n] = sum_p w_p * partial[p][z][h][n] / sum_p w_p * l_p with w_p = 2^(m_p - max_p m_p): the partitions
 // of a sequence put on one scale, added in the order of the partitions, 4 columns per thread.
 template <bool BF16>
@@ -844,6 +998,7 @@ struct Plan {
   int score_parts;   // parts of K in the scores kernel (partial scores, made whole by score_parts_sum_kernel)
   int64_t score_k_per_part;
   int k_per_part;
+  bool chunked;      // few cached rows: one chunk of tokens per workgroup of the weighted sum
   int64_t off_qt, off_s, off_ctx, off_tiles, off_order, off_zero, off_partial, off_ml, off_vp, total;
   int64_t zero_bytes;      // the row of zeros and, behind it, the arrival counters: cleared by the planning workgroup
   int64_t off_vp_counters;
@@ -869,6 +1024,15 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   while ((p.lp + parts - 1) / parts > kWsMaxPart - kWsChunk) parts *= 2;
   p.k_per_part = (int)align_up((p.lp + parts - 1) / parts, kWsChunk);
   p.kparts = (int)((p.lp + p.k_per_part - 1) / p.k_per_part);
+  // few cached rows in all (the host knows only an upper bound of the chunks): a chunk per workgroup
+#ifndef APS_WS_CHUNKED_MAX
+#define APS_WS_CHUNKED_MAX 32
+#endif
+  p.chunked = n_seqs * ((p.lp + kWsChunk - 1) / kWsChunk) <= APS_WS_CHUNKED_MAX;
+  if (p.chunked) {
+    p.k_per_part = kWsChunk;
+    p.kparts = (int)((p.lp + kWsChunk - 1) / kWsChunk);
+  }
   // scores: with few 128-token tiles, K is split by whole 512-element chunks into as many parts as still give
   // at most one workgroup per CU (one round of long-lived workgroups streams fastest)
   {
@@ -1052,14 +1216,17 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     const int mt = g.m_tiles > 1 ? 3 : (num_heads + 15) / 16;
     const dim3 grid((unsigned)((hidden + kWsWaves * 128 - 1) / (kWsWaves * 128)), (unsigned)(n_seqs * g.m_tiles),
                     (unsigned)p.kparts);
-#define APS_LAUNCH_WSUM(B)                                                                          \
-  switch (mt) {                                                                                     \
-    case 1: APS_LAUNCH((hidden_wsum_kernel<B, 1>), grid, dim3(kWsThreads), 0, s, g); break;         \
-    case 2: APS_LAUNCH((hidden_wsum_kernel<B, 2>), grid, dim3(kWsThreads), 0, s, g); break;         \
-    default: APS_LAUNCH((hidden_wsum_kernel<B, 3>), grid, dim3(kWsThreads), 0, s, g); break;        \
+#define APS_LAUNCH_WSUM_K(K, B)                                                             \
+  switch (mt) {                                                                             \
+    case 1: APS_LAUNCH((K<B, 1>), grid, dim3(kWsThreads), 0, s, g); break;                  \
+    case 2: APS_LAUNCH((K<B, 2>), grid, dim3(kWsThreads), 0, s, g); break;                  \
+    default: APS_LAUNCH((K<B, 3>), grid, dim3(kWsThreads), 0, s, g); break;                 \
   }
+#define APS_LAUNCH_WSUM(B) \
+  if (p.chunked) { APS_LAUNCH_WSUM_K(hidden_wsum_chunk_kernel, B) } else { APS_LAUNCH_WSUM_K(hidden_wsum_kernel, B) }
     if (bf16) { APS_LAUNCH_WSUM(true) } else { APS_LAUNCH_WSUM(false) }
 #undef APS_LAUNCH_WSUM
+#undef APS_LAUNCH_WSUM_K
     int st = launch_status();
     if (st != APS_OK) return st;
     if (p.kparts > 1) {

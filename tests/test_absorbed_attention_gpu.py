@@ -124,3 +124,18 @@ def test_absorbed_attention_partitions_agree_with_one_pass(dev):
     sequence inside a batch large enough to need no split runs in one pass: both against the oracle."""
     run_case(dev, 12, 64, 1, 1.0, 900, N=128, seed=9, lens=[900])
     run_case(dev, 12, 64, 1, 1.0, 900, N=2048, seed=9, lens=[900] + [16] * 300)
+
+
+@pytest.mark.parametrize("H,D,lens,N", [(40, 128, [1, 95, 96, 97], 64),           # chunk boundaries, one-token sequence
+                                        (40, 128, [310, 200, 130], 64),           # a serving step's handful
+                                        (12, 64, [192, 193, 3, 289, 96, 40, 7, 100], 128),
+                                        (4, 64, [700, 20], 64),                   # 8 chunks of one sequence, 1 of the other
+                                        (12, 64, [90], 16), (12, 64, [97, 97, 97, 97, 97, 97, 97, 97, 97, 97, 97], 128)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_absorbed_attention_of_few_cached_rows_one_chunk_per_workgroup(dev, H, D, lens, N, dtype):
+    """Batches with few cached rows in all take the weighted-sum kernel that gives every 96-token chunk a
+    workgroup of its own (one chunk: context rows written directly; several: per-chunk sums combined afterwards;
+    chunks past a shorter sequence's end are skipped), up to the bound where the streaming kernel takes over."""
+    # (the ramp makes outputs of magnitude ~25, which bf16's 8 bits cannot hold to the bar: fp16 only)
+    ramp = 1.5 if len(lens) == 3 and dtype == torch.float16 else 0.0
+    run_case(dev, H, D, len(lens), 1.0, max(lens), N, dtype=dtype, lens=lens, ramp=ramp)
