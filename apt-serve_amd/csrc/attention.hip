@@ -1,20 +1,23 @@
 // Paged decode attention over a hybrid cache for gfx950.
 //
-// One wavefront (one 64-thread workgroup) owns (sequence, head, partition): a
-// partition is a run of `partition_size` consecutive tokens of one sequence.
-// Lane layout for a head vector of D elements: LPT = D*elem_bytes/16 lanes
-// hold one token (16 bytes each), so one wave-wide 128-bit load covers
-// TPL = 64/LPT tokens; a tile of 16 tokens (never crossing a block because the
-// block size is a multiple of 16) takes NG = 16/TPL loads for K and NG for V.
-// Each of the TPL token rows of the wave runs its own online softmax over the
-// tokens it sees (no cross-row traffic in the loop); rows are merged once at
-// the end.  The next tile's K/V are requested before the current tile is
-// consumed, so a wave keeps 2 tiles (2 x 16 tokens x 2 x D) in flight.
+// A wavefront owns (sequence, group of HPW adjacent heads, partition): a partition is a run of `partition_size`
+// consecutive tokens of one sequence.  Lane layout for a head vector of D elements: LPT = D*elem_bytes/16 lanes
+// hold one (token, head) (16 bytes each), the HPW heads of a token sit side by side, so one wave-wide 128-bit
+// load covers TPL = 64/(LPT*HPW) tokens; a tile of 16 tokens (never crossing a block because the block size is a
+// multiple of 16) takes NG = 16/TPL loads for K and NG for V.  Each of the TPL token rows of the wave runs its
+// own online softmax over the tokens it sees (no cross-row traffic in the loop); rows are merged once at the end.
+// DEPTH tiles are in flight per wavefront, requested through buffer descriptors so that no load sits under a
+// branch.
 //
-// Per tile the K or V source is chosen per block: block_types[b][i] != 0 reads
-// logical block i from the re-projection workspace, otherwise from the
-// persistent K/V cache.  Partitions of one (sequence, head) are combined by a
-// second small kernel through their log-sum-exp.
+// Per tile the K or V source is chosen per block: block_types[b][i] != 0 reads logical block i from the
+// re-projection workspace, otherwise from the persistent K/V cache.
+//
+// Two ways to put the partitions of a (sequence, head group) together:
+//   group path (a sequence has at most 8 partitions): one workgroup per (head group, sequence), wavefront w walks
+//     partition w, and the wavefront that finishes last merges the partial results through LDS - one launch, no
+//     partial results in HBM.  Workgroups are dealt out longest sequence first.
+//   flat path (more partitions than a workgroup has wavefronts): one 64-thread workgroup per (head group,
+//     partition, sequence) leaves fp32 partial results and their log-sum-exp; combine_partitions_kernel merges them.
 #include <hip/hip_fp16.h>
 
 #include <math.h>
