@@ -15,7 +15,7 @@ The graph ends at the decoder's final LayerNorm; the logits product and the argm
 reductions may record memset nodes, which this runtime replays unreliably).
 
 Mirrors what ``CUDAGraphRunner`` does for the reference's stock decode path
-(additional_designs/worker/aptserve_model_runner.py:1063-1260, which never passes ``shared_cache`` and is
+(additional_designs/worker/aptserve_model_runner.py:1161-1260, which never passes ``shared_cache`` and is
 therefore not usable with hidden-cached sequences there).
 """
 

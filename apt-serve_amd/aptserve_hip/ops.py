@@ -563,7 +563,7 @@ def linear_nt(x, weight, bias=None, out=None, out_row_map=None, workspace=None, 
     With ``split_k`` (default) a problem of few output tiles is split along K through an fp32
     ``workspace`` (allocated here when not given) so that enough workgroups stream the weights.
     ``relu``: negative results are stored as zero (``fc1`` with the activation that follows it,
-    additional_designs/model_executor/models/aptserve_opt.py:205-206).
+    additional_designs/model_executor/models/aptserve_opt.py:204-205).
     The K split of a decode step's few rows is summed inside the same launch (by the workgroup that finishes a
     tile last) with the help of a small array of counters kept per device and stream (:func:`_tile_counters`).
     """

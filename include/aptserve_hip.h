@@ -442,7 +442,7 @@ int aps_build_prefill_metadata(
  * a single-launch kernel runs.  A workspace that is passed but too small or
  * misaligned is an error (APS_ERR_WORKSPACE), never a silent fallback.
  * flags: APS_LINEAR_RELU stores max(result, 0) — the ReLU between fc1 and fc2
- * of the decoder's MLP (model_executor/models/aptserve_opt.py:205-207:
+ * of the decoder's MLP (model_executor/models/aptserve_opt.py:204-206:
  * `fc1`, `activation_fn`, `fc2`) without an element-wise launch of its own; the
  * rounded values are those of "linear, then relu" on 16-bit tensors.
  * tile_counters (nullable): APS_LINEAR_TILE_COUNTERS int32 that are zero on
@@ -545,7 +545,7 @@ int aps_absorbed_attention(
 /* Residual add and LayerNorm of a decoder layer in one launch.
  * ref: model_executor/models/aptserve_opt.py:186-211 (OPTDecoderLayer.forward:
  * `hidden_states = residual + hidden_states` followed by the next nn.LayerNorm,
- * which at :189-190 produces the rows a hidden-cached sequence caches).
+ * which at :188-189 produces the rows a hidden-cached sequence caches).
  *   s[r, :]      = round16(x[r, :] + residual[r, :])        (residual nullable: s = x)
  *   normed[r, :] = LayerNorm(s[r, :]) * gamma + beta        (fp32 statistics over the rounded sum, eps as given)
  * sum (nullable) receives s, the next residual.  f16 / bf16; width a multiple

@@ -94,7 +94,7 @@ def test_few_rows_weight_stream_strides_row_map_and_workspace(dev):
 @pytest.mark.parametrize("M", [1, 2, 5, 16, 30, 48, 49, 100, 300, 3328])   # every kernel family and the tail split
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_relu_epilogue_equals_relu_of_the_rounded_product(dev, M, dtype):
-    """fc1 with its activation (aptserve_opt.py:205-206): negative results are stored as zero, everything else
+    """fc1 with its activation (aptserve_opt.py:204-205): negative results are stored as zero, everything else
     bit for bit as without the flag — in the epilogue of every kernel of the family and in the kernels that add
     K-split partial products."""
     N, K = (512, 192) if M < 1000 else (5120, 1024)
