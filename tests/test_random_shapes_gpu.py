@@ -30,24 +30,27 @@ def test_projection_family_random_shapes(dev, seed):
         M = int(rng.choice(rows)); N = 256 * int(rng.integers(1, 7)); K = 64 * int(rng.integers(1, 22))
         dtype = DT16[int(rng.integers(0, 2))]
         use_map, strided, bias, sk = (bool(rng.integers(0, 2)) for _ in range(4))
+        relu = bool(rng.integers(0, 3) == 0)
         xs = randn((M, 2 * K if strided else K), s, dtype)
         x = xs[:, K:] if strided else xs
         w = (randn((N, K), s + 1) * 0.05).to(dtype)
         b = randn((N,), s + 2, dtype) if bias else None
         ref = OR._linear_fp32(x, w, b)
+        if relu:     # fc1 with its activation: max(., 0) of the rounded product
+            ref = torch.relu(ref)
         dx = xs.to(dev)[:, K:] if strided else xs.to(dev)
         db = None if b is None else b.to(dev)
-        what = f"case {case}: M={M} N={N} K={K} {dtype} map={use_map} strided={strided} bias={bias} split_k={sk}"
+        what = f"case {case}: M={M} N={N} K={K} {dtype} map={use_map} strided={strided} bias={bias} split_k={sk} relu={relu}"
         try:
             if use_map:
                 n_out = M + 7
                 perm = rng.permutation(n_out)[:M]
                 out = torch.full((n_out, N), 5.0, dtype=dtype, device=dev)
-                ops.linear_nt(dx, w.to(dev), db, out=out, out_row_map=torch.from_numpy(perm).to(dev), split_k=sk)
+                ops.linear_nt(dx, w.to(dev), db, out=out, out_row_map=torch.from_numpy(perm).to(dev), split_k=sk, relu=relu)
                 TR.check(out.cpu()[perm], ref, dtype)
                 assert (out.cpu()[np.setdiff1d(np.arange(n_out), perm)] == 5).all()
             else:
-                TR.check(ops.linear_nt(dx, w.to(dev), db, split_k=sk), ref, dtype)
+                TR.check(ops.linear_nt(dx, w.to(dev), db, split_k=sk, relu=relu), ref, dtype)
         except AssertionError as e:
             raise AssertionError(f"{what}: {e}") from e
 
@@ -183,3 +186,97 @@ def test_metadata_random_batches(dev, seed):
         for packed in (False, True):
             md = metadata.build_from_batch(batch, dev, packed=packed, check_totals=True)
             assert_same(md, oracle_metadata(batch))
+
+
+@pytest.mark.parametrize("seed", [61])
+def test_attention_on_hidden_rows_random_batches(dev, seed):
+    """Batches of hidden-cached sequences of random number and lengths: few rows (a chunk of tokens per workgroup of
+    the weighted sum), more (the streaming kernel, token partitions), head layouts 4x64 .. 40x128."""
+    import test_absorbed_attention_gpu as TAB
+    rng = np.random.default_rng(seed)
+    for case in range(14):
+        H, D = [(4, 64), (12, 64), (8, 128), (40, 128)][int(rng.integers(0, 4))]
+        n = int(rng.integers(1, 9))
+        hi = int(rng.choice([30, 97, 200, 700]))
+        lens = [int(x) for x in rng.integers(1, hi + 1, n)]
+        dtype = DT16[int(rng.integers(0, 2))]
+        N = 2 * sum(-(-l // 16) for l in lens) + 8
+        try:
+            TAB.run_case(dev, H, D, n, 1.0, max(lens), N, dtype=dtype, seed=int(rng.integers(0, 1000)), lens=lens)
+        except AssertionError as e:
+            raise AssertionError(f"case {case}: H={H} D={D} lens={lens} {dtype}: {e}") from e
+
+
+@pytest.mark.parametrize("seed", [71])
+def test_prefix_attention_random_batches(dev, seed):
+    """Prompt chunks of random lengths behind cached prefixes of random lengths (none included), both block sizes."""
+    rng = np.random.default_rng(seed)
+    for case in range(12):
+        H, D = [(2, 64), (5, 128), (12, 64)][int(rng.integers(0, 3))]
+        B = int(rng.integers(1, 6))
+        qlens = [int(x) for x in rng.integers(1, int(rng.choice([8, 70, 300])) + 1, B)]
+        ctx = [int(x) for x in rng.integers(0, int(rng.choice([1, 40, 500])) + 1, B)]
+        klens = [q + c for q, c in zip(qlens, ctx)]
+        dtype = DT16[int(rng.integers(0, 2))]
+        try:
+            TP.run_prefix(dev, klens, qlens, H, D, dtype, seed=int(rng.integers(0, 1000)), BS=int(rng.choice([16, 32])))
+        except AssertionError as e:
+            raise AssertionError(f"case {case}: H={H} D={D} klens={klens} qlens={qlens} {dtype}: {e}") from e
+
+
+@pytest.mark.parametrize("seed", [81])
+def test_add_layer_norm_random_shapes(dev, seed):
+    import torch.nn.functional as F
+    rng = np.random.default_rng(seed)
+    for case in range(30):
+        rows = int(rng.integers(1, 40)); width = 8 * int(rng.integers(1, 2049))
+        dtype = DT16[int(rng.integers(0, 2))]
+        strided, with_res = bool(rng.integers(0, 2)), bool(rng.integers(0, 4))
+        wide = randn((rows, 2 * width), case, dtype).to(dev)
+        x = wide[:, :width] if strided else wide[:, :width].contiguous()
+        r = (wide[:, width:] if strided else wide[:, width:].contiguous()) if with_res else None
+        w, b = (1 + 0.1 * randn((width,), case + 1)).to(dtype).to(dev), (0.1 * randn((width,), case + 2)).to(dtype).to(dev)
+        normed, s_ = ops.add_layer_norm(x, r, w, b)
+        s_ref = (x.float() + r.float()).to(dtype) if with_res else x
+        assert bits_equal(s_, s_ref), f"case {case}: rows={rows} width={width} {dtype} strided={strided}: sum differs"
+        n_ref = F.layer_norm(s_ref.float(), (width,), w.float(), b.float(), 1e-5)
+        ulp = 2 ** -10 if dtype == torch.float16 else 2 ** -7
+        d = (normed.float() - n_ref).abs()
+        assert (d <= ulp * n_ref.abs() + 2e-3).all(), f"case {case}: rows={rows} width={width} {dtype}: {d.max().item()}"
+
+
+@pytest.mark.parametrize("seed", [91])
+def test_decode_step_cache_ops_random_batches(dev, seed):
+    """One launch for a decode layer's cache traffic (hidden stores, holder, new K/V rows) on random batches, with and
+    without a holder, against the oracle's separate operators."""
+    rng = np.random.default_rng(seed)
+    for case in range(16):
+        H, D = [(1, 8), (4, 32), (12, 64), (5, 128)][int(rng.integers(0, 4))]
+        N, BS = 96, 16
+        dtype = DT16[int(rng.integers(0, 2))]
+        b = workloads.small_decode_batch(int(rng.integers(0, 1000)), int(rng.integers(1, 12)), int(rng.integers(1, 120)),
+                                         float(rng.choice([0.0, 0.5, 1.0])), N)
+        md, gmd = oracle_metadata(b), metadata.build_from_batch(b, dev)
+        B, T, Hd = len(b.seq_lens), md["num_tot_tokens"], H * D
+        hs, kv = randn((B, Hd), case, dtype), randn((B, 2 * Hd), case + 7, dtype)
+        k, v = kv.chunk(2, -1)
+        cache = sentinel_cache((2, N, BS, H, D), dtype)
+        ref = cache.clone()
+        sm = t64(md["slot_mapping"])
+        O.hidden_to_cache(hs, ref, sm, t64(md["hidden_cache_use_input"]), t64(md["hidden_cache_store_tot"]))
+        holder_ref = O.assemble_hidden_holder(hs, ref, sm, T, t64(md["hidden_holder_upd"]), t64(md["hidden_cache_use_tot"]))
+        seq_idx = torch.tensor([i for i, h in enumerate(b.use_hidden) if not h], dtype=torch.int64)
+        if len(seq_idx):
+            O.reshape_and_cache_flash(k[seq_idx].reshape(-1, H, D), v[seq_idx].reshape(-1, H, D), ref[0], ref[1],
+                                      sm[t64(md["kv_cache_use_tot"])], "auto")
+        with_holder = bool(rng.integers(0, 2)) and T > 0
+        g = cache.to(dev)
+        holder = sentinel_cache((T, Hd), dtype, seed=5).to(dev) if with_holder else None
+        dk, dv = kv.to(dev).chunk(2, -1)
+        ops.decode_step_cache_ops(holder, hs.to(dev), g, gmd.holder_src if with_holder else None, gmd.slot_mapping,
+                                  gmd.hidden_cache_use_input, gmd.hidden_cache_store_tot, dk, dv,
+                                  gmd.kv_cache_use_input, gmd.new_token_slot)
+        what = f"case {case}: H={H} D={D} {dtype} seqs={B} holder={with_holder}"
+        assert bits_equal(g, ref), what
+        if with_holder:
+            assert bits_equal(holder, holder_ref), what
