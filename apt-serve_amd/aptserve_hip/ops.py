@@ -546,6 +546,9 @@ def _tile_counters(dev) -> torch.Tensor:
     key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
     t = _TILE_COUNTERS.get(key)
     if t is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("linear_nt: the first K-split product on a stream allocates and clears its tile counters; "
+                               "run one eager step on the capturing stream before recording it")
         with torch.cuda.stream(torch.cuda.default_stream(dev)):     # allocated and cleared outside any capture
             t = torch.zeros(256, dtype=torch.int32, device=dev)
         torch.cuda.default_stream(dev).synchronize()

@@ -50,6 +50,15 @@ __global__ __launch_bounds__(kLnThreads) void add_layer_norm_kernel(const AddLnA
   const char* r = g.residual ? g.residual + row * g.res_stride_b : nullptr;
   float v[VECS][8];
   float total = 0.f;
+  // scale and shift of the norm are requested with the row itself: on a handful of rows the launch lasts as long
+  // as its chain of memory round trips, and these two would otherwise form a third one after the statistics
+  u32x4 gw[VECS], gb[VECS];
+#pragma unroll
+  for (int j = 0; j < VECS; ++j) {
+    const int i = min((int)threadIdx.x + j * kLnThreads, nvec - 1);
+    gw[j] = *(const u32x4*)(g.gamma + (int64_t)i * 16);
+    gb[j] = g.beta ? *(const u32x4*)(g.beta + (int64_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+  }
 #pragma unroll
   for (int j = 0; j < VECS; ++j) {
     const int i = threadIdx.x + j * kLnThreads;
@@ -90,9 +99,7 @@ __global__ __launch_bounds__(kLnThreads) void add_layer_norm_kernel(const AddLnA
   for (int j = 0; j < VECS; ++j) {
     const int i = threadIdx.x + j * kLnThreads;
     if (i < nvec) {
-      const u32x4 w = *(const u32x4*)(g.gamma + (int64_t)i * 16);
-      u32x4 bb = {0u, 0u, 0u, 0u};
-      if (g.beta) bb = *(const u32x4*)(g.beta + (int64_t)i * 16);
+      const u32x4 w = gw[j], bb = gb[j];
       u32x4 o;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
