@@ -25,7 +25,7 @@ for p in (ROOT, ROOT / "apt-serve_amd"):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (seed 0 workloads), scaled by what the
 # same counters read for the 1 GiB copy kernel (x2.000 and x1.000); summary in profiles/bench_step_hbm_counters.txt
-PMC_TRAFFIC_BYTES = {"step": 1815.2e6, "attention_f16": 1793.3e6, "attention_fp8": 898.3e6,
+PMC_TRAFFIC_BYTES = {"step": 1815.1e6, "attention_f16": 1793.3e6, "attention_fp8": 898.3e6,
                      "gemm_T4096": 868.0e6, "gemm_T16384": 2883.0e6}
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 
