@@ -123,6 +123,9 @@ struct GemmArgs {
   // stores a tile's last partial product adds the parts itself (and puts the counter back to zero) instead of
   // leaving them to a second launch.
   int* tile_counters;
+  // weight_stream_kernel only: weight rows of a workgroup (a multiple of 16, at most 128; 0 = 128).  The wavefronts
+  // beyond them only help to stage the activations.
+  int rows_per_wg;
   // tail split (large M): logical tiles from tail_from on are cut into tail_ways parts of tail_kt k-tiles each;
   // part p of tail tile i stores its fp32 result tile at tail_partial[(i * tail_ways + p)][256][256]
   float* tail_partial;
@@ -692,12 +695,14 @@ __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArg
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int g4 = lane >> 4, c = lane & 15;
-  const int64_t n0 = (int64_t)blockIdx.x * kScTokens;
+  const int rows_wg = g.rows_per_wg ? g.rows_per_wg : kScTokens;
+  const bool streams = wave * 16 < rows_wg;   // a wavefront past the workgroup's rows reads row 0 (cache hits), stores nothing
+  const int64_t n0 = (int64_t)blockIdx.x * rows_wg;
   const int64_t k0 = (int64_t)blockIdx.y * k_per_part;
   const int64_t klen = min(g.k - k0, k_per_part);
   const int64_t m0 = (int64_t)blockIdx.z * (16 * NHT);
-  auto weight_row = [&](int64_t n) {  // rows past the matrix: row 0, never stored
-    return g.w + (n < g.n ? n : 0) * g.ldw_b + (lane & 7) * 16 + k0 * 2;
+  auto weight_row = [&](int64_t n) {  // rows past the matrix or the workgroup's share: row 0, never stored
+    return g.w + ((n < g.n && streams) ? n : 0) * g.ldw_b + (lane & 7) * 16 + k0 * 2;
   };
   float4v acc[NHT];
   // (head-wise x: the 128 weight rows of a workgroup lie inside one head, whose x is the image)
@@ -707,7 +712,7 @@ __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArg
                                      g.a + head_off + m0 * g.lda_b + k0 * 2,
                                      g.lda_b, (int)min((int64_t)(16 * NHT), g.m - m0), klen, lds, acc);
   // lane (g4, c) holds activation rows m0 + 16*ht + 4*g4 + i and weight row n0 + 16*wave + c
-  const int64_t n = n0 + wave * 16 + c;
+  const int64_t n = streams ? n0 + wave * 16 + c : g.n;
   const bool own = g.partial && g.tile_counters;   // the last workgroup of a tile adds the parts
   if (n >= g.n && !own) return;
   if (g.partial && n < g.n) {
@@ -775,32 +780,46 @@ __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArg
     }
 }
 
-// Parts of K for the kernel above: whole chunks, as even as possible, and as many workgroups as still fit one
-// per CU.  Measured (13B layer shapes, 3..48 rows): one round of long-lived workgroups beats more, shorter
-// ones even when they could share a CU (n=5120, k=20480: 240 workgroups 38 us, 400 workgroups 50 us) and even
-// when it leaves CUs idle (n=20480, k=5120: 160 workgroups, no K split, 39 us; 480 workgroups 41-55 us): a
-// workgroup's first loads meet the full memory latency with nothing to overlap, and a CU streams at 34 GB/s
-// while the chip is not saturated.
-int weight_stream_parts(int64_t m, int64_t n, int64_t k, int64_t* k_per_part) {
+// Rows per workgroup and parts of K for the kernel above.  Measured (13B layer shapes, 3..48 rows): one round of
+// long-lived workgroups beats more, shorter ones even when they could share a CU (n=5120, k=20480: 240 workgroups
+// 38 us, 400 workgroups 50 us): a workgroup's first loads meet the full memory latency with nothing to overlap.
+// A CU on its own streams ~34 GB/s and the chip ~6.9 TB/s, so a launch wants all 256 CUs; and a K split costs a
+// cross-workgroup sum at its end (~3.8 us: store acknowledgement, counter, loads of the parts).  Hence the choice by
+// a small cost model over (rows per workgroup in {128, 112, 96, 80, 64}, whole-chunk K parts) with at most one
+// workgroup per CU: time of the longest part at min(34 GB/s, 6.9 TB/s / workgroups) plus the sum if K is split.
+// 13B shapes: n=15360 (qkv) 240 workgroups of 64 rows, no split (was 120 x 2 parts); n=20480 (fc1) 256 workgroups
+// of 80 rows (was 160 of 128: 96 CUs idle); n=5120, k=5120 stays at 40 x 5 parts; n=5120, k=20480 64 x 4 parts.
+struct WsPlan { int rows, parts; int64_t k_per_part; };
+WsPlan weight_stream_plan(int64_t m, int64_t n, int64_t k, bool whole_tiles_only = false) {
   const int nht = m <= 16 ? 1 : (m <= 32 ? 2 : 3);
-  const int64_t tiles = ((n + kScTokens - 1) / kScTokens) * ((m + 16 * nht - 1) / (16 * nht));
+  const int64_t mt = (m + 16 * nht - 1) / (16 * nht);
   const int64_t chunks = (k + kScChunk - 1) / kScChunk;
-  int64_t best_per = chunks;  // one part
-  for (int64_t per = chunks; per >= 1; --per) {
-    const int64_t parts = (chunks + per - 1) / per;
-    if (tiles * parts > kNumCus) break;
-    const int64_t last = chunks - (parts - 1) * per;
-    if (last * 2 < per) continue;  // a last part under half a part leaves its workgroups idle early
-    best_per = per;
+  WsPlan best{kScTokens, 1, chunks * kScChunk};
+  double best_t = 1e30;
+  for (int rows = kScTokens; rows >= (whole_tiles_only ? kScTokens : 64); rows -= 16) {
+    const int64_t tiles = ((n + rows - 1) / rows) * mt;
+    for (int64_t per = chunks; per >= 1; --per) {
+      const int64_t parts = (chunks + per - 1) / per;
+      if (tiles * parts > kNumCus) break;
+      const int64_t last = chunks - (parts - 1) * per;
+      if (last * 2 < per) continue;  // a last part under half a part leaves its workgroups idle early
+      const double wgs = (double)(tiles * parts);
+      const double rate = 34e9 < 6.9e12 / wgs ? 34e9 : 6.9e12 / wgs;
+      const double t = (double)rows * (double)per * kScChunk * 2 / rate + (parts > 1 ? 3.8e-6 : 0.0);
+      if (t < best_t * 0.995) {  // (ties go to the larger workgroup: fewer idle wavefronts)
+        best_t = t;
+        best = WsPlan{rows, (int)parts, per * kScChunk};
+      }
+    }
   }
-  if (k_per_part) *k_per_part = best_per * kScChunk;
-  return (int)((chunks + best_per - 1) / best_per);
+  return best;
 }
 
 template <bool BF16>
 int launch_weight_stream(const GemmArgs& g, int parts, int64_t k_per_part, hipStream_t s) {
   const int nht = g.m <= 16 ? 1 : (g.m <= 32 ? 2 : 3);
-  const dim3 grid((unsigned)((g.n + kScTokens - 1) / kScTokens), (unsigned)parts,
+  const int rows = g.rows_per_wg ? g.rows_per_wg : kScTokens;
+  const dim3 grid((unsigned)((g.n + rows - 1) / rows), (unsigned)parts,
                   (unsigned)((g.m + 16 * nht - 1) / (16 * nht)));
   hipError_t e = hipSuccess;
 #define APS_LAUNCH_WS(N)                                                                                          \
@@ -934,7 +953,7 @@ int aps_linear_nt_splits(int64_t m, int64_t n, int64_t k) {
   // per tile: split K until about two waves of workgroups exist, keeping at least 4 k-tiles per split.
   if (m <= 0 || n <= 0 || k <= 0 || n % BN != 0 || k % BK != 0) return 1;
   if (m <= kRsMaxRows) return 1;  // streamed in one launch
-  if (m <= kWsMaxRows) return weight_stream_parts(m, n, k, nullptr);
+  if (m <= kWsMaxRows) return weight_stream_plan(m, n, k).parts;
   const int64_t bm = 64 * tile_mi(m, n);
   const int64_t tiles = ((m + bm - 1) / bm) * (n / BN);
   const int64_t nk = k / BK;
@@ -1000,9 +1019,11 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   if (!gs && m <= kRsMaxRows)
     return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
   if (!gs && m <= kWsMaxRows) {
-    int64_t k_per_part = 0;
-    const int parts = weight_stream_parts(m, n, k, &k_per_part);
+    const WsPlan wp = weight_stream_plan(m, n, k);
+    const int parts = wp.parts;
+    const int64_t k_per_part = wp.k_per_part;
     if (parts == 1 || (workspace && workspace_bytes >= (int64_t)parts * m * n * 4 && !(addr(workspace) & 15))) {
+      g.rows_per_wg = wp.rows;
       g.partial = parts > 1 ? (float*)workspace : nullptr;
       g.tile_counters = parts > 1 ? (int*)tile_counters : nullptr;   // (at most kNumCus tiles are split)
       int st = dtype == APS_BF16 ? launch_weight_stream<true>(g, parts, k_per_part, s)
@@ -1104,7 +1125,7 @@ __attribute__((visibility("hidden"))) int64_t aps_internal_headwise_workspace_by
                                                                                    int head_rows) {
   if (m < 3 || m > kWsMaxRows || head_rows <= 0 || head_rows % kScTokens != 0 || n % kScTokens != 0 || k % BK != 0)
     return 0;
-  const int parts = weight_stream_parts(m, n, k, nullptr);
+  const int parts = weight_stream_plan(m, n, k, true).parts;
   return parts > 1 ? (int64_t)parts * m * n * 4 : 16;   // (a nonzero size says "this shape is covered")
 }
 
@@ -1132,12 +1153,12 @@ __attribute__((visibility("hidden"))) int aps_internal_headwise_linear(const voi
   if (need > 0 && workspace && tile_counters && workspace_bytes >= need && !(addr(workspace) & 15) &&
       common_vec_bytes({addr(x), addr(weight), (uint64_t)x_stride * 2, (uint64_t)x_head_stride * 2,
                         (uint64_t)w_stride * 2}) == 16) {
-    int64_t k_per_part = 0;
-    const int parts = weight_stream_parts(m, n, k, &k_per_part);
+    const WsPlan wp = weight_stream_plan(m, n, k, true);   // (a workgroup's 128 rows must lie inside one head)
+    const int parts = wp.parts;
     g.partial = parts > 1 ? (float*)workspace : nullptr;
     g.tile_counters = parts > 1 ? (int*)tile_counters : nullptr;
-    return dtype == APS_BF16 ? launch_weight_stream<true>(g, parts, k_per_part, s)
-                             : launch_weight_stream<false>(g, parts, k_per_part, s);
+    return dtype == APS_BF16 ? launch_weight_stream<true>(g, parts, wp.k_per_part, s)
+                             : launch_weight_stream<false>(g, parts, wp.k_per_part, s);
   }
   if (m <= 8 && n % (kRsWaves * kRsRows) == 0)
     return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);

@@ -96,6 +96,7 @@ def test_linear_workspace_planning_is_host_only_and_consistent():
             if m <= 2:
                 assert s == 1                                  # one launch of the dot-product kernel
             elif m <= 48:
+                # whole 512-element chunks of K; workgroups of 64..128 weight rows, at most one per compute unit
                 chunks = -(-k // 512)
                 assert s <= chunks
                 rows = 16 if m <= 16 else (32 if m <= 32 else 48)

@@ -44,11 +44,12 @@ def test_linear_nt_small(dev, M, N, K, dtype):
 
 
 @pytest.mark.parametrize("M", [3, 8, 16, 17, 32, 33, 48])
-@pytest.mark.parametrize("N,K", [(256, 64), (512, 1600), (1024, 2048), (2560, 5120)])
+@pytest.mark.parametrize("N,K", [(256, 64), (512, 1600), (1024, 2048), (2560, 5120), (16896, 1024), (20992, 512)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_linear_nt_few_rows_weight_stream(dev, M, N, K, dtype):
     """3..48 rows: weight rows through the row-streaming MFMA core (16-, 32- and 48-row images), K in one part
-    or in parts added by the reduce kernel, with a short last chunk (K = 64, 1600) and without (2048, 5120);
+    or in parts added by the reduce kernel, with a short last chunk (K = 64, 1600) and without (2048, 5120), and
+    workgroups of fewer than 128 weight rows with a short last one (N = 16896, 20992);
     the same product without a workspace goes through the single-launch kernels and must agree."""
     x = randn((M, K), M + 1, dtype)
     w = (randn((N, K), N + 1) * 0.02).to(dtype)    # outputs of magnitude ~1: the absolute bar holds for bf16 too
@@ -62,7 +63,7 @@ def test_linear_nt_few_rows_weight_stream(dev, M, N, K, dtype):
 
 
 def test_few_rows_weight_stream_strides_row_map_and_workspace(dev):
-    K, N, M = 1024, 2560, 21
+    K, N, M = 2048, 2560, 21
     wide = randn((M, 2 * K + 8), 0)
     x = wide[:, 8:8 + K]                                   # row stride 2K+8, 16-byte aligned start
     wfull = (randn((N + 256, K), 1) * 0.05).half()
@@ -105,8 +106,8 @@ def test_relu_epilogue_equals_relu_of_the_rounded_product(dev, M, dtype):
         assert (plain < 0).any() and torch.equal(act, torch.relu(plain))
 
 
-@pytest.mark.parametrize("M,N,K", [(3, 768, 768), (5, 5120, 5120), (5, 5120, 20480), (17, 1536, 768), (48, 5120, 5120),
-                                   (33, 15360, 5120), (7, 256, 2048)])
+@pytest.mark.parametrize("M,N,K", [(3, 768, 1600), (5, 5120, 5120), (5, 5120, 20480), (17, 1536, 1088), (48, 5120, 5120),
+                                   (33, 7680, 5120), (7, 256, 2048)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_k_split_summed_inside_the_launch_equals_the_two_launch_sum(dev, M, N, K, dtype):
     """The K split of a decode step's few rows with tile counters (the workgroup that stores a tile's last
