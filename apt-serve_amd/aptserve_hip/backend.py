@@ -308,17 +308,20 @@ class HybridOPTAttention:
                 else:
                     ops.reshape_and_cache_flash(k, v, kv_cache[0], kv_cache[1], md.new_token_slot, a.kv_cache_dtype,
                                                 a.k_scale, a.v_scale, token_idx=md.kv_cache_use_input)
-            with phase("attention"):
-                ops.paged_decode_attention(q.view(-1, H, D), kv_cache[0], kv_cache[1], md.private_block_tables,
-                                           md.kv_seq_lens, self.scaling, max_seq_len=md.max_kv_seq_len or None,
-                                           out=attn_output.view(-1, H, D), k_scale=a.k_scale, v_scale=a.v_scale)
+            # planned here, launched by the attention on the hidden rows (the two halves write different rows of
+            # attn_output; a small batch runs them in one launch)
+            kv_job = ops.paged_decode_attention(q.view(-1, H, D), kv_cache[0], kv_cache[1], md.private_block_tables,
+                                                md.kv_seq_lens, self.scaling, max_seq_len=md.max_kv_seq_len or None,
+                                                out=attn_output.view(-1, H, D), k_scale=a.k_scale,
+                                                v_scale=a.v_scale, as_job=True)
         else:
+            kv_job = None
             with phase("projections"):
                 q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
         with phase("attention_on_hidden_rows"):
             ops.absorbed_hidden_attention(q, hidden_cache, md.hidden_slots, md.hidden_seq_start,
                                           md.hidden_cache_use_input, md.max_hidden_seq_len, w[s:2 * s], w[2 * s:],
-                                          None if b is None else b[2 * s:], self.scaling, attn_output)
+                                          None if b is None else b[2 * s:], self.scaling, attn_output, kv_job=kv_job)
         with phase("projections"):
             return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
 

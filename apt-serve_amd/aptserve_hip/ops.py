@@ -9,6 +9,7 @@ HIP library these functions raise.
 from __future__ import annotations
 
 import contextlib
+import ctypes
 from typing import Optional
 
 import torch
@@ -424,11 +425,32 @@ def mixed_kv_to_cache(key, value, k_cache, v_cache, shared_k_cache, shared_v_cac
 
 # --------------------------------------------------------------------- a8
 
+APS_ATTENTION_JOB_BYTES = 320
+
+
+class AttentionJob:
+    """A planned, not yet launched paged decode attention (``paged_decode_attention(..., as_job=True)``):
+    opaque host bytes that the library wrote, and the tensors the launch will touch, kept alive."""
+
+    def __init__(self, out, tensors):
+        self._buf = (ctypes.c_uint64 * (APS_ATTENTION_JOB_BYTES // 8))()
+        self.address = ctypes.addressof(self._buf)
+        self.out = out
+        self._tensors = tensors
+
+    def launch(self):
+        """Launch the job by itself on the current stream of its device; returns the output tensor."""
+        with _on(self.out.device):
+            st = _lib.load().aps_attention_job_launch(self.address, _stream(self.out))
+        _lib.check(st, "attention_job_launch")
+        return self.out
+
+
 def paged_decode_attention(q, k_cache, v_cache, block_tables, seq_lens, softmax_scale=None, *,
                            block_types=None, ws_k_cache=None, ws_v_cache=None, k_scale: float = 1.0,
                            v_scale: float = 1.0, max_seq_len: Optional[int] = None, partition_size: int = 0,
                            out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-                           static_scratch: bool = False):
+                           static_scratch: bool = False, as_job: bool = False):
     """Decode attention of one query token per sequence over paged K/V.
 
     ``q`` ``[B, H, D]`` f16/bf16; caches ``[blocks, BS, H, D]`` in ``q``'s dtype or
@@ -439,7 +461,9 @@ def paged_decode_attention(q, k_cache, v_cache, block_tables, seq_lens, softmax_
     ``W * BS``, which needs no device read-back).  Returns ``[B, H, D]``.
     ``static_scratch=True`` (with ``out`` given) takes the entry point that allocates
     nothing: partial results go to the library's static device array, and a problem
-    that does not fit it raises.
+    that does not fit it raises.  ``as_job=True`` checks and plans the call but launches nothing:
+    the :class:`AttentionJob` that comes back is launched later, by itself or as the K/V-cached half
+    of :func:`absorbed_hidden_attention`.
     """
     dev = q.device
     _check_data("q", q, dev)
@@ -508,6 +532,21 @@ def paged_decode_attention(q, k_cache, v_cache, block_tables, seq_lens, softmax_
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     ws_ptr = workspace.data_ptr() if (need and workspace is not None) else None
     ws_bytes = workspace.numel() * workspace.element_size() if (need and workspace is not None) else 0
+    if as_job:
+        _need(not static_scratch, "a job takes a workspace, not the static scratch")
+        job = AttentionJob(out, (q, k_cache, v_cache, ws_k_cache, ws_v_cache, block_tables, block_types, seq_lens,
+                                 workspace))
+        st = lib.aps_paged_decode_attention_job(
+            job.address, APS_ATTENTION_JOB_BYTES, out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
+            v_cache.data_ptr(), None if block_types is None else ws_k_cache.data_ptr(),
+            None if block_types is None else ws_v_cache.data_ptr(),
+            _ptr(block_tables), None if block_types is None else _ptr(block_types), _ptr(seq_lens), B, H, D, BS, W,
+            block_tables.stride(0) if W else 0, types_stride, q.stride(0), out.stride(0), k_cache.stride(0),
+            k_cache.size(0), ws_stride, ws_blocks, max_seq_len, partition_size, float(softmax_scale),
+            _DTYPE_CODE[q.dtype], APS_FP8_E4M3 if fp8 else _DTYPE_CODE[q.dtype], float(k_scale), float(v_scale),
+            ws_ptr, ws_bytes)
+        _lib.check(st, "paged_decode_attention_job")
+        return job
     with _on(dev):
         st = lib.aps_paged_decode_attention(
             out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
@@ -798,7 +837,7 @@ def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_se
 # ------------------------------------------------------------------ attention on cached hidden rows
 
 def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, seq_rows, max_len, w_k, w_v, b_v,
-                              softmax_scale, out, workspace=None):
+                              softmax_scale, out, workspace=None, kv_job: Optional["AttentionJob"] = None):
     """Decode attention of the hidden-cached sequences of a batch, computed on their cached hidden
     rows with the K/V projection weights absorbed into the query and the output:
     ``s[h,t] = scale <W_k[h]^T q[h], hidden_t>``, ``out[h] = W_v[h] (sum_t p[h,t] hidden_t) + b_v[h]``.
@@ -811,7 +850,12 @@ def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, se
     positions of the hidden-cached sequences; ``hidden_slots`` / ``hidden_seq_start`` from the
     metadata builder; ``w_k``, ``w_v [H*D, H*D]`` row slices of the fused QKV weight; the result of
     sequence ``i`` is written to ``out[seq_rows[i]]`` (``out [B, H*D]``).  The newest hidden row of
-    every sequence must already be in the cache."""
+    every sequence must already be in the cache.
+
+    ``kv_job``: the paged decode attention of the batch's K/V-cached sequences
+    (``paged_decode_attention(..., as_job=True)``), launched by this call as well — inside the
+    launch of the weighted sum over the hidden rows when the batch is small enough for that, by
+    itself otherwise; the results are those of launching the job alone."""
     dev = q.device
     for n, t in (("q", q), ("paged_cache", paged_cache), ("w_k", w_k), ("w_v", w_v), ("out", out)):
         _check_data(n, t, dev)
@@ -834,14 +878,16 @@ def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, se
     n_seqs = seq_rows.numel()
     _need(hidden_seq_start.numel() == n_seqs + 1, "hidden_seq_start needs one entry per sequence plus one")
     if n_seqs == 0:
+        if kv_job is not None:
+            kv_job.launch()
         return out
     lib = _lib.load()
     need = lib.aps_absorbed_attention_workspace_bytes(n_seqs, int(max_len), heads, head_size)
     if workspace is None or workspace.numel() * workspace.element_size() < need:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)      # scratch is host-side plumbing
     with _on(dev):
-        st = lib.aps_absorbed_attention(
-            q.data_ptr(), q.stride(0), seq_rows.data_ptr(), q.size(0), paged_cache.data_ptr(), paged_cache.stride(2),
+        st = lib.aps_hybrid_decode_attention(
+            None if kv_job is None else kv_job.address, q.data_ptr(), q.stride(0), seq_rows.data_ptr(), q.size(0), paged_cache.data_ptr(), paged_cache.stride(2),
             paged_cache.numel() // paged_cache.stride(2), hidden_slots.data_ptr(), hidden_seq_start.data_ptr(),
             n_seqs, int(max_len), w_k.data_ptr(), w_v.data_ptr(), None if b_v is None else b_v.data_ptr(),
             w_k.stride(0), heads, head_size, float(softmax_scale), out.data_ptr(), out.stride(0), out.size(0),

@@ -21,6 +21,7 @@
 
 #include "aps_common.h"
 #include "mfma_common.h"
+#include "paged_decode_core.h"
 #include "row_stream_core.h"
 
 // the per-head value projection lives with the other weight-streaming kernels
@@ -31,6 +32,8 @@ __attribute__((visibility("hidden"))) int aps_internal_headwise_linear(
 // bytes of fp32 partial products that call uses for m rows (0: it runs a kernel that needs none)
 __attribute__((visibility("hidden"))) int64_t aps_internal_headwise_workspace_bytes(int64_t m, int64_t n, int64_t k,
                                                                                    int head_rows);
+// a planned paged decode attention, launched by itself (the attention launcher's translation unit)
+extern "C" int aps_attention_job_launch(const void* job, aps_stream_t stream);
 
 namespace aps {
 namespace {
@@ -507,6 +510,7 @@ __global__ __launch_bounds__(kScThreads) void head_proj_kernel(const HeadProjArg
 #define APS_WS_OCC 2
 #endif
 constexpr int kWsWaves = APS_WS_WAVES, kWsThreads = kWsWaves * 64, kWsRing = APS_WS_RING, kWsChunk = 32 * kWsRing;
+constexpr int kFusedHeadSize = 128;               // head size of the paged attention that can ride in the chunk launch
 constexpr int kWsMaxPart = 4096;                  // tokens of a partition (their slots are staged in LDS)
 constexpr int kWsIds = (kWsMaxPart + kWsChunk - 1) / kWsChunk * kWsChunk + 32 * (kWsRing - 1);
 constexpr int kWsPStride = kWsChunk * 2 + 16;     // bytes between heads of a probability chunk (13 x 16: odd)
@@ -803,7 +807,7 @@ __global__ __launch_bounds__(kWsThreads) __attribute__((amdgpu_waves_per_eu(APS_
 // The price is the fp32 sums of every chunk (heads x hidden values: about as many bytes as the chunk's rows),
 // which is why only small batches come here.
 template <bool BF16, int MT>
-__global__ __launch_bounds__(kWsThreads) void hidden_wsum_chunk_kernel(const WsumArgs g) {
+__device__ __forceinline__ void hidden_wsum_chunk_body(const WsumArgs& g) {
   constexpr int NJ = 16 * MT / kWsHeadsPerPass;
   __shared__ __attribute__((aligned(16))) char p_lds[16 * MT * kWsPStride];
   __shared__ __attribute__((aligned(16))) float fin_s[2][16 * MT];
@@ -947,6 +951,30 @@ __global__ __launch_bounds__(kWsThreads) void hidden_wsum_chunk_kernel(const Wsu
     }
 }
 
+template <bool BF16, int MT>
+__global__ __launch_bounds__(kWsThreads) void hidden_wsum_chunk_kernel(const WsumArgs g) {
+  hidden_wsum_chunk_body<BF16, MT>(g);
+}
+
+// The same launch with the K/V-cached sequences of the step on board: slices z < ws_z of the grid are the chunks
+// above; the workgroups of the slices behind them take the (head group, sequence) items of a paged decode
+// attention's group path, one each, in the grid's linear order.  The chunk workgroups are few and wait on memory
+// most of their time; the attention's workgroups land on compute units that would have been idle, and the step
+// has one launch less on its critical path.  Same code as paged_decode_group_kernel, so the same bits.
+template <bool BF16, int MT>
+__global__ __launch_bounds__(kWsThreads) void hidden_wsum_chunk_and_paged_kernel(const WsumArgs g, const AttnArgs a,
+                                                                                 const int ws_z, const int head_groups,
+                                                                                 const int items) {
+  if ((int)blockIdx.z < ws_z) {
+    hidden_wsum_chunk_body<BF16, MT>(g);
+    return;
+  }
+  const int id = (((int)blockIdx.z - ws_z) * (int)gridDim.y + (int)blockIdx.y) * (int)gridDim.x + (int)blockIdx.x;
+  if (id >= items) return;
+  paged_decode_group_body<BF16 ? APS_BF16 : APS_F16, BF16 ? KV_BF16 : KV_F16, kFusedHeadSize, 1, APS_DEPTH_F16,
+                          kWsWaves>(a, id % head_groups, id / head_groups);
+}
+
 // ctx[z][h][n] = sum_p w_p * partial[p][z][h][n] / sum_p w_p * l_p with w_p = 2^(m_p - max_p m_p): the partitions
 // of a sequence put on one scale, added in the order of the partitions, 4 columns per thread.
 template <bool BF16>
@@ -1079,14 +1107,18 @@ int64_t aps_absorbed_attention_workspace_bytes(int64_t n_seqs, int64_t max_len, 
   return make_plan(n_seqs, max_len, num_heads, (int64_t)num_heads * head_size).total;
 }
 
-int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_rows, int64_t num_q_rows,
-                           const void* paged_cache, int64_t slot_stride, int64_t num_slots,
-                           const int64_t* hidden_slots, const int64_t* seq_start, int64_t n_seqs, int64_t max_len,
-                           const void* w_k, const void* w_v, const void* b_v, int64_t w_stride, int num_heads,
-                           int head_size, float softmax_scale, void* out, int64_t out_stride, int64_t out_rows,
-                           int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream) {
+// kv_job (nullable): the paged decode attention of the step's K/V-cached sequences, launched here as well
+static int hybrid_attention_impl(const PagedJob* kv_job, const void* q, int64_t q_stride, const int64_t* seq_rows,
+                                 int64_t num_q_rows, const void* paged_cache, int64_t slot_stride, int64_t num_slots,
+                                 const int64_t* hidden_slots, const int64_t* seq_start, int64_t n_seqs,
+                                 int64_t max_len, const void* w_k, const void* w_v, const void* b_v, int64_t w_stride,
+                                 int num_heads, int head_size, float softmax_scale, void* out, int64_t out_stride,
+                                 int64_t out_rows, int dtype, void* workspace, int64_t workspace_bytes,
+                                 aps_stream_t stream) {
   if (n_seqs < 0 || max_len < 0 || num_heads <= 0 || head_size <= 0) return APS_ERR_INVALID_ARG;
-  if (n_seqs == 0) return APS_OK;
+  if (kv_job && (kv_job->magic != kPagedJobMagic || kv_job->batch < 0)) return APS_ERR_INVALID_ARG;
+  if (kv_job && kv_job->batch == 0) kv_job = nullptr;
+  if (n_seqs == 0) return kv_job ? aps_attention_job_launch(kv_job, stream) : APS_OK;
   if (!q || !seq_rows || !paged_cache || !hidden_slots || !seq_start || !w_k || !w_v || !out || !workspace)
     return APS_ERR_INVALID_ARG;
   if (dtype != APS_F16 && dtype != APS_BF16) return APS_ERR_UNSUPPORTED;
@@ -1103,6 +1135,16 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
   if (workspace_bytes < p.total) return APS_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
   const bool bf16 = dtype == APS_BF16;
+  // The job's workgroups can ride in the launch of the chunked weighted sum when that launch runs the kernel the
+  // job would have run: group path without a ranking launch of its own, 16-bit cache of the queries' dtype,
+  // one head per wavefront at the head size the combined kernel is built for.
+  const bool ride = kv_job && p.chunked && kWsWaves == kMaxGroupWaves && APS_HPW_F16 == 1 && kv_job->plan.group &&
+                    !kv_job->plan.order_scratch && kv_job->head_size == kFusedHeadSize &&
+                    kv_job->kv_dtype == kv_job->q_dtype && kv_job->q_dtype == dtype;
+  if (kv_job && !ride) {
+    const int st = aps_attention_job_launch(kv_job, stream);
+    if (st != APS_OK) return st;
+  }
   char* ws = (char*)workspace;
   char* qt = ws + p.off_qt;
   float* sc = (float*)(ws + p.off_s);
@@ -1224,7 +1266,25 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
   }
 #define APS_LAUNCH_WSUM(B) \
   if (p.chunked) { APS_LAUNCH_WSUM_K(hidden_wsum_chunk_kernel, B) } else { APS_LAUNCH_WSUM_K(hidden_wsum_kernel, B) }
-    if (bf16) { APS_LAUNCH_WSUM(true) } else { APS_LAUNCH_WSUM(false) }
+#define APS_LAUNCH_WSUM_RIDE(B)                                                                                    \
+  switch (mt) {                                                                                                    \
+    case 1: APS_LAUNCH((hidden_wsum_chunk_and_paged_kernel<B, 1>), rgrid, dim3(kWsThreads), 0, s, g, kv_job->a,    \
+                       (int)grid.z, head_groups, (int)items); break;                                               \
+    case 2: APS_LAUNCH((hidden_wsum_chunk_and_paged_kernel<B, 2>), rgrid, dim3(kWsThreads), 0, s, g, kv_job->a,    \
+                       (int)grid.z, head_groups, (int)items); break;                                               \
+    default: APS_LAUNCH((hidden_wsum_chunk_and_paged_kernel<B, 3>), rgrid, dim3(kWsThreads), 0, s, g, kv_job->a,   \
+                        (int)grid.z, head_groups, (int)items); break;                                              \
+  }
+    if (ride) {   // slices of the grid behind the chunks hold the attention's (head group, sequence) items
+      const int head_groups = kv_job->a.num_heads;
+      const int64_t items = (int64_t)head_groups * kv_job->batch;
+      const int64_t per_slice = (int64_t)grid.x * grid.y;
+      const int64_t slices = (items + per_slice - 1) / per_slice;
+      if (grid.z + slices > 65535) return APS_ERR_UNSUPPORTED;
+      const dim3 rgrid(grid.x, grid.y, (unsigned)(grid.z + slices));
+      if (bf16) { APS_LAUNCH_WSUM_RIDE(true) } else { APS_LAUNCH_WSUM_RIDE(false) }
+    } else if (bf16) { APS_LAUNCH_WSUM(true) } else { APS_LAUNCH_WSUM(false) }
+#undef APS_LAUNCH_WSUM_RIDE
 #undef APS_LAUNCH_WSUM
 #undef APS_LAUNCH_WSUM_K
     int st = launch_status();
@@ -1280,6 +1340,32 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
     if (e != hipSuccess) return (int)e;
     return launch_status();
   }
+}
+
+
+int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_rows, int64_t num_q_rows,
+                           const void* paged_cache, int64_t slot_stride, int64_t num_slots,
+                           const int64_t* hidden_slots, const int64_t* seq_start, int64_t n_seqs, int64_t max_len,
+                           const void* w_k, const void* w_v, const void* b_v, int64_t w_stride, int num_heads,
+                           int head_size, float softmax_scale, void* out, int64_t out_stride, int64_t out_rows,
+                           int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream) {
+  return hybrid_attention_impl(nullptr, q, q_stride, seq_rows, num_q_rows, paged_cache, slot_stride, num_slots,
+                               hidden_slots, seq_start, n_seqs, max_len, w_k, w_v, b_v, w_stride, num_heads, head_size,
+                               softmax_scale, out, out_stride, out_rows, dtype, workspace, workspace_bytes, stream);
+}
+
+int aps_hybrid_decode_attention(const void* kv_job, const void* q, int64_t q_stride, const int64_t* seq_rows,
+                                int64_t num_q_rows, const void* paged_cache, int64_t slot_stride, int64_t num_slots,
+                                const int64_t* hidden_slots, const int64_t* seq_start, int64_t n_seqs,
+                                int64_t max_len, const void* w_k, const void* w_v, const void* b_v, int64_t w_stride,
+                                int num_heads, int head_size, float softmax_scale, void* out, int64_t out_stride,
+                                int64_t out_rows, int dtype, void* workspace, int64_t workspace_bytes,
+                                aps_stream_t stream) {
+  if (kv_job && (addr(kv_job) & 7)) return APS_ERR_INVALID_ARG;
+  return hybrid_attention_impl((const PagedJob*)kv_job, q, q_stride, seq_rows, num_q_rows, paged_cache, slot_stride,
+                               num_slots, hidden_slots, seq_start, n_seqs, max_len, w_k, w_v, b_v, w_stride,
+                               num_heads, head_size, softmax_scale, out, out_stride, out_rows, dtype, workspace,
+                               workspace_bytes, stream);
 }
 
 }  // extern "C"

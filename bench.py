@@ -528,8 +528,11 @@ def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile
         if per.get("attention"):
             frac["attention_hbm"] = work["attention_bytes"] / n_prof / per["attention"] / 1e6 / HBM_PEAK_GBS
         if per.get("attention_on_hidden_rows"):
-            frac["attention_on_hidden_rows_hbm"] = (work["hidden_attention_bytes"] / n_prof /
-                                                    per["attention_on_hidden_rows"] / 1e6 / HBM_PEAK_GBS)
+            # (one call attends both kinds of sequence: the K/V rows of the K/V-cached ones count here when
+            # no phase of their own was timed)
+            both = work["hidden_attention_bytes"] + (0 if per.get("attention") else work["attention_bytes"])
+            frac["attention_on_hidden_rows_hbm"] = (both / n_prof / per["attention_on_hidden_rows"] / 1e6 /
+                                                    HBM_PEAK_GBS)
         if per.get("projections"):
             stream = L * (10 if not absorbed else 12) * Hd * Hd * 2      # q, out, fc1, fc2 (and k, v when projected whole)
             frac["projections_hbm"] = stream / per["projections"] / 1e6 / HBM_PEAK_GBS

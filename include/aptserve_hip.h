@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define APS_ABI_VERSION 9
+#define APS_ABI_VERSION 10
 
 typedef void* aps_stream_t; /* a hipStream_t; NULL = the null stream */
 
@@ -298,6 +298,32 @@ int aps_paged_decode_attention_static(
     int partition_size, float softmax_scale, int q_dtype, int kv_dtype,
     float k_scale, float v_scale, aps_stream_t stream);
 
+/* A call of aps_paged_decode_attention that is checked and planned now and
+ * launched later: the job (APS_ATTENTION_JOB_BYTES of host memory that the
+ * caller owns, 8-byte aligned, opaque) records the arguments, the partitioning
+ * and the kernel that the call would have launched.  Same arguments, checks
+ * and status codes as aps_paged_decode_attention; nothing is enqueued.
+ * aps_attention_job_launch launches a job by itself, with the results of the
+ * direct call bit for bit; aps_hybrid_decode_attention takes one as the K/V-
+ * cached half of a decode step's attention.  The device memory the arguments
+ * point to (workspace included) must be valid when the job is launched; a job
+ * may be launched any number of times.  ref: the same call sites as
+ * aps_paged_decode_attention (attention/backends/aptserve_flash_attn.py:452-461,
+ * :464-473). */
+#define APS_ATTENTION_JOB_BYTES 320
+int aps_paged_decode_attention_job(
+    void* job, int64_t job_bytes, void* out, const void* q,
+    const void* k_cache, const void* v_cache, const void* ws_k_cache,
+    const void* ws_v_cache, const int32_t* block_tables,
+    const uint8_t* block_types, const int32_t* seq_lens, int64_t batch,
+    int num_heads, int head_size, int block_size, int64_t table_width,
+    int64_t table_stride, int64_t types_stride, int64_t q_stride,
+    int64_t out_stride, int64_t cache_block_stride, int64_t num_cache_blocks,
+    int64_t ws_block_stride, int64_t num_ws_blocks, int64_t max_seq_len,
+    int partition_size, float softmax_scale, int q_dtype, int kv_dtype,
+    float k_scale, float v_scale, void* workspace, int64_t workspace_bytes);
+int aps_attention_job_launch(const void* job, aps_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Prompt-step attention on freshly projected q/k/v (no cache read).
  * ref: third-party vllm_flash_attn.flash_attn_varlen_func with causal=True as
@@ -541,6 +567,29 @@ int aps_absorbed_attention(
     const void* b_v, int64_t w_stride, int num_heads, int head_size,
     float softmax_scale, void* out, int64_t out_stride, int64_t out_rows,
     int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream);
+
+/* The attention of a decode step over both kinds of sequence, as one call:
+ * aps_absorbed_attention for the hidden-cached sequences (same arguments,
+ * same results) and, for the K/V-cached ones, the paged decode attention that
+ * kv_job (nullable; from aps_paged_decode_attention_job) describes, with the
+ * results of launching that job by itself.  ref: the reference attends both
+ * kinds in one flash_attn_with_kvcache call over the shared cache
+ * (attention/backends/aptserve_flash_attn.py:464-473) after re-projecting the
+ * hidden-cached ones.  The two halves are independent (they write different
+ * rows of out), so the library is free to overlap them: for a small batch
+ * whose K/V-cached sequences fit the one-workgroup-per-sequence path (f16 /
+ * bf16 cache, head size 128) the job's workgroups ride in the launch of the
+ * weighted sum over the hidden rows, which leaves most compute units idle;
+ * otherwise the job is launched first, by itself.  n_seqs == 0: only the job. */
+int aps_hybrid_decode_attention(
+    const void* kv_job, const void* q, int64_t q_stride,
+    const int64_t* seq_rows, int64_t num_q_rows, const void* paged_cache,
+    int64_t slot_stride, int64_t num_slots, const int64_t* hidden_slots,
+    const int64_t* seq_start, int64_t n_seqs, int64_t max_len, const void* w_k,
+    const void* w_v, const void* b_v, int64_t w_stride, int num_heads,
+    int head_size, float softmax_scale, void* out, int64_t out_stride,
+    int64_t out_rows, int dtype, void* workspace, int64_t workspace_bytes,
+    aps_stream_t stream);
 
 /* Residual add and LayerNorm of a decoder layer in one launch.
  * ref: model_executor/models/aptserve_opt.py:186-211 (OPTDecoderLayer.forward:
