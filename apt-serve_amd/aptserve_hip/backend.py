@@ -291,8 +291,13 @@ class HybridOPTAttention:
         a = self.attn
         n_kv = md.num_decode_tokens - md.num_hidden_cache_tokens
         attn_output = torch.empty_like(hidden_states)
-        one_write = n_kv and not a.fp8 and md.kv_cache_use_input is not None and md.new_token_slot is not None
-        if not one_write:      # the newest hidden row of every hidden-cached sequence joins its cache
+        # The step's cache writes - the newest hidden row of every hidden-cached sequence, the newest K and V rows of
+        # the others - are planned here and launched by the attention call (beside the absorbed queries when the
+        # step is small).  An fp8 K/V cache takes the quantising write instead, and the hidden rows a launch of
+        # their own.
+        one_write = not a.fp8 and (not n_kv or (md.kv_cache_use_input is not None and md.new_token_slot is not None))
+        store_job = None
+        if not one_write:
             with phase("write"):
                 ops.hidden_to_cache(hidden_states, hidden_cache, md.slot_mapping, md.hidden_cache_use_input,
                                     md.hidden_cache_store_tot)
@@ -300,12 +305,13 @@ class HybridOPTAttention:
             with phase("projections"):
                 qkv, _ = self.qkv_proj(hidden_states)
                 q, k, v = qkv.chunk(chunks=3, dim=-1)
-            with phase("write"):
-                if one_write:  # ... in the same launch as the newest K/V rows of the K/V-cached sequences
-                    ops.decode_step_cache_ops(None, hidden_states, hidden_cache, None, md.slot_mapping,
-                                              md.hidden_cache_use_input, md.hidden_cache_store_tot, k, v,
-                                              md.kv_cache_use_input, md.new_token_slot, kv_cache=kv_cache)
-                else:
+            if one_write:
+                store_job = ops.decode_step_cache_ops(None, hidden_states, hidden_cache, None, md.slot_mapping,
+                                                      md.hidden_cache_use_input, md.hidden_cache_store_tot, k, v,
+                                                      md.kv_cache_use_input, md.new_token_slot,
+                                                      kv_cache=kv_cache, as_job=True)
+            else:
+                with phase("write"):
                     ops.reshape_and_cache_flash(k, v, kv_cache[0], kv_cache[1], md.new_token_slot, a.kv_cache_dtype,
                                                 a.k_scale, a.v_scale, token_idx=md.kv_cache_use_input)
             # planned here, launched by the attention on the hidden rows (the two halves write different rows of
@@ -318,10 +324,15 @@ class HybridOPTAttention:
             kv_job = None
             with phase("projections"):
                 q, _ = self.qkv_proj(hidden_states, q_only=True, kv_only=False)
+            if one_write:
+                store_job = ops.decode_step_cache_ops(None, hidden_states, hidden_cache, None, md.slot_mapping,
+                                                      md.hidden_cache_use_input, md.hidden_cache_store_tot, None, None,
+                                                      None, None, as_job=True)
         with phase("attention_on_hidden_rows"):
             ops.absorbed_hidden_attention(q, hidden_cache, md.hidden_slots, md.hidden_seq_start,
                                           md.hidden_cache_use_input, md.max_hidden_seq_len, w[s:2 * s], w[2 * s:],
-                                          None if b is None else b[2 * s:], self.scaling, attn_output, kv_job=kv_job)
+                                          None if b is None else b[2 * s:], self.scaling, attn_output, kv_job=kv_job,
+                                          store_job=store_job)
         with phase("projections"):
             return ops.linear_nt(attn_output, self.out_weight, self.out_bias)
 

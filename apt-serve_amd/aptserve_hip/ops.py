@@ -189,9 +189,29 @@ def gather_hidden_rows(holder, hidden_states, paged_cache, holder_src, slot_mapp
     _lib.check(st, "gather_hidden_rows")
 
 
+APS_CACHE_JOB_BYTES = 320
+
+
+class CacheJob:
+    """A decode step's planned, not yet launched cache writes (``decode_step_cache_ops(..., as_job=True)``):
+    opaque host bytes that the library wrote, and the tensors the launch will touch, kept alive."""
+
+    def __init__(self, anchor, tensors):
+        self._buf = (ctypes.c_uint64 * (APS_CACHE_JOB_BYTES // 8))()
+        self.address = ctypes.addressof(self._buf)
+        self._anchor = anchor
+        self._tensors = tensors
+
+    def launch(self) -> None:
+        """Launch the job by itself on the current stream of its device."""
+        with _on(self._anchor.device):
+            st = _lib.load().aps_cache_job_launch(self.address, _stream(self._anchor))
+        _lib.check(st, "cache_job_launch")
+
+
 def decode_step_cache_ops(holder, hidden_states, paged_cache, holder_src, slot_mapping, hidden_cache_use_input,
                           hidden_cache_store_tot, key, value, kv_cache_use_input, new_token_slot,
-                          kv_cache=None) -> None:
+                          kv_cache=None, as_job: bool = False):
     """The cache traffic of one decode layer in one launch: ``gather_hidden_rows`` (store of the newest hidden
     rows, holder assembly: additional_designs/model_executor/models/aptserve_opt.py:108-121) and the write of
     the newest K/V rows of the K/V-cached sequences into the two planes of ``paged_cache``
@@ -199,9 +219,15 @@ def decode_step_cache_ops(holder, hidden_states, paged_cache, holder_src, slot_m
     ``key`` / ``value`` ``[batch, H*D]`` or ``[batch, H, D]``; ``kv_cache_use_input`` and ``new_token_slot``
     from the metadata builder.  Same bytes in the cache and the holder as the two separate calls.
     ``holder`` (and ``holder_src``) may be ``None``: the stores alone, for a data flow that assembles no holder.
-    ``kv_cache``: the K/V planes when they are not ``paged_cache`` (a separate hidden-row cache)."""
+    ``key`` and ``value`` may be ``None``: a step without K/V-cached sequences.
+    ``kv_cache``: the K/V planes when they are not ``paged_cache`` (a separate hidden-row cache).
+    ``as_job=True`` checks and plans the call but launches nothing: the :class:`CacheJob` that comes back is
+    launched later, by itself or as the stores that precede :func:`absorbed_hidden_attention`."""
     dev = hidden_states.device
-    for n, t in (("hidden_states", hidden_states), ("paged_cache", paged_cache), ("key", key), ("value", value)):
+    no_kv = key is None
+    _need((value is None) == no_kv, "key and value come together")
+    for n, t in (("hidden_states", hidden_states), ("paged_cache", paged_cache)) + (
+            () if no_kv else (("key", key), ("value", value))):
         _check_data(n, t, dev)
     _need(hidden_states.dim() == 2, "hidden_states must be 2-D")
     width = hidden_states.size(1)
@@ -215,32 +241,42 @@ def decode_step_cache_ops(holder, hidden_states, paged_cache, holder_src, slot_m
         _need(holder_src.numel() == n_rows, "holder_src must have one entry per holder row")
     kvc = paged_cache if kv_cache is None else kv_cache
     _check_data("kv_cache", kvc, dev)
-    _need(hidden_states.dtype == paged_cache.dtype == kvc.dtype == key.dtype == value.dtype, "dtypes differ")
+    _need(hidden_states.dtype == paged_cache.dtype == kvc.dtype, "dtypes differ")
+    _need(no_kv or hidden_states.dtype == key.dtype == value.dtype, "dtypes differ")
     for c in (paged_cache, kvc):
         _check_paged(c, width)
         _need(c.size(0) == 2 and c.size(3) * c.size(4) == width,
               "a cache must be (2, num_blocks, block_size, heads, head_dim) with heads*head_dim == hidden width")
-    key = _as_thd("key", key, kvc.size(3), kvc.size(4))
-    value = _as_thd("value", value, kvc.size(3), kvc.size(4))
     B = hidden_states.size(0)
-    _need(key.size(0) == B and value.size(0) == B, "one key / value row per sequence expected")
     for n, t in (("slot_mapping", slot_mapping), ("hidden_cache_use_input", hidden_cache_use_input),
-                 ("hidden_cache_store_tot", hidden_cache_store_tot), ("kv_cache_use_input", kv_cache_use_input),
-                 ("new_token_slot", new_token_slot)):
+                 ("hidden_cache_store_tot", hidden_cache_store_tot)):
         _check_index(n, t, dev)
     _need(hidden_cache_use_input.numel() == hidden_cache_store_tot.numel(), "store index lengths differ")
-    _need(new_token_slot.numel() == B, "new_token_slot must have one entry per sequence")
+    if not no_kv:
+        key = _as_thd("key", key, kvc.size(3), kvc.size(4))
+        value = _as_thd("value", value, kvc.size(3), kvc.size(4))
+        _need(key.size(0) == B and value.size(0) == B, "one key / value row per sequence expected")
+        for n, t in (("kv_cache_use_input", kv_cache_use_input), ("new_token_slot", new_token_slot)):
+            _check_index(n, t, dev)
+        _need(new_token_slot.numel() == B, "new_token_slot must have one entry per sequence")
     slot_stride = paged_cache.stride(2)
-    with _on(dev):
-        st = _lib.load().aps_decode_step_cache_ops(
-            None if holder is None else _ptr(holder), hidden_states.data_ptr(), paged_cache.data_ptr(),
+    args = (None if holder is None else _ptr(holder), hidden_states.data_ptr(), paged_cache.data_ptr(),
             None if holder is None else _ptr(holder_src), n_rows,
             _ptr(slot_mapping), _ptr(hidden_cache_use_input), _ptr(hidden_cache_store_tot),
             hidden_cache_store_tot.numel(), B, width, 0 if holder is None else holder.stride(0), hidden_states.stride(0),
-            slot_stride, paged_cache.numel() // slot_stride, key.data_ptr(), value.data_ptr(), kvc[0].data_ptr(),
-            kvc[1].data_ptr(), _ptr(kv_cache_use_input), _ptr(new_token_slot), kv_cache_use_input.numel(),
-            key.stride(0), value.stride(0), kvc.size(2), kvc.stride(1), kvc.size(1),
-            hidden_states.element_size(), _stream(hidden_states))
+            slot_stride, paged_cache.numel() // slot_stride) + (
+        (None, None, None, None, None, None, 0, 0, 0) if no_kv else
+        (key.data_ptr(), value.data_ptr(), kvc[0].data_ptr(), kvc[1].data_ptr(), _ptr(kv_cache_use_input),
+         _ptr(new_token_slot), kv_cache_use_input.numel(), key.stride(0), value.stride(0))) + (
+        kvc.size(2), kvc.stride(1), kvc.size(1), hidden_states.element_size())
+    if as_job:
+        job = CacheJob(hidden_states, (holder, paged_cache, holder_src, slot_mapping, hidden_cache_use_input,
+                                       hidden_cache_store_tot, key, value, kvc, kv_cache_use_input, new_token_slot))
+        _lib.check(_lib.load().aps_decode_step_cache_ops_job(job.address, APS_CACHE_JOB_BYTES, *args),
+                   "decode_step_cache_ops_job")
+        return job
+    with _on(dev):
+        st = _lib.load().aps_decode_step_cache_ops(*args, _stream(hidden_states))
     _lib.check(st, "decode_step_cache_ops")
 
 
@@ -837,7 +873,8 @@ def flash_attn_varlen_func(q, k, v, cu_seqlens_q=None, cu_seqlens_k=None, max_se
 # ------------------------------------------------------------------ attention on cached hidden rows
 
 def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, seq_rows, max_len, w_k, w_v, b_v,
-                              softmax_scale, out, workspace=None, kv_job: Optional["AttentionJob"] = None):
+                              softmax_scale, out, workspace=None, kv_job: Optional["AttentionJob"] = None,
+                              store_job: Optional["CacheJob"] = None):
     """Decode attention of the hidden-cached sequences of a batch, computed on their cached hidden
     rows with the K/V projection weights absorbed into the query and the output:
     ``s[h,t] = scale <W_k[h]^T q[h], hidden_t>``, ``out[h] = W_v[h] (sum_t p[h,t] hidden_t) + b_v[h]``.
@@ -855,7 +892,10 @@ def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, se
     ``kv_job``: the paged decode attention of the batch's K/V-cached sequences
     (``paged_decode_attention(..., as_job=True)``), launched by this call as well — inside the
     launch of the weighted sum over the hidden rows when the batch is small enough for that, by
-    itself otherwise; the results are those of launching the job alone."""
+    itself otherwise; the results are those of launching the job alone.  ``store_job``: the step's
+    cache writes (``decode_step_cache_ops(..., as_job=True)``), complete before any cache row is
+    read: beside the absorbed queries in one launch when they fit there, first and by themselves
+    otherwise."""
     dev = q.device
     for n, t in (("q", q), ("paged_cache", paged_cache), ("w_k", w_k), ("w_v", w_v), ("out", out)):
         _check_data(n, t, dev)
@@ -878,6 +918,8 @@ def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, se
     n_seqs = seq_rows.numel()
     _need(hidden_seq_start.numel() == n_seqs + 1, "hidden_seq_start needs one entry per sequence plus one")
     if n_seqs == 0:
+        if store_job is not None:
+            store_job.launch()
         if kv_job is not None:
             kv_job.launch()
         return out
@@ -887,7 +929,7 @@ def absorbed_hidden_attention(q, paged_cache, hidden_slots, hidden_seq_start, se
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)      # scratch is host-side plumbing
     with _on(dev):
         st = lib.aps_hybrid_decode_attention(
-            None if kv_job is None else kv_job.address, q.data_ptr(), q.stride(0), seq_rows.data_ptr(), q.size(0), paged_cache.data_ptr(), paged_cache.stride(2),
+            None if store_job is None else store_job.address, None if kv_job is None else kv_job.address, q.data_ptr(), q.stride(0), seq_rows.data_ptr(), q.size(0), paged_cache.data_ptr(), paged_cache.stride(2),
             paged_cache.numel() // paged_cache.stride(2), hidden_slots.data_ptr(), hidden_seq_start.data_ptr(),
             n_seqs, int(max_len), w_k.data_ptr(), w_v.data_ptr(), None if b_v is None else b_v.data_ptr(),
             w_k.stride(0), heads, head_size, float(softmax_scale), out.data_ptr(), out.stride(0), out.size(0),

@@ -7,14 +7,23 @@
 //     out[h]  = W_v[h] (sum_t p[h][t] h_t) + b_v[h]
 // so the hidden rows are read twice (scores, then the weighted sum) and the projections shrink to
 // products with one row per sequence and head:
-//   1. qt[s][h][:]  = scale*log2(e) * W_k[h]^T q[s][h]            nn_few_rows_kernel (B = rows of W_k)
-//   2. S[s][h][t]   = <qt[s][h], h_t>                               seq_plan_kernel (work list of the ragged
-//                                                                   batch), hidden_scores_kernel (paged rows)
-//   3. P[s][h][:]   = softmax_t, 16-bit, zero padded to 32 tokens   softmax_rows_kernel
-//   4. ctx[s][h][:] = sum_t P[s][h][t] h_t                          nn_few_rows_kernel (B = paged rows)
-//   5. out[s][h*D+d] = <W_v[h*D+d], ctx[s][h]> + b_v                head_proj_kernel; up to 16 sequences: the
-//                                                                   weight-streaming kernels of the projection
-//                                                                   file, x chosen per head
+//   1. qt[s][h][:]  = scale*log2(e) * W_k[h]^T q[s][h]     query_image_kernel (a head's slab of W_k in registers; one
+//                                                            extra workgroup plans the ragged batch for the kernels
+//                                                            below); heads wider than 128: nn_few_rows_kernel and
+//                                                            seq_plan_kernel
+//   2. S[s][h][t]   = <qt[s][h], h_t>  (fp32)               hidden_scores_kernel: tiles of 128 cached rows through
+//                                                            the row-streaming MFMA core, K in parts for small
+//                                                            batches (score_parts_sum_kernel adds them)
+//   3. ctx[s][h][:] = sum_t softmax_t(S[s][h])[t] h_t        hidden_wsum_kernel: one pass over the rows with the
+//                                                            online softmax inside (long sequences in partitions);
+//                                                            few cached rows in all: hidden_wsum_chunk_kernel, one
+//                                                            96-token chunk per workgroup; wsum_combine_kernel
+//                                                            merges partitions / chunks
+//   4. out[s][h*D+d] = <W_v[h*D+d], ctx[s][h]> + b_v         head_proj_kernel; up to 16 sequences: the
+//                                                            weight-streaming kernels of the projection file, x
+//                                                            chosen per head
+// A decode step's other work can share these launches (aps_hybrid_decode_attention): the step's cache writes
+// ride beside the absorbed queries, the paged attention of the K/V-cached sequences beside the chunked sum.
 // Per cached token and layer that is 2 x Hd x 2 bytes of HBM reads and ~4*H*Hd flops, against a
 // gather, a 4*Hd*Hd-flop GEMM, a cache write and an attention read for the re-projection flow.
 #include <type_traits>
@@ -22,6 +31,7 @@
 #include "aps_common.h"
 #include "mfma_common.h"
 #include "paged_decode_core.h"
+#include "row_mover_core.h"
 #include "row_stream_core.h"
 
 // the per-head value projection lives with the other weight-streaming kernels
@@ -34,6 +44,8 @@ __attribute__((visibility("hidden"))) int64_t aps_internal_headwise_workspace_by
                                                                                    int head_rows);
 // a planned paged decode attention, launched by itself (the attention launcher's translation unit)
 extern "C" int aps_attention_job_launch(const void* job, aps_stream_t stream);
+// a decode step's planned cache writes, launched by themselves (the cache operators' translation unit)
+extern "C" int aps_cache_job_launch(const void* job, aps_stream_t stream);
 
 namespace aps {
 namespace {
@@ -262,18 +274,36 @@ struct QImageArgs {
   u32x4* zero_row; int zero_vecs;
 };
 
-template <bool BF16, int KS>
-__global__ __launch_bounds__(256) void query_image_kernel(const QImageArgs g) {
-  if ((int)blockIdx.y == g.heads) {
-    if (blockIdx.x == 0)
+// The rows of the grid in front of the heads' rows hold the launch's other work, one workgroup each in the
+// grid's linear order: first the plan, then (a launch that has a decode step's cache writes on board) the row
+// mover's workgroups.  Those writes touch no operand of this kernel; they only have to be complete before the
+// next launch reads the caches, and their short index chains run under the weight stream instead of in a launch
+// of their own.
+struct StoreRider {
+  DecodeStepOp op;
+  int64_t n_items;
+  uint32_t segs_per_row, row_bytes, items_per_y, blocks;
+};
+
+template <bool BF16, int KS, bool STORES>
+__device__ __forceinline__ void query_image_body(const QImageArgs& g, const StoreRider* rider) {
+  const int aux_rows = (int)gridDim.y - g.heads;
+  if ((int)blockIdx.y < aux_rows) {
+    const uint32_t id = blockIdx.y * gridDim.x + blockIdx.x;
+    if (id == 0) {
       plan_ragged_batch(g.row_start, g.n_seqs, g.tile_tokens, g.tile_start, g.order, g.zero_row, g.zero_vecs);
+    } else if constexpr (STORES) {
+      if (id - 1 < rider->blocks)
+        row_mover_body<16, DecodeStepOp::kChunks, DecodeStepOp>(rider->op, rider->n_items, rider->segs_per_row,
+                                                                rider->row_bytes, rider->items_per_y, id - 1, 0);
+    }
     return;
   }
   constexpr int D = KS * 32;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int g4 = lane >> 4, c = lane & 15;
-  const int h = blockIdx.y;
+  const int h = (int)blockIdx.y - aux_rows;
   const int64_t col0 = (int64_t)blockIdx.x * 512 + wave * 128 + 8 * c;
   const bool col_ok = col0 < g.hidden;
   const char* b_col = g.w + (col_ok ? col0 : 0) * 2 + (int64_t)h * D * g.w_stride_b;
@@ -346,6 +376,16 @@ __global__ __launch_bounds__(256) void query_image_kernel(const QImageArgs g) {
       }
     }
   }
+}
+
+template <bool BF16, int KS>
+__global__ __launch_bounds__(256) void query_image_kernel(const QImageArgs g) {
+  query_image_body<BF16, KS, false>(g, nullptr);
+}
+static_assert(kMaxThreads == 256, "the row mover's workgroups have the size of this kernel's");
+template <bool BF16, int KS>
+__global__ __launch_bounds__(256) void query_image_and_stores_kernel(const QImageArgs g, const StoreRider rider) {
+  query_image_body<BF16, KS, true>(g, &rider);
 }
 
 template <bool BF16, int NHT>
@@ -1108,7 +1148,7 @@ int64_t aps_absorbed_attention_workspace_bytes(int64_t n_seqs, int64_t max_len, 
 }
 
 // kv_job (nullable): the paged decode attention of the step's K/V-cached sequences, launched here as well
-static int hybrid_attention_impl(const PagedJob* kv_job, const void* q, int64_t q_stride, const int64_t* seq_rows,
+static int hybrid_attention_impl(const StoreJob* store_job, const PagedJob* kv_job, const void* q, int64_t q_stride, const int64_t* seq_rows,
                                  int64_t num_q_rows, const void* paged_cache, int64_t slot_stride, int64_t num_slots,
                                  const int64_t* hidden_slots, const int64_t* seq_start, int64_t n_seqs,
                                  int64_t max_len, const void* w_k, const void* w_v, const void* b_v, int64_t w_stride,
@@ -1118,7 +1158,12 @@ static int hybrid_attention_impl(const PagedJob* kv_job, const void* q, int64_t 
   if (n_seqs < 0 || max_len < 0 || num_heads <= 0 || head_size <= 0) return APS_ERR_INVALID_ARG;
   if (kv_job && (kv_job->magic != kPagedJobMagic || kv_job->batch < 0)) return APS_ERR_INVALID_ARG;
   if (kv_job && kv_job->batch == 0) kv_job = nullptr;
-  if (n_seqs == 0) return kv_job ? aps_attention_job_launch(kv_job, stream) : APS_OK;
+  if (store_job && (store_job->magic != kStoreJobMagic || store_job->n_items < 0)) return APS_ERR_INVALID_ARG;
+  if (store_job && store_job->n_items == 0) store_job = nullptr;
+  if (n_seqs == 0) {
+    const int st = store_job ? aps_cache_job_launch(store_job, stream) : APS_OK;
+    return st != APS_OK || !kv_job ? st : aps_attention_job_launch(kv_job, stream);
+  }
   if (!q || !seq_rows || !paged_cache || !hidden_slots || !seq_start || !w_k || !w_v || !out || !workspace)
     return APS_ERR_INVALID_ARG;
   if (dtype != APS_F16 && dtype != APS_BF16) return APS_ERR_UNSUPPORTED;
@@ -1141,8 +1186,16 @@ static int hybrid_attention_impl(const PagedJob* kv_job, const void* q, int64_t 
   const bool ride = kv_job && p.chunked && kWsWaves == kMaxGroupWaves && APS_HPW_F16 == 1 && kv_job->plan.group &&
                     !kv_job->plan.order_scratch && kv_job->head_size == kFusedHeadSize &&
                     kv_job->kv_dtype == kv_job->q_dtype && kv_job->q_dtype == dtype;
-  if (kv_job && !ride) {
-    const int st = aps_attention_job_launch(kv_job, stream);
+  // The stores can ride beside the absorbed queries when that launch is the kernel with the auxiliary rows and
+  // the job is the one-row grid of 16-byte accesses.
+  MoverGrid mg{};
+  bool stores_ride = false;
+  if (store_job && head_size <= 128 && store_job->vb == 16) {
+    mg = mover_grid(store_job->n_items, store_job->row_bytes, 16, DecodeStepOp::kChunks);
+    stores_ride = mg.grid_y == 1 && mg.grid_x <= 4096;
+  }
+  if (store_job && !stores_ride) {
+    const int st = aps_cache_job_launch(store_job, stream);
     if (st != APS_OK) return st;
   }
   char* ws = (char*)workspace;
@@ -1166,7 +1219,10 @@ static int hybrid_attention_impl(const PagedJob* kv_job, const void* q, int64_t 
     g.alpha = softmax_scale * 1.4426950408889634f;
     g.row_start = seq_start; g.tile_tokens = kScTokens; g.tile_start = tiles; g.order = order;
     g.zero_row = (u32x4*)(ws + p.off_zero); g.zero_vecs = (int)(p.zero_bytes / 16);
-    const dim3 grid((unsigned)((hidden + 511) / 512), (unsigned)num_heads + 1);
+    const unsigned gx = (unsigned)((hidden + 511) / 512);
+    // rows in front of the heads: the plan's workgroup and, with the stores on board, the row mover's
+    const unsigned aux = stores_ride ? (unsigned)((1 + mg.grid_x + gx - 1) / gx) : 1u;
+    const dim3 grid(gx, (unsigned)num_heads + aux);
 #define APS_LAUNCH_QI(B)                                                                     \
   switch (head_size / 32) {                                                                  \
     case 1: APS_LAUNCH((query_image_kernel<B, 1>), grid, dim3(256), 0, s, g); break;         \
@@ -1174,7 +1230,19 @@ static int hybrid_attention_impl(const PagedJob* kv_job, const void* q, int64_t 
     case 3: APS_LAUNCH((query_image_kernel<B, 3>), grid, dim3(256), 0, s, g); break;         \
     default: APS_LAUNCH((query_image_kernel<B, 4>), grid, dim3(256), 0, s, g); break;        \
   }
-    if (bf16) { APS_LAUNCH_QI(true) } else { APS_LAUNCH_QI(false) }
+#define APS_LAUNCH_QI_STORES(B)                                                                              \
+  switch (head_size / 32) {                                                                                  \
+    case 1: APS_LAUNCH((query_image_and_stores_kernel<B, 1>), grid, dim3(256), 0, s, g, rider); break;       \
+    case 2: APS_LAUNCH((query_image_and_stores_kernel<B, 2>), grid, dim3(256), 0, s, g, rider); break;       \
+    case 3: APS_LAUNCH((query_image_and_stores_kernel<B, 3>), grid, dim3(256), 0, s, g, rider); break;       \
+    default: APS_LAUNCH((query_image_and_stores_kernel<B, 4>), grid, dim3(256), 0, s, g, rider); break;      \
+  }
+    if (stores_ride) {
+      const StoreRider rider{store_job->op, store_job->n_items, (uint32_t)mg.segs_per_row,
+                             (uint32_t)store_job->row_bytes, (uint32_t)mg.items_per_y, (uint32_t)mg.grid_x};
+      if (bf16) { APS_LAUNCH_QI_STORES(true) } else { APS_LAUNCH_QI_STORES(false) }
+    } else if (bf16) { APS_LAUNCH_QI(true) } else { APS_LAUNCH_QI(false) }
+#undef APS_LAUNCH_QI_STORES
 #undef APS_LAUNCH_QI
     const int st = launch_status();
     if (st != APS_OK) return st;
@@ -1194,6 +1262,11 @@ static int hybrid_attention_impl(const PagedJob* kv_job, const void* q, int64_t 
     APS_LAUNCH(seq_plan_kernel, dim3(1), dim3(256), 0, s, seq_start, (int)n_seqs, kScTokens, tiles, order,
                (u32x4*)(ws + p.off_zero), (int)(p.zero_bytes / 16));
     st = launch_status();
+    if (st != APS_OK) return st;
+  }
+  // (the stores are complete or enqueued by now: an attention job that cannot ride goes here, by itself)
+  if (kv_job && !ride) {
+    const int st = aps_attention_job_launch(kv_job, stream);
     if (st != APS_OK) return st;
   }
   // 2. S[s][h][t] = <qt[s][h], hidden row t of sequence s>
@@ -1349,20 +1422,20 @@ int aps_absorbed_attention(const void* q, int64_t q_stride, const int64_t* seq_r
                            const void* w_k, const void* w_v, const void* b_v, int64_t w_stride, int num_heads,
                            int head_size, float softmax_scale, void* out, int64_t out_stride, int64_t out_rows,
                            int dtype, void* workspace, int64_t workspace_bytes, aps_stream_t stream) {
-  return hybrid_attention_impl(nullptr, q, q_stride, seq_rows, num_q_rows, paged_cache, slot_stride, num_slots,
+  return hybrid_attention_impl(nullptr, nullptr, q, q_stride, seq_rows, num_q_rows, paged_cache, slot_stride, num_slots,
                                hidden_slots, seq_start, n_seqs, max_len, w_k, w_v, b_v, w_stride, num_heads, head_size,
                                softmax_scale, out, out_stride, out_rows, dtype, workspace, workspace_bytes, stream);
 }
 
-int aps_hybrid_decode_attention(const void* kv_job, const void* q, int64_t q_stride, const int64_t* seq_rows,
-                                int64_t num_q_rows, const void* paged_cache, int64_t slot_stride, int64_t num_slots,
+int aps_hybrid_decode_attention(const void* store_job, const void* kv_job, const void* q, int64_t q_stride,
+                                const int64_t* seq_rows, int64_t num_q_rows, const void* paged_cache, int64_t slot_stride, int64_t num_slots,
                                 const int64_t* hidden_slots, const int64_t* seq_start, int64_t n_seqs,
                                 int64_t max_len, const void* w_k, const void* w_v, const void* b_v, int64_t w_stride,
                                 int num_heads, int head_size, float softmax_scale, void* out, int64_t out_stride,
                                 int64_t out_rows, int dtype, void* workspace, int64_t workspace_bytes,
                                 aps_stream_t stream) {
-  if (kv_job && (addr(kv_job) & 7)) return APS_ERR_INVALID_ARG;
-  return hybrid_attention_impl((const PagedJob*)kv_job, q, q_stride, seq_rows, num_q_rows, paged_cache, slot_stride,
+  if ((kv_job && (addr(kv_job) & 7)) || (store_job && (addr(store_job) & 7))) return APS_ERR_INVALID_ARG;
+  return hybrid_attention_impl((const StoreJob*)store_job, (const PagedJob*)kv_job, q, q_stride, seq_rows, num_q_rows, paged_cache, slot_stride,
                                num_slots, hidden_slots, seq_start, n_seqs, max_len, w_k, w_v, b_v, w_stride,
                                num_heads, head_size, softmax_scale, out, out_stride, out_rows, dtype, workspace,
                                workspace_bytes, stream);

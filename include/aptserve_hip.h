@@ -157,6 +157,29 @@ int aps_decode_step_cache_ops(
     int64_t value_stride, int block_size, int64_t block_stride,
     int64_t num_blocks, int elem_size, aps_stream_t stream);
 
+/* A call of aps_decode_step_cache_ops that is checked and planned now and
+ * launched later: the job (APS_CACHE_JOB_BYTES of host memory that the caller
+ * owns, 8-byte aligned, opaque) records the arguments and the shape of the
+ * launch.  Same arguments, checks and status codes as
+ * aps_decode_step_cache_ops (same reference call sites); nothing is enqueued.
+ * aps_cache_job_launch launches a job by itself, with the result of the direct
+ * call; aps_hybrid_decode_attention takes one as the cache writes that precede
+ * a decode step's attention.  The device memory the arguments point to must be
+ * valid when the job is launched. */
+#define APS_CACHE_JOB_BYTES 320
+int aps_decode_step_cache_ops_job(
+    void* job, int64_t job_bytes, void* holder, const void* hidden_states,
+    void* paged_cache, const int64_t* holder_src, int64_t n_rows,
+    const int64_t* slot_mapping, const int64_t* hidden_cache_use_input,
+    const int64_t* hidden_cache_store_tot, int64_t n_store, int64_t num_inputs,
+    int64_t hidden_size, int64_t holder_stride, int64_t hidden_stride,
+    int64_t slot_stride, int64_t num_slots, const void* key, const void* value,
+    void* key_cache, void* value_cache, const int64_t* kv_cache_use_input,
+    const int64_t* new_token_slot, int64_t n_kv, int64_t key_stride,
+    int64_t value_stride, int block_size, int64_t block_stride,
+    int64_t num_blocks, int elem_size);
+int aps_cache_job_launch(const void* job, aps_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * K/V row scatter into [num_blocks, block_size, H, D] caches.
  * ------------------------------------------------------------------------ */
@@ -580,9 +603,17 @@ int aps_absorbed_attention(
  * whose K/V-cached sequences fit the one-workgroup-per-sequence path (f16 /
  * bf16 cache, head size 128) the job's workgroups ride in the launch of the
  * weighted sum over the hidden rows, which leaves most compute units idle;
- * otherwise the job is launched first, by itself.  n_seqs == 0: only the job. */
+ * otherwise the job is launched by itself, after the stores.
+ * store_job (nullable; from aps_decode_step_cache_ops_job): the step's cache
+ * writes, which the reference's attention forward also begins with
+ * (attention/backends/aptserve_flash_attn.py:338-345, after
+ * model_executor/models/aptserve_opt.py:108-111).  They are complete before
+ * either kind of attention reads the caches: inside the launch of the absorbed
+ * queries (which touches no cache) when the job moves 16 bytes per lane in one
+ * grid row and the head size is at most 128, by a launch of their own before
+ * everything else otherwise.  n_seqs == 0: only the jobs, stores first. */
 int aps_hybrid_decode_attention(
-    const void* kv_job, const void* q, int64_t q_stride,
+    const void* store_job, const void* kv_job, const void* q, int64_t q_stride,
     const int64_t* seq_rows, int64_t num_q_rows, const void* paged_cache,
     int64_t slot_stride, int64_t num_slots, const int64_t* hidden_slots,
     const int64_t* seq_start, int64_t n_seqs, int64_t max_len, const void* w_k,

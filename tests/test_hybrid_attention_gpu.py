@@ -68,6 +68,43 @@ def test_one_call_for_both_kinds_of_sequence_equals_the_two_calls(dev, H, D, bat
         assert (alone[hid_rows] == 0).all()          # length 0 in kv_seq_lens: zeros, as in the direct call
 
 
+@pytest.mark.parametrize("H,D,batch,frac,max_len,dtype", [
+    (40, 128, 5, 0.5, 400, torch.float16),      # stores beside the absorbed queries, attention in the chunk launch
+    (40, 128, 7, 0.6, 150, torch.bfloat16),
+    (12, 64, 6, 0.5, 200, torch.float16),       # stores ride, the attention job is launched behind them
+    (4, 256, 4, 0.5, 100, torch.float16),       # wide heads: both jobs by themselves, stores first
+    (40, 128, 60, 0.5, 300, torch.float16),     # a large batch: stores ride, nothing else does
+])
+def test_step_stores_and_both_attentions_as_one_call_equal_the_three_calls(dev, H, D, batch, frac, max_len, dtype):
+    """The newest K/V rows and hidden rows of the step are written by the same call that then reads them: the
+    caches and the attention output must equal those of store, paged attention and hidden-row attention called one
+    after the other."""
+    b, md, cache, w, b_v, q = _batch(dev, H, D, batch, frac, max_len, 512, dtype, 21)
+    B, Hd = len(b.seq_lens), H * D
+    hs, k, v = (randn((B, Hd), 30 + i, dtype).to(dev) for i in range(3))
+
+    def stores(c, **kw):
+        return ops.decode_step_cache_ops(None, hs, c, None, md.slot_mapping, md.hidden_cache_use_input,
+                                         md.hidden_cache_store_tot, k, v, md.kv_cache_use_input, md.new_token_slot, **kw)
+
+    cache_a, want = cache.clone(), torch.full_like(q, 7.0)
+    stores(cache_a)
+    _paged(q, cache_a, md, H, D, want)
+    _hidden(q, cache_a, md, w, b_v, D, want)
+    assert not torch.equal(cache_a, cache)
+    cache_b, got = cache.clone(), torch.full_like(q, 7.0)
+    store_job = stores(cache_b, as_job=True)
+    kv_job = _paged(q, cache_b, md, H, D, got, as_job=True)
+    torch.cuda.synchronize()
+    assert torch.equal(cache_b, cache) and (got == 7).all()      # planning launches nothing
+    _hidden(q, cache_b, md, w, b_v, D, got, kv_job=kv_job, store_job=store_job)
+    assert torch.equal(cache_b, cache_a) and torch.equal(got, want)
+    # the store job by itself
+    cache_c = cache.clone()
+    stores(cache_c, as_job=True).launch()
+    assert torch.equal(cache_c, cache_a)
+
+
 def test_job_of_split_sequences_and_of_an_fp8_cache_equals_the_direct_call(dev):
     """Long sequences (partial results in a workspace, the second launch that merges them) and fp8 codes."""
     H, D, N = 8, 128, 1024
@@ -114,17 +151,27 @@ def test_only_one_kind_of_sequence_and_bad_jobs(dev):
                                      md.kv_seq_lens[:0], D ** -0.5, out=got[:0].view(-1, H, D), as_job=True)
     _hidden(q, cache, md, w, b_v, D, got, kv_job=job)
     assert torch.equal(got, want)
+    # ... and its stores are the hidden rows alone (no key, no value)
+    hs = randn((3, H * D), 9).to(dev)
+    cache_a, cache_b = cache.clone(), cache.clone()
+    ops.hidden_to_cache(hs, cache_a, md.slot_mapping, md.hidden_cache_use_input, md.hidden_cache_store_tot)
+    _hidden(q, cache_a, md, w, b_v, D, want)
+    sj = ops.decode_step_cache_ops(None, hs, cache_b, None, md.slot_mapping, md.hidden_cache_use_input,
+                                   md.hidden_cache_store_tot, None, None, None, None, as_job=True)
+    _hidden(q, cache_b, md, w, b_v, D, got, store_job=sj)
+    assert torch.equal(cache_a, cache_b) and not torch.equal(cache_a, cache) and torch.equal(got, want)
     # bytes that no planning call wrote are refused, and so is a buffer that is too small
     junk = (ctypes.c_uint64 * 40)()
     assert lib.aps_attention_job_launch(ctypes.addressof(junk), None) == -1
     ws = torch.empty(lib.aps_absorbed_attention_workspace_bytes(3, 100, H, D), dtype=torch.uint8, device=dev)
     st = lib.aps_hybrid_decode_attention(
-        ctypes.addressof(junk), q.data_ptr(), q.stride(0), md.hidden_cache_use_input.data_ptr(), q.size(0),
+        None, ctypes.addressof(junk), q.data_ptr(), q.stride(0), md.hidden_cache_use_input.data_ptr(), q.size(0),
         cache.data_ptr(), cache.stride(2), cache.numel() // cache.stride(2), md.hidden_slots.data_ptr(),
         md.hidden_seq_start.data_ptr(), 3, int(md.max_hidden_seq_len), w[0].data_ptr(), w[1].data_ptr(),
         b_v.data_ptr(), w[0].stride(0), H, D, D ** -0.5, got.data_ptr(), got.stride(0), got.size(0), 0, ws.data_ptr(),
         ws.numel(), None)
     assert st == -1
+    assert lib.aps_cache_job_launch(ctypes.addressof(junk), None) == -1
     out = torch.empty(2, H, D, dtype=torch.float16, device=dev)
     st = lib.aps_paged_decode_attention_job(
         ctypes.addressof(junk), 64, out.data_ptr(), out.data_ptr(), cache[0].data_ptr(), cache[1].data_ptr(), None,
