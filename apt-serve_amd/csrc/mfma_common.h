@@ -97,7 +97,7 @@ __device__ __forceinline__ float load_16bit_as_f32(const void* p, int64_t i) {
 // More than 64 KiB of dynamic LDS has to be allowed per function and device: done once per (kernel, device)
 // instead of on every launch.  `slot` numbers the kernel instantiations of one source file that need it.
 inline hipError_t allow_dynamic_lds(const void* fn, int bytes, int slot) {
-  static std::atomic<uint64_t> done[24];
+  static std::atomic<uint64_t> done[40];
   int device = 0;
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return e;

@@ -787,8 +787,9 @@ __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArg
 // cross-workgroup sum at its end (~3.8 us: store acknowledgement, counter, loads of the parts).  Hence the choice by
 // a small cost model over (rows per workgroup in {128, 112, 96, 80, 64}, whole-chunk K parts) with at most one
 // workgroup per CU: time of the longest part at min(34 GB/s, 6.9 TB/s / workgroups) plus the sum if K is split.
-// 13B shapes: n=15360 (qkv) 240 workgroups of 64 rows, no split (was 120 x 2 parts); n=20480 (fc1) 256 workgroups
-// of 80 rows (was 160 of 128: 96 CUs idle); n=5120, k=5120 stays at 40 x 5 parts; n=5120, k=20480 64 x 4 parts.
+// 13B shapes at 9..16 rows: n=15360 (qkv) 240 workgroups of 64 rows, no split (was 120 x 2 parts); n=20480 (fc1)
+// 214 workgroups of 96 rows (was 160 of 128: 96 CUs idle); n=5120, k=5120 46 x 5 parts of 112 rows; n=5120,
+// k=20480 64 x 4 parts of 80 rows.  (3..8 rows with K up to 6144 go to weight_ksplit_kernel instead.)
 struct WsPlan { int rows, parts; int64_t k_per_part; };
 WsPlan weight_stream_plan(int64_t m, int64_t n, int64_t k, bool whole_tiles_only = false) {
   const int nht = m <= 16 ? 1 : (m <= 32 ? 2 : 3);
@@ -831,6 +832,156 @@ int launch_weight_stream(const GemmArgs& g, int parts, int64_t k_per_part, hipSt
   } while (0)
   if (nht == 1) APS_LAUNCH_WS(1); else if (nht == 2) APS_LAUNCH_WS(2); else APS_LAUNCH_WS(3);
 #undef APS_LAUNCH_WS
+  if (e != hipSuccess) return (int)e;
+  return launch_status();
+}
+
+// ---------------------------------------------------------------- 3 .. 8 rows, K up to 6144: K split inside the workgroup
+// Workgroup = 16 weight rows; its 8 wavefronts take an eighth of K each (P pairs of wave-wide loads = 64 P elements)
+// and add their partial products through LDS, in wavefront order.  Nothing crosses workgroups, so a launch has no
+// sum at its end, and the unit of work is small (16 rows x K: 160 KB at K = 5120), so n / 16 workgroups spread
+// over the CUs where n / 128 tiles x K parts left some idle.  The price: every workgroup needs the activations of
+// its whole K at once - the image is all m rows, staged once (m x K x 2 bytes of LDS, read from L2) - which is why
+// this is for few rows and one-digit thousands of K.  A wavefront requests everything it streams before anything
+// else happens (2 P loads of 1 KiB), stages its share of the image, and multiplies as the rows arrive.
+constexpr int kKsMaxRows = 8, kKsMaxPairs = 12;
+constexpr int ksplit_lds_bytes(int m, int pairs) { return m * pairs * 512 * 2 + kScWaves * kKsMaxRows * 16 * 4; }
+#ifndef APS_KSPLIT
+#define APS_KSPLIT 1
+#endif
+
+// ROWS = 16, or 8 (the second wave-wide load of every pair is left out and half of each MFMA multiplies zeros):
+// twice the workgroups of half the size, for products whose n / 16 workgroups are too few to balance over the CUs.
+template <bool BF16, int P, int ROWS>
+__global__ __launch_bounds__(kScThreads) void weight_ksplit_kernel(const GemmArgs g) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  constexpr int kRowPieces = 64 * P;   // 16-byte pieces of an image row: K / 8, K = 512 P
+  constexpr int kRowBytes = kRowPieces * 16;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int g4 = lane >> 4, c = lane & 15;
+  const int m = (int)g.m;
+  const int64_t n0 = (int64_t)blockIdx.x * ROWS;
+  // The image goes global -> LDS without passing through registers: one wave-wide copy fills 64 consecutive
+  // 16-byte slots of a row, and the swizzle (slot s of row r holds piece s ^ (r & 15) of its group of 16) is applied
+  // on the source side, every lane fetching the piece that belongs in its slot.  m x P copies, dealt over the
+  // wavefronts; they are requested before the weight rows, so that waiting for them leaves the rows in flight.
+  // (The copies are issued from assembly: the compiler, seeing a copy into LDS and a later LDS read, waits for
+  // every load in flight before the first read, weight rows included; it cannot know which bytes the copy wrote.)
+  const int64_t head_off = g.head_rows ? (n0 / g.head_rows) * g.x_head_stride_b : 0;
+  const uint64_t xa = (uint64_t)(g.a + head_off);
+  u32x4 rsrc;   // buffer descriptor over the m rows of x
+  rsrc[0] = __builtin_amdgcn_readfirstlane((uint32_t)xa);
+  rsrc[1] = __builtin_amdgcn_readfirstlane((uint32_t)(xa >> 32));
+  rsrc[2] = __builtin_amdgcn_readfirstlane((uint32_t)((m - 1) * g.lda_b + g.k * 2));
+  rsrc[3] = 0x00020000u;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+#pragma unroll
+  for (int j = 0; j < P; ++j) {   // (8 rows x P copies / 8 wavefronts = P copies per wavefront at most)
+    const int t = wave + j * kScWaves;
+    const int r = t / P, jg = t % P;
+    if (r < m) {
+      const int slot = 64 * jg + lane;
+      const int piece = (slot & ~15) | ((slot ^ r) & 15);
+      asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                   :
+                   : "s"(__builtin_amdgcn_readfirstlane(lds_base + (uint32_t)(r * kRowBytes + jg * 1024))),
+                     "v"((uint32_t)(r * g.lda_b) + (uint32_t)(piece * 16)), "s"(rsrc)
+                   : "memory");
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // this wavefront's weight rows: lane l = row l / 8 (and 8 + l / 8), 16-byte piece l % 8 of every 128 bytes
+  const char* rowp0 = g.w + (n0 + (lane >> 3)) * g.ldw_b + (lane & 7) * 16 + (int64_t)wave * (P * 128);
+  const char* rowp1 = rowp0 + 8 * g.ldw_b;
+  constexpr int kLoads = ROWS == 16 ? 2 * P : P;
+  u32x4 ring[2 * P];
+#pragma unroll
+  for (int u = 0; u < P; ++u) {
+    ring[2 * u] = __builtin_nontemporal_load((const u32x4*)(rowp0 + u * 128));
+    if constexpr (ROWS == 16) ring[2 * u + 1] = __builtin_nontemporal_load((const u32x4*)(rowp1 + u * 128));
+    else ring[2 * u + 1] = u32x4{0u, 0u, 0u, 0u};
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads) : "memory");   // the image copies of this wavefront have landed
+  APS_BARRIER();
+  __builtin_amdgcn_sched_barrier(0);   // (nothing that waits for a weight row moves in front of the barrier)
+
+  const int upper = c >> 3;
+  const int src_even = (8 * (c & 7) + g4 + 4 * upper) * 4;
+  const int src_odd = (8 * (c & 7) + g4 + 4 * (1 - upper)) * 4;
+  const char* qrow = lds + c * kRowBytes;
+  float4v acc = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int st = 0; st < 2 * P; ++st) {
+    const int u = st >> 1;
+    u32x4 bf;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const int lo = (int)ring[2 * u][d], hi = (int)ring[2 * u + 1][d];
+      const int merged = (st & 1) == 0 ? __builtin_amdgcn_update_dpp(lo, hi, 0x114 /* row_shr:4 */, 0xf, 0xa, false)
+                                       : __builtin_amdgcn_update_dpp(lo, hi, 0x104 /* row_shl:4 */, 0xf, 0x5, false);
+      bf[d] = (uint32_t)__builtin_amdgcn_ds_bpermute((st & 1) == 0 ? src_even : src_odd, merged);
+    }
+    const int ch = wave * (8 * P) + 4 * st + g4;   // piece of the image row: k = 8 ch .. 8 ch + 7
+    u32x4 af = u32x4{0u, 0u, 0u, 0u};
+    if (c < m) af = *(const u32x4*)(qrow + ((ch & ~15) | ((ch ^ c) & 15)) * 16);
+    acc = mfma16<BF16>(af, bf, acc);
+  }
+  // lane (g4, c) holds image rows 4 g4 + i (rows 8..15 do not exist) x weight row n0 + c
+  float* red = (float*)(lds + m * kRowBytes);
+  if (g4 < 2) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[(wave * kKsMaxRows + 4 * g4 + i) * 16 + c] = acc[i];
+  }
+  __syncthreads();
+  if (tid >= 16 * m || (tid & 15) >= ROWS) return;
+  const int row = tid >> 4, col = tid & 15;
+  float sum = red[row * 16 + col];
+#pragma unroll
+  for (int w = 1; w < kScWaves; ++w) sum += red[(w * kKsMaxRows + row) * 16 + col];
+  const int64_t n = n0 + col;
+  if (g.bias) sum += load_16bit_as_f32<BF16>(g.bias, n);
+  const int half = (g.out.n_split && n >= g.out.n_split) ? 1 : 0;
+  uint16_t* dst = out_row(g.out, row, half);
+  if (!dst) return;
+  const float v = act(g.out, sum);
+  dst[n - (half ? g.out.n_split : 0)] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+}
+
+inline bool ksplit_covers(int64_t m, int64_t n, int64_t k) {
+  const int64_t pairs = k / 512;
+  return m >= 3 && m <= kKsMaxRows && k % 512 == 0 && n % 16 == 0 &&
+         (pairs == 4 || pairs == 8 || pairs == 10 || pairs == 12);
+}
+
+#ifndef APS_KS_ROWS8_BELOW
+#define APS_KS_ROWS8_BELOW 512   // workgroups of 16 rows below which 8-row workgroups are launched instead
+#endif
+template <bool BF16>
+int launch_weight_ksplit(const GemmArgs& g, hipStream_t s) {
+  const int pairs = (int)(g.k / 512);
+  const int lds_bytes = ksplit_lds_bytes((int)g.m, pairs), lds_max = ksplit_lds_bytes(kKsMaxRows, pairs);
+  const bool rows8 = g.n / 16 < APS_KS_ROWS8_BELOW;
+  const dim3 grid((unsigned)(g.n / (rows8 ? 8 : 16)));
+  hipError_t e = hipSuccess;
+#define APS_LAUNCH_KS_R(P_, SLOT, R_)                                                                                \
+  do {                                                                                                               \
+    e = allow_dynamic_lds((const void*)weight_ksplit_kernel<BF16, P_, R_>, lds_max,                                  \
+                          24 + (BF16 ? 8 : 0) + 2 * SLOT + (R_ == 8 ? 1 : 0));                                       \
+    if (e == hipSuccess)                                                                                             \
+      APS_LAUNCH((weight_ksplit_kernel<BF16, P_, R_>), grid, dim3(kScThreads), lds_bytes, s, g);                     \
+  } while (0)
+#define APS_LAUNCH_KS(P_, SLOT) \
+  if (rows8) APS_LAUNCH_KS_R(P_, SLOT, 8); else APS_LAUNCH_KS_R(P_, SLOT, 16)
+  switch (pairs) {
+    case 4: APS_LAUNCH_KS(4, 0); break;
+    case 8: APS_LAUNCH_KS(8, 1); break;
+    case 10: APS_LAUNCH_KS(10, 2); break;
+    default: APS_LAUNCH_KS(12, 3); break;
+  }
+#undef APS_LAUNCH_KS
+#undef APS_LAUNCH_KS_R
   if (e != hipSuccess) return (int)e;
   return launch_status();
 }
@@ -953,6 +1104,7 @@ int aps_linear_nt_splits(int64_t m, int64_t n, int64_t k) {
   // per tile: split K until about two waves of workgroups exist, keeping at least 4 k-tiles per split.
   if (m <= 0 || n <= 0 || k <= 0 || n % BN != 0 || k % BK != 0) return 1;
   if (m <= kRsMaxRows) return 1;  // streamed in one launch
+  if (APS_KSPLIT && ksplit_covers(m, n, k)) return 1;   // K split inside the workgroups
   if (m <= kWsMaxRows) return weight_stream_plan(m, n, k).parts;
   const int64_t bm = 64 * tile_mi(m, n);
   const int64_t tiles = ((m + bm - 1) / bm) * (n / BN);
@@ -1018,6 +1170,8 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
   }
   if (!gs && m <= kRsMaxRows)
     return dtype == APS_BF16 ? launch_rowstream_m<true>(g, s) : launch_rowstream_m<false>(g, s);
+  if (APS_KSPLIT && !gs && ksplit_covers(m, n, k))
+    return dtype == APS_BF16 ? launch_weight_ksplit<true>(g, s) : launch_weight_ksplit<false>(g, s);
   if (!gs && m <= kWsMaxRows) {
     const WsPlan wp = weight_stream_plan(m, n, k);
     const int parts = wp.parts;
@@ -1125,6 +1279,7 @@ __attribute__((visibility("hidden"))) int64_t aps_internal_headwise_workspace_by
                                                                                    int head_rows) {
   if (m < 3 || m > kWsMaxRows || head_rows <= 0 || head_rows % kScTokens != 0 || n % kScTokens != 0 || k % BK != 0)
     return 0;
+  if (APS_KSPLIT && ksplit_covers(m, n, k)) return 16;
   const int parts = weight_stream_plan(m, n, k, true).parts;
   return parts > 1 ? (int64_t)parts * m * n * 4 : 16;   // (a nonzero size says "this shape is covered")
 }
@@ -1147,6 +1302,10 @@ __attribute__((visibility("hidden"))) int aps_internal_headwise_linear(const voi
   g.out.map = out_row_map; g.out.limit0 = out_rows;
   g.out.aligned16 = common_vec_bytes({addr(out), (uint64_t)out_stride * 2}) == 16;
   g.x_head_stride_b = x_head_stride * 2; g.head_rows = head_rows;
+  const bool vec16 = common_vec_bytes({addr(x), addr(weight), (uint64_t)x_stride * 2, (uint64_t)x_head_stride * 2,
+                                       (uint64_t)w_stride * 2}) == 16;
+  if (APS_KSPLIT && vec16 && ksplit_covers(m, n, k))   // (16 rows of a workgroup lie inside one head)
+    return dtype == APS_BF16 ? launch_weight_ksplit<true>(g, s) : launch_weight_ksplit<false>(g, s);
   // 3..48 rows and heads of whole 128-row tiles: the weight rows through the streaming core, K split over
   // enough workgroups to fill the chip, the parts added by the last workgroup of each tile
   const int64_t need = aps_internal_headwise_workspace_bytes(m, n, k, head_rows);

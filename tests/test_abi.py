@@ -95,6 +95,8 @@ def test_linear_workspace_planning_is_host_only_and_consistent():
                 assert 2 <= ways <= 4 and ways * rest <= 256 and ws == ways * rest * tile_bytes
             if m <= 2:
                 assert s == 1                                  # one launch of the dot-product kernel
+            elif m <= 8 and k in (2048, 4096, 5120, 6144):
+                assert s == 1 and ws == 0                      # K split inside the workgroups: nothing to add
             elif m <= 48:
                 # whole 512-element chunks of K; workgroups of 64..128 weight rows, at most one per compute unit
                 chunks = -(-k // 512)
@@ -145,7 +147,8 @@ int main(void) {
   if (strcmp(aps_status_string(APS_OK), "ok") != 0) return 2;
   /* argument errors are reported as negative statuses before anything is launched */
   if (aps_hidden_to_cache(NULL, NULL, NULL, NULL, NULL, -1, 0, 0, 0, 0, 0, 0, 0, NULL) >= 0) return 3;
-  if (aps_linear_nt_workspace_bytes(5, 5120, 5120) <= 0) return 4;      /* a decode step's projection splits K */
+  if (aps_linear_nt_workspace_bytes(12, 5120, 5120) <= 0) return 4;     /* a dozen rows: K split over workgroups */
+  if (aps_linear_nt_workspace_bytes(5, 5120, 5120) != 0) return 6;      /* a handful: split inside the workgroups */
   if (aps_decode_attention_workspace_bytes(4, 40, 128, 8192, 512) <= 0) return 5;   /* 16 partitions: flat path */
   printf("abi %d static scratch %d bytes\n", aps_abi_version(), (int)APS_STATIC_SCRATCH_BYTES);
   return 0;

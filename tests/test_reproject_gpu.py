@@ -62,6 +62,34 @@ def test_linear_nt_few_rows_weight_stream(dev, M, N, K, dtype):
     check(ops.linear_nt(x.to(dev), w.to(dev), None), OR._linear_fp32(x, w, None), dtype)
 
 
+@pytest.mark.parametrize("M", [3, 5, 8])
+@pytest.mark.parametrize("N,K", [(5120, 5120), (15360, 5120), (1024, 2048), (768, 4096), (512, 6144), (8192, 2048)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_linear_nt_k_split_inside_the_workgroups(dev, M, N, K, dtype):
+    """3..8 rows with K of 2048, 4096, 5120 or 6144: 16 (or, for few weight rows, 8) weight rows per workgroup,
+    the eight wavefronts an eighth of K each, all activation rows staged in LDS; no workspace is planned for these
+    shapes.  Against the fp32 oracle, with a row map, a strided x, the ReLU flag and without bias."""
+    assert ops._lib.load().aps_linear_nt_splits(M, N, K) == 1
+    assert ops._lib.load().aps_linear_nt_workspace_bytes(M, N, K) == 0
+    wide = randn((M, K + 24), M + K, dtype)
+    x = wide[:, 8:8 + K]
+    w = (randn((N, K), N + 1) * 0.02).to(dtype)
+    b = (randn((N,), 5) * 0.2).to(dtype)
+    ref = OR._linear_fp32(x, w, b)
+    xd, wd, bd = wide.to(dev)[:, 8:8 + K], w.to(dev), b.to(dev)
+    out = ops.linear_nt(xd, wd, bd)
+    check(out, ref, dtype)
+    assert torch.equal(ops.linear_nt(xd, wd, bd, relu=True), torch.relu(out))
+    check(ops.linear_nt(xd, wd, None), OR._linear_fp32(x, w, None), dtype)
+    perm = torch.from_numpy(np.random.default_rng(M).permutation(16)[:M].astype(np.int64)); perm[1] = -1
+    dest = torch.full((16, N), 7.0, dtype=dtype, device=dev)
+    ops.linear_nt(xd, wd, bd, out=dest, out_row_map=perm.to(dev))
+    keep = perm >= 0
+    assert torch.equal(dest[perm[keep].to(dev)], out[keep.to(dev)])
+    untouched = torch.ones(16, dtype=torch.bool); untouched[perm[keep]] = False
+    assert (dest[untouched.to(dev)] == 7).all()
+
+
 def test_few_rows_weight_stream_strides_row_map_and_workspace(dev):
     K, N, M = 2048, 2560, 21
     wide = randn((M, 2 * K + 8), 0)
@@ -106,8 +134,8 @@ def test_relu_epilogue_equals_relu_of_the_rounded_product(dev, M, dtype):
         assert (plain < 0).any() and torch.equal(act, torch.relu(plain))
 
 
-@pytest.mark.parametrize("M,N,K", [(3, 768, 1600), (5, 5120, 5120), (5, 5120, 20480), (17, 1536, 1088), (48, 5120, 5120),
-                                   (33, 7680, 5120), (7, 256, 2048)])
+@pytest.mark.parametrize("M,N,K", [(3, 768, 1600), (9, 5120, 5120), (5, 5120, 20480), (17, 1536, 1088), (48, 5120, 5120),
+                                   (33, 7680, 5120), (9, 256, 2048)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_k_split_summed_inside_the_launch_equals_the_two_launch_sum(dev, M, N, K, dtype):
     """The K split of a decode step's few rows with tile counters (the workgroup that stores a tile's last
