@@ -33,7 +33,13 @@ __device__ __forceinline__ float16v mfma32(const u32x4& a, const u32x4& b, const
                                                   0);
 }
 
-__device__ __forceinline__ uint16_t f32_to_f16_bits(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }
+// x is rounded to fp32 first, whatever produced it: the conversion of a product can otherwise be fused with the
+// multiply into one instruction that rounds once (v_fma_mixlo_f16) in some of the kernels a function is inlined
+// into and not in others, and kernels that share code are compared bit for bit.
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float x) {
+  asm volatile("" : "+v"(x));
+  return __builtin_bit_cast(uint16_t, (_Float16)x);
+}
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
   uint32_t u = __float_as_uint(x);
   if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);

@@ -12,6 +12,11 @@
 namespace aps {
 namespace {
 
+// No implicit fused multiply-adds in this header (the ones wanted are spelled fmaf): which products the compiler
+// fuses with a following add depends on the code around them, and these functions are inlined into more than one
+// kernel whose results are compared bit for bit.
+#pragma clang fp contract(off)
+
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -92,6 +97,10 @@ __device__ __forceinline__ float q_to_f32(uint16_t bits) {
 template <int QT>
 __device__ __forceinline__ uint16_t f32_to_q(float x) {
   if constexpr (QT == APS_F16) {
+    // x is rounded to fp32 first, whatever produced it: the conversion of a product can otherwise be fused with the
+    // multiply into one instruction that rounds once (v_fma_mixlo_f16), in some of the kernels this is inlined into
+    // and not in others
+    asm volatile("" : "+v"(x));
     return __builtin_bit_cast(uint16_t, (_Float16)x);
   } else {  // bf16, round to nearest even
     uint32_t u = __float_as_uint(x);
@@ -271,7 +280,7 @@ __device__ __forceinline__ void decode_wave(const AttnArgs& a, int seq, int head
       p[g] = __builtin_amdgcn_exp2f(s[g] - m_use);
       psum += p[g];
     }
-    l = l * alpha + psum;
+    l = fmaf(l, alpha, psum);   // (every multiply-add is spelled out: the same bits whichever kernel the code is inlined into)
 #pragma unroll
     for (int i = 0; i < EPL; ++i) acc[i] *= alpha;
 #pragma unroll
@@ -309,9 +318,9 @@ __device__ __forceinline__ void decode_wave(const AttnArgs& a, int seq, int head
     const float m_n = fmaxf(m, m_o);
     const float m_u = (m_n == -INFINITY) ? 0.f : m_n;
     const float wa = __builtin_amdgcn_exp2f(m - m_u), wb = __builtin_amdgcn_exp2f(m_o - m_u);
-    l = l * wa + l_o * wb;
+    l = fmaf(l_o, wb, l * wa);
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) acc[i] = acc[i] * wa + __shfl_xor(acc[i], off) * wb;
+    for (int i = 0; i < EPL; ++i) acc[i] = fmaf(__shfl_xor(acc[i], off), wb, acc[i] * wa);
     m = m_n;
   }
   res.m = m;
@@ -489,6 +498,8 @@ struct PagedJob {
   DecodePlan plan;
   AttnArgs a;
 };
+
+#pragma clang fp contract(fast)   // (the compiler's default for device code, for what follows the include)
 
 }  // namespace
 }  // namespace aps

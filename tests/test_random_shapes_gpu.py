@@ -280,3 +280,39 @@ def test_decode_step_cache_ops_random_batches(dev, seed):
         assert bits_equal(g, ref), what
         if with_holder:
             assert bits_equal(holder, holder_ref), what
+
+
+@pytest.mark.parametrize("seed", [101])
+def test_one_call_decode_attention_random_batches(dev, seed):
+    """Mixed decode batches of random size, mix and lengths: the step's stores, the paged attention of the K/V-cached
+    sequences and the attention on hidden rows as ONE call (jobs riding in its launches where they fit, launched by
+    themselves where they do not) against the three direct calls: caches and output bit for bit."""
+    import test_hybrid_attention_gpu as TH
+    rng = np.random.default_rng(seed)
+    for case in range(16):
+        H, D = [(4, 64), (8, 128), (40, 128), (2, 256)][int(rng.integers(0, 4))]
+        B = int(rng.integers(2, 24))
+        frac = float(rng.choice([0.2, 0.5, 0.8]))
+        max_len = int(rng.choice([20, 150, 600, 1500]))
+        dtype = DT16[int(rng.integers(0, 2))]
+        what = f"case {case}: H={H} D={D} B={B} frac={frac} max_len={max_len} {dtype}"
+        b, md, cache, w, b_v, q = TH._batch(dev, H, D, B, frac, max_len, 2048, dtype, int(rng.integers(0, 1000)))
+        n_h = md.num_hidden_cache_tokens
+        if n_h == 0 or n_h == len(b.seq_lens):
+            continue
+        hs, k, v = (randn((len(b.seq_lens), H * D), 40 + case + i, dtype).to(dev) for i in range(3))
+
+        def stores(c, **kw):
+            return ops.decode_step_cache_ops(None, hs, c, None, md.slot_mapping, md.hidden_cache_use_input,
+                                             md.hidden_cache_store_tot, k, v, md.kv_cache_use_input,
+                                             md.new_token_slot, **kw)
+
+        cache_a, want = cache.clone(), torch.full_like(q, 7.0)
+        stores(cache_a)
+        TH._paged(q, cache_a, md, H, D, want)
+        TH._hidden(q, cache_a, md, w, b_v, D, want)
+        cache_b, got = cache.clone(), torch.full_like(q, 7.0)
+        TH._hidden(q, cache_b, md, w, b_v, D, got, kv_job=TH._paged(q, cache_b, md, H, D, got, as_job=True),
+                   store_job=stores(cache_b, as_job=True))
+        assert torch.equal(cache_b, cache_a), what + ": caches differ"
+        assert torch.equal(got, want), what + ": outputs differ"
