@@ -282,7 +282,7 @@ def test_decode_step_cache_ops_random_batches(dev, seed):
             assert bits_equal(holder, holder_ref), what
 
 
-@pytest.mark.parametrize("seed", [101])
+@pytest.mark.parametrize("seed", [101, 102, 103, 104])
 def test_one_call_decode_attention_random_batches(dev, seed):
     """Mixed decode batches of random size, mix and lengths: the step's stores, the paged attention of the K/V-cached
     sequences and the attention on hidden rows as ONE call (jobs riding in its launches where they fit, launched by
