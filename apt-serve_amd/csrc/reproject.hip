@@ -842,9 +842,9 @@ int launch_weight_stream(const GemmArgs& g, int parts, int64_t k_per_part, hipSt
 // sum at its end, and the unit of work is small (16 rows x K: 160 KB at K = 5120), so n / 16 workgroups spread
 // over the CUs where n / 128 tiles x K parts left some idle.  The price: every workgroup needs the activations of
 // its whole K at once - the image is all m rows, staged once (m x K x 2 bytes of LDS, read from L2) - which is why
-// this is for few rows and one-digit thousands of K.  A wavefront requests everything it streams before anything
-// else happens (2 P loads of 1 KiB), stages its share of the image, and multiplies as the rows arrive.
-constexpr int kKsMaxRows = 8, kKsMaxPairs = 12;
+// this is for few rows and one-digit thousands of K.  A wavefront requests its share of the image copies, then
+// everything it streams (2 P loads of 1 KiB), waits for the copies alone, and multiplies as the rows arrive.
+constexpr int kKsMaxRows = 8;
 constexpr int ksplit_lds_bytes(int m, int pairs) { return m * pairs * 512 * 2 + kScWaves * kKsMaxRows * 16 * 4; }
 #ifndef APS_KSPLIT
 #define APS_KSPLIT 1
