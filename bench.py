@@ -39,7 +39,7 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip attention / re-projection figures")
     ap.add_argument("--extras", default="literal,attention,prefill,metadata,write,ceilings,reproject,layer,step_loop,cost,cpu",
-                    help="comma-separated subset of the extra figures to run")
+                    help="comma-separated subset of the extra figures to run (step_replay: not in the default list)")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="first run the plain copy kernel on 1 GiB three times (known traffic for counter scaling)")
     return ap.parse_args()
@@ -301,6 +301,9 @@ def main():
             a_, b_ = extras["opt13b_step_loop"].pop("schedule"), extras["opt13b_step_loop_absorbed"].pop("schedule")
             c_ = extras["opt13b_step_loop_reference_sequence"].pop("schedule")
             extras["opt13b_step_loop_same_schedule"] = a_ == b_ == c_ == d_
+        if "step_replay" in want:   # (not in the default list: the kernel split of one decode step, for a profiler)
+            extras["opt13b_step_replay"] = step_replay_figures(torch, dev, args.seed)
+            torch.cuda.empty_cache()
         if "cost" in want:
             extras["cost_coef"] = cost_coef_figures(torch, dev)
         if not args.no_cpu and "cpu" in want:
@@ -447,6 +450,40 @@ def mfma_ceiling_figures(torch, dev):
             out[f"f16_{name}_{data}"] = {"ms": ms, "tflops": flops / ms / 1e9,
                                           "frac_of_mfma_peak": flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS}
     return out
+
+
+def step_replay_figures(torch, dev, seed, seq_lens=(310, 120, 200, 260, 130), use_hidden=(1, 0, 1, 0, 1), reps=26):
+    """One OPT-13B decode step of a fixed small batch (absorbed flow), recorded into a HIP graph once and replayed:
+    under ``rocprofv3 --kernel-trace`` the kernels of the replays run back to back, so their durations add up to the
+    step and give its split by kernel."""
+    from aptserve_hip import backend, graph_step, opt_model
+    cfg = opt_model.OPTConfig.opt_13b()
+    model = opt_model.HybridOPTModel(cfg, opt_model.random_weights(cfg, seed, dev), absorbed=True)
+    BS = 16
+    kv, shared = backend.allocate_caches(cfg.num_hidden_layers, 2048, BS, cfg.num_attention_heads,
+                                         cfg.hidden_size // cfg.num_attention_heads, torch.float16, dev)
+    for c in kv:
+        c.normal_(0, 0.3)
+    tables, shared_tables, nxt = [], [], 0
+    for n, h in zip([-(-l // BS) for l in seq_lens], use_hidden):
+        tables.append(list(range(nxt, nxt + n))); nxt += n
+        shared_tables.append(list(range(nxt, nxt + n)) if h else []); nxt += n if h else 0
+    runner = graph_step.DecodeGraphRunner(model, kv, shared, BS, dev)
+    ids = torch.randint(0, cfg.vocab_size, (len(seq_lens),), device=dev)
+    rec = runner.prepare(list(seq_lens), [bool(h) for h in use_hidden], tables, shared_tables, ids)
+    torch.cuda.synchronize()
+    for _ in range(5):
+        runner.run(rec)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        runner.run(rec)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / reps * 1e3
+    return {"workload": f"OPT-13B 40 layers fp16 random-init, decode batch of {len(seq_lens)} sequences "
+                        f"({sum(bool(h) for h in use_hidden)} hidden-cached with "
+                        f"{sum(l for l, h in zip(seq_lens, use_hidden) if h)} cached rows), one HIP graph replayed",
+            "replays": reps, "ms_per_step": ms}
 
 
 def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile_steps=12, absorbed=False,
