@@ -480,10 +480,22 @@ def step_replay_figures(torch, dev, seed, seq_lens=(310, 120, 200, 260, 130), us
         runner.run(rec)
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / reps * 1e3
+    # the same step eagerly with GPU event timers around the phases of every layer (their synchronisations serialise
+    # the step: a split, not a step time)
+    per = {}
+    for _ in range(3):
+        with backend.PhaseTimes() as pt:
+            model(rec.ids, rec.md.input_positions, kv, shared, rec.md)
+        for k_, v_ in pt.totals().items():
+            per[k_] = per.get(k_, 0.0) + v_ / 3
+    L = cfg.num_hidden_layers
     return {"workload": f"OPT-13B 40 layers fp16 random-init, decode batch of {len(seq_lens)} sequences "
                         f"({sum(bool(h) for h in use_hidden)} hidden-cached with "
                         f"{sum(l for l, h in zip(seq_lens, use_hidden) if h)} cached rows), one HIP graph replayed",
-            "replays": reps, "ms_per_step": ms}
+            "replays": reps, "ms_per_step": ms,
+            "eager_phase_us_per_layer": {k_: v_ * 1e3 / L for k_, v_ in per.items()},
+            "note": "attention_on_hidden_rows = the one call for both kinds of sequence (stores, K/V attention, "
+                    "attention on hidden rows with its value projection); projections = qkv, out, fc1, fc2"}
 
 
 def step_loop_figures(torch, dev, seed, warm_steps=240, timed_steps=320, profile_steps=12, absorbed=False,
