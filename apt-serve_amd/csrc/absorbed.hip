@@ -365,7 +365,7 @@ __device__ __forceinline__ void query_image_body(const QImageArgs& g, const Stor
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
               const float v = acc[j][i] * g.alpha;
-              hh[j] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+              hh[j] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits_rounded(v);
             }
             u32x4 o;
 #pragma unroll
@@ -923,7 +923,7 @@ __device__ __forceinline__ void hidden_wsum_chunk_body(const WsumArgs& g) {
     for (int i = 0; i < 4; ++i) {
       const float e = ok[i] ? __builtin_amdgcn_exp2f(sv[j][i] - cmax) : 0.f;
       sum += e;
-      o[i] = BF16 ? f32_to_bf16_bits(e) : f32_to_f16_bits(e);
+      o[i] = BF16 ? f32_to_bf16_bits(e) : f32_to_f16_bits_rounded(e);
     }
 #pragma unroll
     for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
@@ -981,7 +981,7 @@ __device__ __forceinline__ void hidden_wsum_chunk_body(const WsumArgs& g) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float v = acc[ht][j][i] * inv;
-          h[j] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v);
+          h[j] = BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits_rounded(v);
         }
         u32x4 o;
 #pragma unroll

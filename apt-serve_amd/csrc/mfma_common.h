@@ -33,10 +33,13 @@ __device__ __forceinline__ float16v mfma32(const u32x4& a, const u32x4& b, const
                                                   0);
 }
 
-// x is rounded to fp32 first, whatever produced it: the conversion of a product can otherwise be fused with the
-// multiply into one instruction that rounds once (v_fma_mixlo_f16) in some of the kernels a function is inlined
-// into and not in others, and kernels that share code are compared bit for bit.
-__device__ __forceinline__ uint16_t f32_to_f16_bits(float x) {
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }
+// The same for code that is inlined into more than one kernel whose results are compared bit for bit: x is rounded
+// to fp32 first, whatever produced it.  The conversion of a product can otherwise be fused with the multiply into
+// one instruction that rounds once (v_fma_mixlo_f16) in one of those kernels and not in another.  (Not the default:
+// the empty asm is a scheduling obstacle, and the streaming weighted sum, at its register limit, runs 60 % longer
+// with it.)
+__device__ __forceinline__ uint16_t f32_to_f16_bits_rounded(float x) {
   asm volatile("" : "+v"(x));
   return __builtin_bit_cast(uint16_t, (_Float16)x);
 }
