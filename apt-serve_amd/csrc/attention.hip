@@ -210,6 +210,8 @@ static int plan_decode_job(PagedJob& job, void* out, const void* q, const void* 
   if (block_size % kTile != 0) return APS_ERR_UNSUPPORTED;
   if (q_dtype != APS_F16 && q_dtype != APS_BF16) return APS_ERR_UNSUPPORTED;
   if (kv_dtype != q_dtype && kv_dtype != APS_FP8_E4M3) return APS_ERR_UNSUPPORTED;
+  if (head_size != 64 && head_size != 128 && head_size != 256 && !(head_size == 32 && kv_dtype != APS_FP8_E4M3))
+    return APS_ERR_UNSUPPORTED;   // (the head sizes the kernels are built for: known when a job is planned)
   if (q_stride < (int64_t)num_heads * head_size || out_stride < (int64_t)num_heads * head_size)
     return APS_ERR_INVALID_ARG;
   const int kv_b = kv_dtype == APS_FP8_E4M3 ? 1 : 2;

@@ -71,6 +71,50 @@ def test_argument_errors_return_without_launching():
     assert pl.aps_mfma_probe(1, 0, 16, 16, 0, 1, None) == 0
 
 
+def test_jobs_are_planned_on_the_host_and_checked_before_a_launch():
+    """Planning a job is arithmetic on the arguments (no GPU call, so made-up addresses will do here): the checks of
+    the direct call, a buffer of the promised size, and launches that refuse what no planning call wrote.  A job
+    over an empty batch launches nothing and is not an error, also through the hybrid call."""
+    import ctypes
+    lib = _lib.load()
+    A = 1 << 20                                           # an aligned address that is never dereferenced
+    H, D, BS, B, W = 40, 128, 16, 4, 8
+    job = (ctypes.c_uint64 * 40)()
+    ja = ctypes.addressof(job)
+    assert ctypes.sizeof(job) == 320                      # APS_ATTENTION_JOB_BYTES = APS_CACHE_JOB_BYTES
+
+    def plan_attention(addr, nbytes, batch, q_dtype=0, head_size=D):
+        return lib.aps_paged_decode_attention_job(addr, nbytes, A, A, A, A, None, None, A, None, A, batch, H, head_size,
+                                                  BS, W, W, 0, H * head_size, H * head_size, BS * H * head_size, 64, 0,
+                                                  0, W * BS, 0, 0.1, q_dtype, q_dtype, 1.0, 1.0, None, 0)
+
+    assert plan_attention(ja, 320, B) == 0
+    assert plan_attention(ja, 64, B) == -1                # buffer too small
+    assert plan_attention(ja + 4, 320, B) == -1           # not 8-byte aligned
+    assert plan_attention(None, 320, B) == -1
+    assert plan_attention(ja, 320, -1) == -1              # the direct call's checks
+    assert plan_attention(ja, 320, B, q_dtype=7) == -2    # unsupported dtype
+    assert plan_attention(ja, 320, B, head_size=48) == -2
+    junk = (ctypes.c_uint64 * 40)()
+    assert lib.aps_attention_job_launch(ctypes.addressof(junk), None) == -1
+    assert lib.aps_cache_job_launch(ctypes.addressof(junk), None) == -1
+    assert lib.aps_attention_job_launch(None, None) == -1 and lib.aps_cache_job_launch(None, None) == -1
+    # empty jobs: planned, launched (nothing to do), and accepted by the hybrid call without sequences
+    assert plan_attention(ja, 320, 0) == 0 and lib.aps_attention_job_launch(ja, None) == 0
+    store = (ctypes.c_uint64 * 40)()
+    sa = ctypes.addressof(store)
+    plan_store = lambda n_store, n_kv, elem=2: lib.aps_decode_step_cache_ops_job(
+        sa, 320, None, A, A, None, 0, A, A, A, n_store, B, H * D, 0, H * D, H * D, 64 * BS, A, A, A, A, A, A, n_kv,
+        H * D, H * D, BS, BS * H * D, 64, elem)
+    assert plan_store(0, 0) == 0 and lib.aps_cache_job_launch(sa, None) == 0
+    assert plan_store(2, -1) == -1 and plan_store(2, 2, elem=3) == -1
+    assert plan_store(0, 0) == 0
+    assert lib.aps_hybrid_decode_attention(sa, ja, None, 0, None, 0, None, 0, 0, None, None, 0, 0, None, None, None, 0,
+                                           H, D, 0.1, None, 0, 0, 0, None, 0, None) == 0
+    assert lib.aps_hybrid_decode_attention(ctypes.addressof(junk), None, None, 0, None, 0, None, 0, 0, None, None, 0, 0,
+                                           None, None, None, 0, H, D, 0.1, None, 0, 0, 0, None, 0, None) == -1
+
+
 def test_linear_workspace_planning_is_host_only_and_consistent():
     """aps_linear_nt_splits / _workspace_bytes are pure host functions (no launch): the workspace is the fp32
     partial tiles of every split, few-row products are split into whole 512-element chunks of K, and no plan asks
