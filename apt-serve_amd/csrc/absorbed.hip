@@ -550,6 +550,7 @@ __global__ __launch_bounds__(kScThreads) void head_proj_kernel(const HeadProjArg
 #define APS_WS_OCC 2
 #endif
 constexpr int kWsWaves = APS_WS_WAVES, kWsThreads = kWsWaves * 64, kWsRing = APS_WS_RING, kWsChunk = 32 * kWsRing;
+constexpr int kHeadwiseMaxSeqs = 256;             // sequences up to which the value projection may take the weight streams
 constexpr int kFusedHeadSize = 128;               // head size of the paged attention that can ride in the chunk launch
 constexpr int kWsMaxPart = 4096;                  // tokens of a partition (their slots are staged in LDS)
 constexpr int kWsIds = (kWsMaxPart + kWsChunk - 1) / kWsChunk * kWsChunk + 32 * (kWsRing - 1);
@@ -1130,7 +1131,8 @@ Plan make_plan(int64_t n_seqs, int64_t max_len, int heads, int64_t hidden) {
   p.off_ml = o;
   if (p.kparts > 1) o += align_up((int64_t)p.kparts * n_seqs * heads * 2 * 4, 256);
   p.off_vp = o;   // fp32 partial products of the value projection's K split (few sequences)
-  if (n_seqs <= 16) o += align_up(aps_internal_headwise_workspace_bytes(n_seqs, hidden, hidden, (int)(hidden / heads)), 256);
+  if (n_seqs <= kHeadwiseMaxSeqs)
+    o += align_up(aps_internal_headwise_workspace_bytes(n_seqs, hidden, hidden, (int)(hidden / heads)), 256);
   p.total = o;
   return p;
 }
@@ -1376,7 +1378,10 @@ static int hybrid_attention_impl(const StoreJob* store_job, const PagedJob* kv_j
     }
   }
   // 5. out[seq_rows[s]][h*D + d] = <W_v[h*D + d], ctx[s][h]> + b_v
-  if (n_seqs <= 16)  // few sequences: the weight-streaming kernels read W_v once
+  // few sequences: the weight-streaming kernels read W_v once; up to kHeadwiseMaxSeqs where those kernels cover the
+  // shape (heads of whole 128-row tiles): K parts fill the chip where (head, 48 sequences) workgroups do not
+  if (n_seqs <= 16 || (n_seqs <= kHeadwiseMaxSeqs &&
+                       aps_internal_headwise_workspace_bytes(n_seqs, hidden, hidden, head_size) > 0))
     return aps_internal_headwise_linear(ctx, w_v, b_v, out, n_seqs, hidden, hidden, (int64_t)num_heads * hidden,
                                         hidden, head_size, w_stride, out_stride, seq_rows, out_rows, dtype,
                                         ws + p.off_vp, p.total - p.off_vp, (int32_t*)(ws + p.off_vp_counters), s);

@@ -688,6 +688,7 @@ int launch_rowstream_m(const GemmArgs& g, hipStream_t s) {
 // do not fill the chip: K is split over blockIdx.y into parts of whole 512-element chunks, and the fp32
 // partial tiles [part][m][n] are added by splitk_reduce_kernel.
 constexpr int kWsMaxRows = 48;
+constexpr int kHeadwiseMaxRows = 256;   // head-wise x (the value projection of the attention on hidden rows)
 
 template <bool BF16, int NHT>
 __global__ __launch_bounds__(kScThreads) void weight_stream_kernel(const GemmArgs g, int64_t k_per_part) {
@@ -1277,7 +1278,8 @@ static int launch_gemm(const void* x, const void* weight, const void* bias, cons
 
 __attribute__((visibility("hidden"))) int64_t aps_internal_headwise_workspace_bytes(int64_t m, int64_t n, int64_t k,
                                                                                    int head_rows) {
-  if (m < 3 || m > kWsMaxRows || head_rows <= 0 || head_rows % kScTokens != 0 || n % kScTokens != 0 || k % BK != 0)
+  // (more rows than one image holds go over the grid's z: every 48 rows stream the weights again, from L2)
+  if (m < 3 || m > kHeadwiseMaxRows || head_rows <= 0 || head_rows % kScTokens != 0 || n % kScTokens != 0 || k % BK != 0)
     return 0;
   if (APS_KSPLIT && ksplit_covers(m, n, k)) return 16;
   const int parts = weight_stream_plan(m, n, k, true).parts;
