@@ -161,7 +161,9 @@ int aps_decode_step_cache_ops(
  * launched later: the job (APS_CACHE_JOB_BYTES of host memory that the caller
  * owns, 8-byte aligned, opaque) records the arguments and the shape of the
  * launch.  Same arguments, checks and status codes as
- * aps_decode_step_cache_ops (same reference call sites); nothing is enqueued.
+ * aps_decode_step_cache_ops, whose reference call sites it shares
+ * (model_executor/models/aptserve_opt.py:108-121,
+ * attention/backends/aptserve_flash_attn.py:338-345); nothing is enqueued.
  * aps_cache_job_launch launches a job by itself, with the result of the direct
  * call; aps_hybrid_decode_attention takes one as the cache writes that precede
  * a decode step's attention.  The device memory the arguments point to must be
